@@ -1,0 +1,101 @@
+"""A stand-in for the HIP kernel library, in plain torch on the CPU, used only
+by tests that check the engine's own logic (batch packing, block tables, cache
+manager, run order, scheduler) without a GPU.  The product never loads this:
+its kernel library is tiny_llm_infer_amd.kernels.ops.HipOps and nothing else.
+"""
+from __future__ import annotations
+
+import torch
+
+
+class CpuOps:
+    name = "cpu-test-double"
+
+    def check_attention_sizes(self, heads, kv_heads, head_dim):
+        pass
+
+    def check_page_size(self, page_size):
+        pass
+
+    def embed(self, table, token_ids, num_rows):
+        return table[token_ids.long()].to(torch.float32)
+
+    def add_rmsnorm(self, resid, delta, weight, eps, out_dtype, rows=None, num_rows=None):
+        if rows is None:
+            if delta is not None:
+                resid += delta.to(torch.float32)
+            x = resid
+        else:
+            x = resid[rows.long()]
+            if delta is not None:
+                x = x + delta[rows.long()].to(torch.float32)
+        scale = torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + eps)
+        return (weight * x * scale).to(out_dtype)
+
+    def linear(self, x, w, out_dtype=None):
+        y = x.to(torch.float32) @ w.to(torch.float32).t()
+        return y.to(out_dtype or x.dtype)
+
+    def swiglu(self, gu):
+        inter = gu.shape[1] // 2
+        g, u = gu[:, :inter].to(torch.float32), gu[:, inter:].to(torch.float32)
+        return (g / (1 + torch.exp(-g)) * u).to(gu.dtype)
+
+    def qkv_to_cache(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary):
+        T = step.num_rows
+        qd, kd = heads * head_dim, kv_heads * head_dim
+        x = qkv.to(torch.float32)
+        q = x[:, :qd].reshape(T, heads, head_dim)
+        k = x[:, qd:qd + kd].reshape(T, kv_heads, head_dim)
+        v = x[:, qd + kd:].reshape(T, kv_heads, head_dim)
+
+        def norm(t, wn):
+            if wn is None:
+                return t
+            w, eps = wn
+            return w * t * torch.rsqrt((t * t).mean(dim=-1, keepdim=True) + eps)
+
+        q, k = norm(q, q_norm), norm(k, k_norm)
+        pos = step.positions.long()
+        if rotary is not None:
+            cos, sin, rd = rotary
+            half = rd // 2
+            c, s = cos[pos][:, None, :], sin[pos][:, None, :]
+
+            def rot(t):
+                a, b, rest = t[..., :half], t[..., half:rd], t[..., rd:]
+                return torch.cat([a * c - b * s, a * s + b * c, rest], dim=-1)
+            q, k = rot(q), rot(k)
+        if cache is not None and cache.writes:
+            page = cache.group.page_size
+            tables = cache.group.tables
+            seq = step.seq_of_row.long()
+            pages = tables[seq, pos // page].long()
+            assert (pages >= 0).all(), "a row writes to a page that is not held"
+            slots = pos % page
+            cache.k[pages, :, slots] = k.to(cache.k.dtype)
+            cache.v[pages, :, slots] = v.to(cache.v.dtype)
+        return q.reshape(T, qd).to(qkv.dtype)
+
+    def paged_attention(self, q, step, cache, heads, kv_heads, head_dim, scale, window):
+        T = step.num_rows
+        page = cache.group.page_size
+        tables = cache.group.tables
+        qf = q.to(torch.float32).reshape(T, heads, head_dim)
+        out = torch.zeros(T, heads, head_dim, dtype=torch.float32)
+        mul = heads // kv_heads
+        pos_l = step.positions.tolist()
+        seq_l = step.seq_of_row.tolist()
+        for r in range(T):
+            p = pos_l[r]
+            lo = 0 if window is None else max(0, p - window + 1)
+            idx = torch.arange(lo, p + 1)
+            pages = tables[seq_l[r], idx // page].long()
+            assert (pages >= 0).all(), "a row reads a page that is not held"
+            kk = cache.k[pages, :, idx % page].to(torch.float32)     # [n, kv, d]
+            vv = cache.v[pages, :, idx % page].to(torch.float32)
+            for h in range(heads):
+                s = (kk[:, h // mul] @ qf[r, h]) * scale
+                w = torch.softmax(s, dim=0)
+                out[r, h] = w @ vv[:, h // mul]
+        return out.reshape(T, heads * head_dim).to(q.dtype)

@@ -1,0 +1,262 @@
+"""The step function.
+
+``ModelRunner.step(entries)`` takes a batch of (request, its next tokens,
+places whose logits are wanted): portions of prompts beside single decoded
+tokens, cut anywhere.  It runs only those tokens, as one batch, against the
+cache that earlier steps left, and returns float32 logits at the wanted places.
+The reference's counterpart is Qwen3Model::forward_paged_batch
+(model/src/qwen3_paged_batch.cpp:44-366) with the batch assembly of
+LLMEngine::step (engine/src/llm_engine.cpp:164-183); there every row carries a
+copy of its request's block table, here tables are per request and rows carry
+the index of their request.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheFull, CacheManager
+from ..parts.base import BuildEnv, GroupView, LayerCache, StepView
+from .model import Model
+
+
+@dataclass
+class StepEntry:
+    key: Hashable                 # the request
+    tokens: Sequence[int]         # its next tokens
+    want: Sequence[int] = ()      # places among ``tokens`` whose logits are wanted
+
+
+class StepError(ValueError):
+    pass
+
+
+def _pow2_at_least(n: int, floor: int = 4) -> int:
+    w = floor
+    while w < n:
+        w *= 2
+    return w
+
+
+def _pad4(n: int) -> int:
+    return (n + 3) & ~3
+
+
+class StepInputs:
+    """One host staging buffer and one device buffer that hold every integer
+    input of a step; a step costs one host-to-device copy.  The layout depends
+    only on (rows, sequences, wanted, table width)."""
+
+    def __init__(self, device, max_rows: int, max_seqs: int, num_groups: int, max_width: int):
+        self.device = torch.device(device)
+        cap = (3 * _pad4(max_rows) + _pad4(max_rows) + _pad4(max_seqs + 1) + 3 * _pad4(max_seqs)
+               + num_groups * max_seqs * max_width + 64)
+        pin = self.device.type == "cuda"
+        self.host = [torch.zeros(cap, dtype=torch.int32, pin_memory=pin) for _ in range(2)]
+        self.host_np = [h.numpy() for h in self.host]
+        self.events = [None, None]
+        self.dev = torch.zeros(cap, dtype=torch.int32, device=self.device)
+        self.turn = 0
+        self.num_groups = num_groups
+
+    def layout(self, rows: int, seqs: int, wanted: int, width: int) -> Dict[str, slice]:
+        off = 0
+        out = {}
+        for name, n in (("token_ids", rows), ("positions", rows), ("seq_of_row", rows),
+                        ("row_start", seqs + 1), ("seq_start", seqs), ("seq_len", seqs),
+                        ("slots", seqs), ("sample_rows", wanted)):
+            out[name] = slice(off, off + n)
+            off += _pad4(max(n, 1))
+        for g in range(self.num_groups):
+            out[f"tables{g}"] = slice(off, off + seqs * width)
+            off += _pad4(seqs * width)
+        out["_end"] = slice(0, off)
+        return out
+
+    def begin(self):
+        self.turn ^= 1
+        ev = self.events[self.turn]
+        if ev is not None:
+            ev.synchronize()
+        return self.host_np[self.turn]
+
+    def upload(self, n: int) -> None:
+        if self.device.type == "cuda":
+            self.dev[:n].copy_(self.host[self.turn][:n], non_blocking=True)
+            ev = self.events[self.turn] or torch.cuda.Event()
+            ev.record()
+            self.events[self.turn] = ev
+        else:
+            self.dev[:n].copy_(self.host[self.turn][:n])
+
+
+class ModelRunner:
+    def __init__(self, model: Model, env: BuildEnv, page_size: int, num_pages: int,
+                 max_requests: int, max_batch_tokens: int):
+        self.model = model
+        self.env = env
+        self.page_size = page_size
+        self.max_batch_tokens = max_batch_tokens
+        self.max_requests = max_requests
+        self.max_model_len = min(env.max_model_len, model.spec.max_positions)
+        env.ops.check_page_size(page_size)
+        self.cache = CacheManager(model.cache_needs(), page_size, num_pages, max_requests)
+        self.group_tensors = []
+        for g in self.cache.groups:
+            shape = (len(g.cache_layers), num_pages, g.need.num_kv_heads, page_size, g.need.head_dim)
+            k = torch.zeros(shape, dtype=env.dtype, device=env.device)
+            v = torch.zeros(shape, dtype=env.dtype, device=env.device)
+            self.group_tensors.append((k, v))
+        self.states: List[Optional[torch.Tensor]] = []
+        for need in model.state_needs():
+            self.states.append(None if need is None else torch.zeros(
+                (max_requests,) + tuple(need.shape), dtype=need.dtype, device=env.device))
+        max_width = _pow2_at_least((self.max_model_len + page_size - 1) // page_size)
+        self.inputs = StepInputs(env.device, max_batch_tokens, max_requests,
+                                 len(self.cache.groups), max_width)
+        self.steps_run = 0
+
+    # ---- requests ---------------------------------------------------------
+    def admit(self, key: Hashable):
+        return self.cache.admit(key)
+
+    def release(self, key: Hashable) -> None:
+        self.cache.release(key)
+
+    def cache_bytes(self) -> int:
+        return sum(k.numel() * k.element_size() * 2 for k, _ in self.group_tensors)
+
+    # ---- the step -----------------------------------------------------------
+    def _check(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        if len(entries) > self.max_requests:
+            raise StepError(f"{len(entries)} requests in one step, at most {self.max_requests}")
+        seen = set()
+        rows = 0
+        vocab = self.model.spec.vocab_size
+        for e in entries:
+            if e.key in seen:
+                raise StepError(f"request {e.key!r} appears twice in one step")
+            seen.add(e.key)
+            if e.key not in self.cache:
+                raise StepError(f"request {e.key!r} has not been admitted")
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"request {e.key!r} brings no tokens")
+            rows += n
+            total = self.cache.get(e.key).num_tokens + n
+            if total > self.max_model_len:
+                raise StepError(f"request {e.key!r} would reach {total} tokens, "
+                                f"the limit is {self.max_model_len}")
+            for t in e.tokens:
+                if not 0 <= int(t) < vocab:
+                    raise StepError(f"token id {t} of request {e.key!r} is outside the "
+                                    f"vocabulary of {vocab}")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise StepError(f"wanted place {w} of request {e.key!r} is outside its "
+                                    f"{n} tokens")
+        if rows > self.max_batch_tokens:
+            raise StepError(f"{rows} tokens in one step, at most {self.max_batch_tokens}")
+
+    def _pack(self, entries: Sequence[StepEntry]) -> StepView:
+        page = self.page_size
+        rcs = [self.cache.get(e.key) for e in entries]
+        starts = [rc.num_tokens for rc in rcs]
+        counts = [len(e.tokens) for e in entries]
+        totals = [s + c for s, c in zip(starts, counts)]
+        rows, seqs = sum(counts), len(entries)
+        wanted = sum(len(e.want) for e in entries)
+        width = _pow2_at_least(max((t + page - 1) // page for t in totals))
+        lay = self.inputs.layout(rows, seqs, wanted, width)
+        buf = self.inputs.begin()
+        row_start = [0]
+        r = 0
+        sample = []
+        for i, e in enumerate(entries):
+            n = counts[i]
+            buf[lay["token_ids"].start + r: lay["token_ids"].start + r + n] = np.asarray(e.tokens, dtype=np.int32)
+            buf[lay["positions"].start + r: lay["positions"].start + r + n] = np.arange(
+                starts[i], starts[i] + n, dtype=np.int32)
+            buf[lay["seq_of_row"].start + r: lay["seq_of_row"].start + r + n] = i
+            sample.extend(r + int(w) for w in e.want)
+            r += n
+            row_start.append(r)
+        buf[lay["row_start"]] = row_start
+        buf[lay["seq_start"]] = starts
+        buf[lay["seq_len"]] = totals
+        buf[lay["slots"]] = [rc.slot for rc in rcs]
+        if wanted:
+            buf[lay["sample_rows"]] = sample
+        for g in range(len(self.cache.groups)):
+            t = buf[lay[f"tables{g}"]].reshape(seqs, width)
+            t[:] = -1
+            for i, rc in enumerate(rcs):
+                tab = rc.tables[g]
+                t[i, :len(tab)] = tab
+        self.inputs.upload(lay["_end"].stop)
+        dev = self.inputs.dev
+        groups = []
+        for g, gl in enumerate(self.cache.groups):
+            k, v = self.group_tensors[g]
+            groups.append(GroupView(k=k, v=v, tables=dev[lay[f"tables{g}"]].view(seqs, width),
+                                    table_width=width, page_size=page, window=gl.need.window))
+        return StepView(
+            num_rows=rows, num_seqs=seqs,
+            token_ids=dev[lay["token_ids"]], positions=dev[lay["positions"]],
+            seq_of_row=dev[lay["seq_of_row"]], row_start=dev[lay["row_start"]],
+            seq_start=dev[lay["seq_start"]], seq_len=dev[lay["seq_len"]],
+            slots=dev[lay["slots"]], sample_rows=dev[lay["sample_rows"]],
+            h_row_start=row_start, h_seq_start=starts, h_seq_len=totals,
+            h_slots=[rc.slot for rc in rcs], max_rows_per_seq=max(counts),
+            max_seq_len=max(totals), groups=groups)
+
+    def forward(self, step: StepView, num_wanted: int) -> Optional[torch.Tensor]:
+        """Run the model over a packed step; float32 logits [wanted, vocab] or None."""
+        model = self.model
+        resid = model.embedding.forward(step.token_ids, step.num_rows)
+        pending = None
+        for i, call in enumerate(model.schedule):
+            if call.cache >= 0 and call.cache in self.cache.group_of_layer:
+                gi = self.cache.group_of_layer[call.cache]
+                step.cache = LayerCache(step.groups[gi],
+                                        self.cache.groups[gi].local_layer(call.cache),
+                                        call.writes_cache)
+            else:
+                step.cache = None
+            step.state = self.states[i]
+            pending = model.blocks[call.block].forward(resid, pending, step)
+        step.cache = None
+        step.state = None
+        if num_wanted == 0:
+            return None
+        x = model.final_norm.forward(resid, pending, rows=step.sample_rows, num_rows=num_wanted)
+        return model.head.forward(x)
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Run one batch.  Pages are reserved for every entry first; if the pool
+        cannot hold the batch, CacheFull is raised and no token has been run."""
+        self._check(entries)
+        # all or nothing over the whole batch: groups are independent, requests compete
+        need = [0] * len(self.cache.groups)
+        for e in entries:
+            total = self.cache.get(e.key).num_tokens + len(e.tokens)
+            for g, n in enumerate(self.cache.pages_needed(e.key, total)):
+                need[g] += n
+        for g, n in enumerate(need):
+            if n > self.cache.groups[g].pool.free_count:
+                raise CacheFull(f"the step needs {n} pages of group {g}, "
+                                f"{self.cache.groups[g].pool.free_count} are free")
+        for e in entries:
+            self.cache.reserve(e.key, self.cache.get(e.key).num_tokens + len(e.tokens))
+        view = self._pack(entries)
+        wanted = sum(len(e.want) for e in entries)
+        logits = self.forward(view, wanted)
+        for e in entries:
+            self.cache.advance(e.key, self.cache.get(e.key).num_tokens + len(e.tokens))
+        self.steps_run += 1
+        return logits

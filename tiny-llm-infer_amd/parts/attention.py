@@ -1,0 +1,83 @@
+"""Attention over the paged cache with grouped heads.
+
+Order (model/src/qwen3_paged_batch.cpp:147-271): q, k, v projections (no
+bias) -> optional per-head norm of q and of k -> optional rotation of q and k
+-> k and v into the cache at (table[pos // page], pos % page) -> for the row at
+position p and head h, kv head h // (heads / kv_heads), scores (q.k) * scale
+over the keys 0..p (kernels/src/paged_attention_cpu.cpp:16-69), or over
+p-window+1..p for a windowed layer, softmax, weighted sum of values -> output
+projection.  v is neither normed nor rotated.  Every row reads its keys from
+the cache, the step's own rows included, so a portion of a prompt and a single
+decoded token are the same case.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..cache.manager import CacheNeed
+from ..weights.loader import TensorDecl
+from .base import BuildEnv, Mixer, StepView, build_part, register_part
+from .linear import as_matrix, fuse_rows
+
+
+class PagedAttention(Mixer):
+    def __init__(self, spec):
+        super().__init__(spec)
+        p = spec.params
+        self.hidden = int(p["hidden_size"])
+        self.heads = int(p["num_heads"])
+        self.kv_heads = int(p["num_kv_heads"])
+        self.head_dim = int(p["head_dim"])
+        self.scale = float(p["scale"])
+        self.window = None if p.get("window") is None else int(p["window"])
+        if self.heads % self.kv_heads:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        if self.window is not None and self.window <= 0:
+            raise ValueError("window must be positive")
+        self.q_dim = self.heads * self.head_dim
+        self.kv_dim = self.kv_heads * self.head_dim
+        self.position = build_part("position", spec.parts["position"]) if "position" in spec.parts else None
+        self.q_norm = build_part("norm", spec.parts["q_norm"]) if "q_norm" in spec.parts else None
+        self.k_norm = build_part("norm", spec.parts["k_norm"]) if "k_norm" in spec.parts else None
+
+    def tensors(self) -> List[TensorDecl]:
+        n = self.spec.names
+        out = [TensorDecl(n["q"], (self.q_dim, self.hidden)),
+               TensorDecl(n["k"], (self.kv_dim, self.hidden)),
+               TensorDecl(n["v"], (self.kv_dim, self.hidden)),
+               TensorDecl(n["o"], (self.hidden, self.q_dim))]
+        for part in (self.q_norm, self.k_norm, self.position):
+            if part is not None:
+                out += part.tensors()
+        return out
+
+    def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
+        super().load(weights, env)
+        n = self.spec.names
+        self.w_qkv = fuse_rows([weights[n["q"]], weights[n["k"]], weights[n["v"]]], env)
+        self.w_o = as_matrix(weights[n["o"]], env)
+        for part in (self.q_norm, self.k_norm, self.position):
+            if part is not None:
+                part.load(weights, env)
+        env.ops.check_attention_sizes(self.heads, self.kv_heads, self.head_dim)
+
+    def cache_need(self) -> Optional[CacheNeed]:
+        return CacheNeed(self.kv_heads, self.head_dim, self.window)
+
+    def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
+        ops = self.env.ops
+        qkv = ops.linear(x, self.w_qkv)
+        rot = self.position.rotary() if self.position is not None else None
+        q = ops.qkv_to_cache(
+            qkv, step, step.cache, self.heads, self.kv_heads, self.head_dim,
+            None if self.q_norm is None else (self.q_norm.weight, self.q_norm.eps),
+            None if self.k_norm is None else (self.k_norm.weight, self.k_norm.eps),
+            rot)
+        o = ops.paged_attention(q, step, step.cache, self.heads, self.kv_heads, self.head_dim,
+                                self.scale, self.window)
+        return ops.linear(o, self.w_o)
+
+
+register_part("mixer", "paged_attention", PagedAttention)

@@ -1,0 +1,168 @@
+"""Interfaces of the parts a model is put together from, and their registries.
+
+Kinds of parts: position encoding, norm, mixer, feed-forward, block
+(arrangement), embedding, head.  A part is built from a ``PartSpec`` alone: its
+sizes and constants are ``spec.params``, the checkpoint names of its weights
+are ``spec.names``, nested parts are ``spec.parts``.  Life cycle:
+
+    part = build_part(kind_of_part, spec)        # no device needed
+    part.tensors()                               # -> [TensorDecl] it wants loaded
+    part.load(weights, env)                      # weights: name -> tensor on env.device
+    part.forward(...)                            # see each interface
+
+No part knows which architecture it is in.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional
+
+import torch
+
+from ..cache.manager import CacheNeed, StateNeed
+from ..config.base import PartSpec
+from ..weights.loader import TensorDecl
+
+
+@dataclass
+class BuildEnv:
+    """Where and how parts run."""
+    dtype: torch.dtype            # torch.bfloat16 or torch.float32: storage of activations and matrices
+    device: torch.device
+    ops: Any                      # the kernel library (kernels.ops.HipOps)
+    max_model_len: int            # highest number of positions a request may reach
+
+
+@dataclass
+class GroupView:
+    """One cache group as a step sees it."""
+    k: torch.Tensor               # [layers in group, pages, kv heads, page_size, head_dim]
+    v: torch.Tensor
+    tables: torch.Tensor          # int32 [sequences in step, table width], -1 where no page
+    table_width: int
+    page_size: int
+    window: Optional[int]
+
+
+@dataclass
+class LayerCache:
+    """The cache of the one layer call that is running."""
+    group: GroupView
+    layer: int                    # index inside the group's tensors
+    writes: bool                  # False: keys/values were written by another call of this step
+
+    @property
+    def k(self) -> torch.Tensor:
+        return self.group.k[self.layer]
+
+    @property
+    def v(self) -> torch.Tensor:
+        return self.group.v[self.layer]
+
+
+@dataclass
+class StepView:
+    """The flattened batch of one step.  Rows of one sequence are contiguous
+    and in ascending position.  Device tensors are int32."""
+    num_rows: int
+    num_seqs: int
+    token_ids: torch.Tensor       # [rows]
+    positions: torch.Tensor       # [rows]
+    seq_of_row: torch.Tensor      # [rows]  index into this step's sequences
+    row_start: torch.Tensor       # [seqs + 1]  first row of each sequence
+    seq_start: torch.Tensor       # [seqs]  position of the sequence's first row
+    seq_len: torch.Tensor         # [seqs]  tokens of the sequence after this step
+    slots: torch.Tensor           # [seqs]  the sequence's state slot
+    sample_rows: torch.Tensor     # [wanted]
+    # the same on the host, for parts that plan launches
+    h_row_start: List[int] = field(default_factory=list)
+    h_seq_start: List[int] = field(default_factory=list)
+    h_seq_len: List[int] = field(default_factory=list)
+    h_slots: List[int] = field(default_factory=list)
+    max_rows_per_seq: int = 1
+    max_seq_len: int = 1
+    groups: List[GroupView] = field(default_factory=list)
+    # filled by the runner for the layer call that is running
+    cache: Optional[LayerCache] = None
+    state: Optional[torch.Tensor] = None      # [slots, *StateNeed.shape] of the running mixer
+
+
+class Part:
+    def __init__(self, spec: PartSpec):
+        self.spec = spec
+
+    def tensors(self) -> List[TensorDecl]:
+        return []
+
+    def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
+        self.env = env
+
+
+class PositionEncoding(Part):
+    """Rotary encodings expose ``rotary()``: cos and sin tables
+    [positions, rotary_dim/2] in float32 and the pairing of elements."""
+
+    def rotary(self):
+        return None
+
+
+class Norm(Part):
+    def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor],
+                rows: Optional[torch.Tensor] = None, num_rows: Optional[int] = None) -> torch.Tensor:
+        """``resid`` (float32 [T, n]) += ``delta`` if given; return the
+        normalised rows in the run dtype.  With ``rows`` only those rows are
+        computed and ``resid`` is left unchanged."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_need(self) -> Optional[CacheNeed]:
+        return None
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
+        """x: normalised rows [T, hidden] in the run dtype; returns what is
+        added to the residual, same shape."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of norms, a mixer and a feed-forward around the residual.
+    ``forward(resid, pending, step)``: ``pending`` is what the previous block
+    still owes the residual (None for the first); returns the new pending."""
+    mixer: Mixer
+    ffn: FeedForward
+
+    def forward(self, resid: torch.Tensor, pending: Optional[torch.Tensor],
+                step: StepView) -> torch.Tensor:
+        raise NotImplementedError
+
+
+_REGISTRIES: Dict[str, Dict[str, Callable[[PartSpec], Part]]] = {
+    "position": {}, "norm": {}, "mixer": {}, "ffn": {}, "block": {}, "embedding": {}, "head": {},
+}
+
+
+def register_part(family: str, kind: str, factory: Callable[..., Part], replace: bool = False) -> None:
+    """Make ``factory(spec)`` (``factory(spec, mixer, ffn, norms)`` for blocks)
+    the implementation of ``kind`` in ``family`` (position, norm, mixer, ffn,
+    block, embedding, head)."""
+    reg = _REGISTRIES[family]
+    if kind in reg and not replace:
+        raise ValueError(f"{family} part '{kind}' is already registered")
+    reg[kind] = factory
+
+
+def build_part(family: str, spec: PartSpec, *args) -> Part:
+    reg = _REGISTRIES[family]
+    if spec.kind not in reg:
+        raise KeyError(f"no {family} part of kind '{spec.kind}' is registered; known: "
+                       f"{', '.join(sorted(reg)) or 'none'}")
+    return reg[spec.kind](spec, *args)

@@ -1,0 +1,40 @@
+"""Pre-norm residual block: n = norm(h); r = h + mixer(n); m = norm(r);
+h' = r + ffn(m) (model/src/qwen3_paged_batch.cpp:146-148, 273-279, 297-301).
+The second sum is left to whoever normalises next (the following block or the
+final norm), which adds it in float32 in the same pass as its norm."""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..weights.loader import TensorDecl
+from .base import Block, BuildEnv, StepView, register_part
+
+
+class PreNormBlock(Block):
+    def __init__(self, spec, mixer, ffn, norms):
+        super().__init__(spec)
+        self.mixer = mixer
+        self.ffn = ffn
+        self.norm_mixer = norms["mixer"]
+        self.norm_ffn = norms["ffn"]
+
+    def tensors(self) -> List[TensorDecl]:
+        return (self.norm_mixer.tensors() + self.mixer.tensors()
+                + self.norm_ffn.tensors() + self.ffn.tensors())
+
+    def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
+        super().load(weights, env)
+        for part in (self.norm_mixer, self.mixer, self.norm_ffn, self.ffn):
+            part.load(weights, env)
+
+    def forward(self, resid: torch.Tensor, pending: Optional[torch.Tensor],
+                step: StepView) -> torch.Tensor:
+        n = self.norm_mixer.forward(resid, pending)
+        a = self.mixer.forward(n, step)
+        m = self.norm_ffn.forward(resid, a)
+        return self.ffn.forward(m, step)
+
+
+register_part("block", "prenorm", PreNormBlock)

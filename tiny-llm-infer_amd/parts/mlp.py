@@ -1,0 +1,40 @@
+"""Dense gated feed-forward: down( silu(gate(x)) * up(x) ) with
+silu(g) = g / (1 + exp(-g)) (model/src/qwen3_paged_batch.cpp:281-295,
+kernels/src/swiglu_kernel_cpu.cpp:20-24).  gate and up are stacked into one
+matrix so that one product reads x once."""
+from __future__ import annotations
+
+from typing import Dict, List
+
+import torch
+
+from ..weights.loader import TensorDecl
+from .base import BuildEnv, FeedForward, StepView, register_part
+from .linear import as_matrix, fuse_rows
+
+
+class SwiGLU(FeedForward):
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.hidden = int(spec.params["hidden_size"])
+        self.inter = int(spec.params["intermediate_size"])
+
+    def tensors(self) -> List[TensorDecl]:
+        n = self.spec.names
+        return [TensorDecl(n["gate"], (self.inter, self.hidden)),
+                TensorDecl(n["up"], (self.inter, self.hidden)),
+                TensorDecl(n["down"], (self.hidden, self.inter))]
+
+    def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
+        super().load(weights, env)
+        n = self.spec.names
+        self.w_gate_up = fuse_rows([weights[n["gate"]], weights[n["up"]]], env)
+        self.w_down = as_matrix(weights[n["down"]], env)
+
+    def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
+        ops = self.env.ops
+        gu = ops.linear(x, self.w_gate_up)
+        return ops.linear(ops.swiglu(gu), self.w_down)
+
+
+register_part("ffn", "swiglu", SwiGLU)
