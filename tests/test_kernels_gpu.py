@@ -1,0 +1,367 @@
+"""Each HIP kernel alone against a plain float64 reference of the same
+operation, at sizes other than the engine's tiny configurations: odd widths,
+head sizes in steps of 16, one and many kv heads, windows, permuted pages."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from tiny_llm_infer_amd.kernels.ops import HipOps
+    return HipOps(DEV)
+
+
+def tol(dtype, scale=1.0):
+    return (3e-6 if dtype == torch.float32 else 1.2e-2) * scale
+
+
+def rnd(shape, dtype, seed, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * std).to(dtype)
+
+
+def close(got, want, dtype, what, scale=None):
+    got = got.detach().to("cpu", torch.float64)
+    want = want.to(torch.float64)
+    s = float(want.abs().max()) if scale is None else scale
+    err = float((got - want).abs().max())
+    assert err <= tol(dtype, max(s, 1e-6)), f"{what}: error {err} against scale {s}"
+
+
+# ---------------------------------------------------------------- simple ops --
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(ops, dtype):
+    table = rnd((301, 80), dtype, 1)
+    ids = torch.tensor([0, 300, 17, 17, 255], dtype=torch.int32)
+    out = ops.embed(table.to(DEV), ids.to(DEV), 5)
+    assert out.dtype == torch.float32
+    assert torch.equal(out.cpu(), table[ids.long()].float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n", [80, 100, 4096, 5120])
+def test_add_rmsnorm(ops, dtype, n):
+    rows = 7
+    resid = rnd((rows, n), torch.float32, 2, 3.0)
+    delta = rnd((rows, n), dtype, 3)
+    w = 1 + rnd((n,), torch.float32, 4, 0.1)
+    eps = 1e-5
+
+    def ref(x):
+        x = x.double()
+        return w.double() * x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+
+    # without delta the residual is untouched
+    r = resid.to(DEV)
+    out = ops.add_rmsnorm(r, None, w.to(DEV), eps, dtype)
+    assert torch.equal(r.cpu(), resid)
+    close(out, ref(resid), dtype, "norm")
+    # with delta the residual takes the float32 sum
+    out = ops.add_rmsnorm(r, delta.to(DEV), w.to(DEV), eps, dtype)
+    total = resid + delta.float()
+    assert torch.equal(r.cpu(), total)
+    close(out, ref(total), dtype, "add+norm")
+    # with a row list only those rows are computed and the residual is left alone
+    r = resid.to(DEV)
+    pick = torch.tensor([5, 0, 5], dtype=torch.int32)
+    out = ops.add_rmsnorm(r, delta.to(DEV), w.to(DEV), eps, dtype, rows=pick.to(DEV))
+    assert torch.equal(r.cpu(), resid)
+    close(out, ref(total[pick.long()]), dtype, "gathered add+norm")
+
+
+def test_rmsnorm_weight_is_a_plain_multiplier(ops):
+    x = rnd((3, 96), torch.float32, 5)
+    zero = ops.add_rmsnorm(x.to(DEV), None, torch.zeros(96, device=DEV), 1e-6, torch.float32)
+    assert float(zero.abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("inter", [112, 12288])
+def test_swiglu(ops, dtype, inter):
+    gu = rnd((5, 2 * inter), dtype, 6, 2.0)
+    out = ops.swiglu(gu.to(DEV))
+    g, u = gu[:, :inter].double(), gu[:, inter:].double()
+    close(out, torch.nn.functional.silu(g) * u, dtype, "swiglu")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("mnk", [(1, 301, 80), (37, 130, 100), (130, 70, 257), (64, 64, 64), (3, 1000, 4096)])
+def test_linear(ops, dtype, mnk):
+    M, N, K = mnk
+    x, w = rnd((M, K), dtype, 7), rnd((N, K), dtype, 8, 0.05)
+    want = x.double() @ w.double().t()
+    close(ops.linear(x.to(DEV), w.to(DEV)), want, dtype, "linear")
+    y32 = ops.linear(x.to(DEV), w.to(DEV), out_dtype=torch.float32)
+    assert y32.dtype == torch.float32
+    close(y32, want, torch.float32 if dtype == torch.float32 else dtype, "linear, float32 out",
+          scale=float(want.abs().max()) * (1.0 if dtype == torch.float32 else 0.05))
+
+
+def test_linear_rows_do_not_depend_on_the_batch(ops):
+    """float32: a row's product is bit-identical whatever else is in the batch."""
+    x, w = rnd((70, 100), torch.float32, 9), rnd((130, 100), torch.float32, 10)
+    full = ops.linear(x.to(DEV), w.to(DEV))
+    one = ops.linear(x[41:42].contiguous().to(DEV), w.to(DEV))
+    assert torch.equal(full[41:42], one)
+
+
+# ------------------------------------------------------ cache and attention --
+class FakeStep:
+    pass
+
+
+def make_step(seq_lens, new_counts, page, num_pages, seed, kv_heads, head_dim, dtype, window=None):
+    """Sequences of ``seq_lens`` tokens of which the last ``new_counts`` are
+    this step's rows; pages handed out in a random order."""
+    from tiny_llm_infer_amd.parts.base import GroupView, LayerCache, StepView
+    rng = np.random.default_rng(seed)
+    perm = rng.permutation(num_pages)
+    width = 4
+    need = max((n + page - 1) // page for n in seq_lens)
+    while width < need:
+        width *= 2
+    tables = -np.ones((len(seq_lens), width), dtype=np.int32)
+    at = 0
+    for i, n in enumerate(seq_lens):
+        nb = (n + page - 1) // page
+        tables[i, :nb] = perm[at:at + nb]
+        at += nb
+    assert at <= num_pages
+    pos, seq, row_start = [], [], [0]
+    for i, (n, c) in enumerate(zip(seq_lens, new_counts)):
+        pos += list(range(n - c, n))
+        seq += [i] * c
+        row_start.append(len(pos))
+    k = torch.zeros((1, num_pages, kv_heads, page, head_dim), dtype=dtype, device=DEV)
+    v = torch.zeros_like(k)
+    # garbage in every slot: pages not held and slots not yet written must never be read
+    k.normal_(0, 50.0)
+    v.normal_(0, 50.0)
+    i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=DEV)
+    g = GroupView(k=k, v=v, tables=i32(tables), table_width=width, page_size=page, window=window)
+    step = StepView(num_rows=len(pos), num_seqs=len(seq_lens), token_ids=i32(pos), positions=i32(pos),
+                    seq_of_row=i32(seq), row_start=i32(row_start),
+                    seq_start=i32([n - c for n, c in zip(seq_lens, new_counts)]), seq_len=i32(seq_lens),
+                    slots=i32(list(range(len(seq_lens)))), sample_rows=i32([0]),
+                    h_row_start=row_start, h_seq_start=[n - c for n, c in zip(seq_lens, new_counts)],
+                    h_seq_len=list(seq_lens), h_slots=list(range(len(seq_lens))),
+                    max_rows_per_seq=max(new_counts), max_seq_len=max(seq_lens), groups=[g])
+    step.cache = LayerCache(g, 0, True)
+    return step, tables, pos, seq
+
+
+def fill_cache(step, tables, seq_lens, kv_heads, head_dim, dtype, seed, std=1.0):
+    """Write keys and values of whole sequences into the pages; returns them."""
+    page = step.cache.group.page_size
+    ks, vs = [], []
+    for i, n in enumerate(seq_lens):
+        kk, vv = rnd((n, kv_heads, head_dim), dtype, seed + 2 * i, std), rnd((n, kv_heads, head_dim), dtype, seed + 2 * i + 1, std)
+        for t in range(n):
+            p = int(tables[i, t // page])
+            step.cache.k[p, :, t % page] = kk[t].to(DEV)
+            step.cache.v[p, :, t % page] = vv[t].to(DEV)
+        ks.append(kk)
+        vs.append(vv)
+    return ks, vs
+
+
+def ref_attention(q, ks, vs, pos, seq, heads, kv_heads, scale, window):
+    T, hd = q.shape[0], q.shape[1] // heads
+    q = q.double().reshape(T, heads, hd)
+    out = torch.zeros(T, heads, hd, dtype=torch.float64)
+    for r in range(T):
+        p = pos[r]
+        lo = 0 if not window else max(0, p - window + 1)
+        kk, vv = ks[seq[r]][lo:p + 1].double(), vs[seq[r]][lo:p + 1].double()
+        for h in range(heads):
+            g = h // (heads // kv_heads)
+            s = (kk[:, g] @ q[r, h]) * scale
+            out[r, h] = torch.softmax(s, 0) @ vv[:, g]
+    return out.reshape(T, heads * hd)
+
+
+ATT_CASES = [
+    # heads, kv_heads, head_dim, page, seq_lens, new_counts, window
+    (4, 2, 16, 8, [5, 17, 33], [5, 1, 33], None),
+    (5, 1, 48, 32, [300, 64, 1], [3, 64, 1], None),
+    (8, 2, 128, 16, [700, 259], [1, 1], None),
+    (8, 8, 64, 16, [130, 257], [130, 2], 19),
+    (6, 3, 256, 16, [90], [7], 64),
+    (32, 8, 128, 16, [513], [2], None),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", ATT_CASES)
+def test_paged_attention(ops, dtype, case):
+    heads, kv_heads, hd, page, seq_lens, new_counts, window = case
+    num_pages = sum((n + page - 1) // page for n in seq_lens) + 5
+    step, tables, pos, seq = make_step(seq_lens, new_counts, page, num_pages, 3, kv_heads, hd, dtype, window)
+    ks, vs = fill_cache(step, tables, seq_lens, kv_heads, hd, dtype, 100)
+    q = rnd((len(pos), heads * hd), dtype, 50)
+    scale = 1.0 / math.sqrt(hd)
+    out = ops.paged_attention(q.to(DEV), step, step.cache, heads, kv_heads, hd, scale, window)
+    close(out, ref_attention(q, ks, vs, pos, seq, heads, kv_heads, scale, window), dtype, "attention")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_one_far_key(ops, dtype):
+    """One key among hundreds is made to stand out: the output must be its
+    value, which a kernel that skips or misplaces a tile or a page would miss."""
+    heads, kv_heads, hd, page = 4, 1, 64, 16
+    n = 777
+    for far in (0, 15, 16, 255, 256, 300, 776):
+        step, tables, pos, seq = make_step([n], [1], page, 60, far, kv_heads, hd, dtype)
+        ks, vs = fill_cache(step, tables, [n], kv_heads, hd, dtype, 7, std=0.1)
+        q = rnd((1, heads * hd), dtype, 8, 0.1)
+        direction = torch.ones(hd) * 2.0
+        q[0, :] = direction.repeat(heads).to(dtype)
+        kfar = (direction * 2.0).to(dtype)
+        p = int(tables[0, far // page])
+        step.cache.k[p, 0, far % page] = kfar.to(DEV)
+        out = ops.paged_attention(q.to(DEV), step, step.cache, heads, kv_heads, hd, 1.0, None)
+        want = vs[0][far, 0].double().repeat(heads)
+        close(out[0], want, dtype, f"far key {far}", scale=1.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_window_edge(ops, dtype):
+    """The key just outside the window is made to stand out and must be ignored;
+    the key just inside must be found."""
+    heads, kv_heads, hd, page, window, n = 2, 2, 32, 16, 40, 100
+    for far, seen in ((n - window, True), (n - window - 1, False)):
+        step, tables, pos, seq = make_step([n], [1], page, 12, 1, kv_heads, hd, dtype, window)
+        ks, vs = fill_cache(step, tables, [n], kv_heads, hd, dtype, 9, std=0.1)
+        q = torch.full((1, heads * hd), 2.0).to(dtype)
+        p = int(tables[0, far // page])
+        step.cache.k[p, :, far % page] = torch.full((kv_heads, hd), 4.0, dtype=dtype, device=DEV)
+        ks[0][far] = 4.0
+        out = ops.paged_attention(q.to(DEV), step, step.cache, heads, kv_heads, hd, 1.0, window)
+        want = ref_attention(q, ks, vs, pos, seq, heads, kv_heads, 1.0, window)
+        close(out, want, dtype, f"window edge {far}", scale=1.0)
+        hit = float((out[0, :hd].cpu().double() - vs[0][far, 0].double()).abs().max()) < 0.05
+        assert hit == seen
+
+
+QKV_CASES = [
+    # heads, kv_heads, head_dim, rotary_dim, norms, page
+    (4, 2, 16, 16, True, 8),
+    (5, 1, 48, 48, True, 32),
+    (8, 2, 128, 128, True, 16),
+    (3, 3, 64, 32, False, 16),      # partial rotation, no norms
+    (2, 1, 80, 0, True, 16),        # no rotation at all
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", QKV_CASES)
+def test_qkv_to_cache(ops, dtype, case):
+    heads, kv_heads, hd, rd, norms, page = case
+    seq_lens, new_counts = [37, 9, 70], [5, 9, 1]
+    step, tables, pos, seq = make_step(seq_lens, new_counts, page, 20, 4, kv_heads, hd, dtype)
+    before_k = step.cache.k.clone()
+    T = len(pos)
+    qd, kd = heads * hd, kv_heads * hd
+    qkv = rnd((T, qd + 2 * kd), dtype, 11)
+    qw, kw = 1 + rnd((hd,), torch.float32, 12, 0.2), 1 + rnd((hd,), torch.float32, 13, 0.2)
+    eps_q, eps_k = 1e-5, 3e-6
+    rotary = None
+    if rd:
+        half = rd // 2
+        ang = torch.arange(128, dtype=torch.float64)[:, None] * (10000.0 ** (-2.0 * torch.arange(half, dtype=torch.float64) / rd))[None, :]
+        cos, sin = torch.cos(ang).float(), torch.sin(ang).float()
+        rotary = (cos.to(DEV), sin.to(DEV), rd)
+    q = ops.qkv_to_cache(qkv.to(DEV), step, step.cache, heads, kv_heads, hd,
+                         (qw.to(DEV), eps_q) if norms else None, (kw.to(DEV), eps_k) if norms else None, rotary)
+    x = qkv.double()
+    qq = x[:, :qd].reshape(T, heads, hd)
+    kk = x[:, qd:qd + kd].reshape(T, kv_heads, hd)
+    vv = x[:, qd + kd:].reshape(T, kv_heads, hd)
+    if norms:
+        qq = qw.double() * qq / torch.sqrt((qq * qq).mean(-1, keepdim=True) + eps_q)
+        kk = kw.double() * kk / torch.sqrt((kk * kk).mean(-1, keepdim=True) + eps_k)
+    if rd:
+        c, s = cos.double()[pos][:, None, :], sin.double()[pos][:, None, :]
+
+        def rot(t):
+            a, b, rest = t[..., :half], t[..., half:rd], t[..., rd:]
+            return torch.cat([a * c - b * s, a * s + b * c, rest], -1)
+        qq, kk = rot(qq), rot(kk)
+    close(q, qq.reshape(T, qd), dtype, "q")
+    written = torch.zeros(step.cache.k.shape[:1] + (page,), dtype=torch.bool)
+    for r in range(T):
+        p, slot = int(tables[seq[r], pos[r] // page]), pos[r] % page
+        close(step.cache.k[p, :, slot], kk[r], dtype, "k in cache")
+        assert torch.equal(step.cache.v[p, :, slot].cpu(), qkv[r, qd + kd:].reshape(kv_heads, hd))
+        written[p, slot] = True
+    # nothing else in the cache was touched
+    untouched = ~written[:, None, :, None].expand_as(before_k.cpu())
+    assert torch.equal(step.cache.k.cpu()[untouched], before_k.cpu()[untouched])
+
+
+def test_rotation_pairs_halves_not_neighbours(ops):
+    """A head with only element i set: after the rotation at a position whose
+    angle for pair i is 90 degrees, the value has moved to element i + d/2."""
+    heads, kv_heads, hd, page = 1, 1, 16, 8
+    step, tables, pos, seq = make_step([2], [1], page, 2, 0, kv_heads, hd, torch.float32)
+    half = hd // 2
+    cos = torch.zeros(4, half)
+    sin = torch.ones(4, half)           # every pair turned by 90 degrees
+    qkv = torch.zeros(1, 3 * hd)
+    qkv[0, 3] = 1.0
+    q = ops.qkv_to_cache(qkv.to(DEV), step, step.cache, heads, kv_heads, hd, None, None,
+                         (cos.to(DEV), sin.to(DEV), hd))
+    want = torch.zeros(hd)
+    want[3 + half] = 1.0
+    assert torch.allclose(q[0].cpu(), want, atol=1e-7)
+
+
+# ------------------------------------------------------------------ sampling --
+def test_greedy_takes_the_lowest_index_on_ties(ops):
+    logits = torch.zeros(3, 5000)
+    logits[0, 4000] = logits[0, 77] = logits[0, 4999] = 3.0
+    logits[1, 0] = 1.0
+    logits[2, 4999] = 1.0
+    out = ops.sample(logits.to(DEV))
+    assert out.cpu().tolist() == [77, 0, 4999]
+
+
+def test_temperature_sampling_is_gumbel_max_over_a_hash(ops):
+    from tiny_llm_infer_amd.kernels.ops import sample_uniform
+    rows, vocab = 4, 301
+    logits = rnd((rows, vocab), torch.float32, 21, 2.0)
+    temps = torch.tensor([0.7, 0.0, 1.5, 0.7])
+    seeds = torch.tensor([12345, 1, 2 ** 40 + 17, 12346], dtype=torch.int64)
+    out = ops.sample(logits.to(DEV), temps.to(DEV), seeds.to(DEV)).cpu().tolist()
+    for r in range(rows):
+        if temps[r] <= 1e-6:
+            want = int(torch.argmax(logits[r]))
+        else:
+            u = np.array([sample_uniform(int(seeds[r]), t) for t in range(vocab)], dtype=np.float64)
+            assert 0 < u.min() and u.max() < 1
+            score = logits[r].double().numpy() + float(temps[r]) * -np.log(-np.log(u))
+            want = int(np.argmax(score))
+        assert out[r] == want
+    # the same seed gives the same token whatever else is in the batch
+    alone = ops.sample(logits[3:4].contiguous().to(DEV), temps[3:4].to(DEV), seeds[3:4].to(DEV)).cpu().tolist()
+    assert alone[0] == out[3]
+
+
+def test_temperature_sampling_follows_softmax(ops):
+    vocab, n = 6, 4000
+    base = torch.tensor([2.0, 1.0, 0.0, -1.0, 0.5, 1.5])
+    T = 0.8
+    logits = base.repeat(n, 1)
+    seeds = torch.arange(1, n + 1, dtype=torch.int64) * 7919
+    out = ops.sample(logits.to(DEV), torch.full((n,), T).to(DEV), seeds.to(DEV)).cpu()
+    freq = torch.bincount(out.long(), minlength=vocab).double() / n
+    want = torch.softmax(base.double() / T, 0)
+    assert float((freq - want).abs().max()) < 0.03

@@ -1,0 +1,139 @@
+"""Replay on the GPU against the plain implementation, in float32 and in
+bfloat16: each request alone and whole; most of it in one step and the last 32
+tokens one by one; in portions of changing size, down to two tokens; and
+mixed, up to four live requests with so few pages that they are used again."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import (TINY, collect, max_error, plain_logits, random_prompt, trace_mixed,
+                     trace_portions, trace_prefill_then_decode, trace_whole)
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# largest |difference| allowed, relative to the largest |logit| of the request
+TOL = {"float32": 2e-5, "bfloat16": 2.5e-2}
+
+
+def _runner(folder, name, dtype, max_tokens, page=None):
+    from tiny_llm_infer_amd.engine.loading import load_model
+    from tiny_llm_infer_amd.engine.runner import ModelRunner
+    model, cfg = load_model(folder, dtype, "cuda:0")
+    page = page or TINY[name]["page_size"]
+    return ModelRunner(model, model.env, page_size=page, num_pages=max_tokens // page,
+                       max_requests=4, max_batch_tokens=1024)
+
+
+def _requests(name, lengths, seed):
+    vocab = TINY[name]["vocab_size"]
+    return {f"r{i}": random_prompt(vocab, n, seed + i) for i, n in enumerate(lengths)}
+
+
+def _replay(runner, steps):
+    from tiny_llm_infer_amd.engine.replay import Replayer
+    rp = Replayer(runner)
+    return {st["step"]: rp.run_step(st) for st in steps}
+
+
+def _check(got, want, dtype, label):
+    worst = 0.0
+    for rid in want:
+        err, row, scale = max_error(got[rid], want[rid])
+        worst = max(worst, err / scale)
+        assert err <= TOL[dtype] * scale, (f"{label}/{rid}: error {err:.3e} at token {row} "
+                                           f"(logit scale {scale:.3e})")
+    return worst
+
+
+@pytest.fixture(scope="module")
+def oracle(model_folders):
+    out = {}
+    for name in TINY:
+        reqs = _requests(name, [70, 45, 97, 33, 58, 121], seed=5)
+        out[name] = (reqs, plain_logits(model_folders[name], reqs))
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("cut", ["whole", "decode", "portions", "mixed"])
+def test_cuts_match_plain(model_folders, oracle, name, dtype, cut):
+    reqs, want = oracle[name]
+    max_tokens = 320
+    steps = {"whole": lambda: trace_whole(reqs),
+             "decode": lambda: trace_prefill_then_decode(reqs),
+             "portions": lambda: trace_portions(reqs, seed=3),
+             "mixed": lambda: trace_mixed(reqs, max_tokens=max_tokens, seed=9)}[cut]()
+    runner = _runner(model_folders[name], name, dtype, max_tokens)
+    got = collect(steps, _replay(runner, steps))
+    worst = _check(got, want, dtype, f"{name}/{dtype}/{cut}")
+    print(f"{name} {dtype} {cut}: worst relative error {worst:.2e}")
+    runner.cache.check()
+    assert all(f == runner.cache.num_pages for f in runner.cache.free_pages())
+    if cut == "mixed":
+        assert runner.cache.pages_taken_total > runner.cache.num_pages
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_float32_cuts_agree_bit_for_bit(model_folders, oracle, name):
+    """In float32 every kernel adds in an order that depends on the row alone,
+    so all ways of cutting give identical logits."""
+    reqs, _ = oracle[name]
+    outs = []
+    for steps in (trace_whole(reqs), trace_prefill_then_decode(reqs), trace_portions(reqs, 1),
+                  trace_mixed(reqs, 320, seed=4)):
+        runner = _runner(model_folders[name], name, "float32", 320)
+        outs.append(collect(steps, _replay(runner, steps)))
+    for other in outs[1:]:
+        for rid in reqs:
+            assert np.array_equal(outs[0][rid], other[rid]), rid
+
+
+def test_long_decoding_and_first_tokens(model_folders):
+    """One request decoded token by token from its very first token, far past
+    several pages and past the window of configuration B."""
+    name = "B"
+    reqs = _requests(name, [300], seed=77)
+    want = plain_logits(model_folders[name], reqs)
+    toks = reqs["r0"]
+    steps = [{"step": i, "entries": [{"id": "r0", "tokens": [t], "want": [0]}],
+              "end": ["r0"] if i == len(toks) - 1 else []} for i, t in enumerate(toks)]
+    for dtype in ("float32", "bfloat16"):
+        runner = _runner(model_folders[name], name, dtype, 320)
+        got = collect(steps, _replay(runner, steps))
+        _check(got, want, dtype, f"long decode {dtype}")
+        # the first tokens on their own
+        err, _, scale = max_error(got["r0"][:3], want["r0"][:3])
+        assert err <= TOL[dtype] * scale
+
+
+def test_trace_run_program(model_folders, tmp_path):
+    """bin/trace_run as a user runs it: JSON lines in, 'done <step>' lines and
+    <step>.f32 files out."""
+    name = "A"
+    reqs = _requests(name, [40, 70], seed=31)
+    want = plain_logits(model_folders[name], reqs)
+    steps = trace_mixed(reqs, max_tokens=192, seed=2)
+    for dtype in ("float32", "bfloat16"):
+        out_dir = tmp_path / dtype
+        proc = subprocess.run(
+            [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_folders[name],
+             "--dtype", dtype, "--out", str(out_dir), "--max-tokens", "192"],
+            input="".join(json.dumps(s) + "\n" for s in steps), text=True,
+            stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert proc.stdout.split("\n")[:-1] == [f"done {s['step']}" for s in steps]
+        vocab = TINY[name]["vocab_size"]
+        outputs = {}
+        for s in steps:
+            path = out_dir / f"{s['step']}.f32"
+            if sum(len(e["want"]) for e in s["entries"]):
+                outputs[s["step"]] = np.fromfile(path, dtype="<f4").reshape(-1, vocab)
+        got = collect(steps, outputs)
+        _check(got, want, dtype, f"trace_run {dtype}")

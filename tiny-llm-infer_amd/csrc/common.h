@@ -1,0 +1,79 @@
+// Shared by all kernels: storage types, conversions, reductions over a
+// 64-lane wavefront and over a workgroup, and the error channel of the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define TLI_WAVE 64
+
+typedef uint16_t bf16_t;   // bfloat16 storage: the upper 16 bits of a float
+
+// dtype codes of the C ABI
+#define TLI_F32 0
+#define TLI_BF16 1
+
+extern "C" const char* tli_last_error();
+int tli_fail(const char* fmt, ...);          // records a message, returns 1
+int tli_check_launch(const char* what);      // hipGetLastError -> message
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+    return __uint_as_float(((uint32_t)v) << 16);
+}
+
+// round to nearest, ties to even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return bf16_to_f32(v); }
+__device__ __forceinline__ void from_f32(float* p, float v) { *p = v; }
+__device__ __forceinline__ void from_f32(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+
+// Makes LDS writes of this wavefront's lanes visible to its other lanes.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = TLI_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, TLI_WAVE);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = TLI_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, TLI_WAVE));
+    return v;
+}
+
+// Sum over a workgroup of up to 1024 threads; every thread gets the result.
+// `scratch` holds at least 16 floats of LDS.  The order of additions is fixed.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE;
+    const int waves = (blockDim.x + TLI_WAVE - 1) / TLI_WAVE;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < waves; ++w) total += scratch[w];
+    return total;
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE;
+    const int waves = (blockDim.x + TLI_WAVE - 1) / TLI_WAVE;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = scratch[0];
+    for (int w = 1; w < waves; ++w) total = fmaxf(total, scratch[w]);
+    return total;
+}

@@ -1,0 +1,106 @@
+// Embedding gather, residual-add + RMSNorm, SwiGLU.
+//
+// embed:       resid[t, :] = float(table[id[t], :])                       (layers/src/embedding.cpp:37-44)
+// add_rmsnorm: v = resid[r] (+ delta[r]);  out = w * v * 1/sqrt(mean(v^2) + eps), in float32
+//              (kernels/src/rmsnorm_kernel_cpu.cpp:27-43; the sum h + a of
+//              model/src/qwen3_paged_batch.cpp:273-275 is done here, unrounded)
+// swiglu:      out = g / (1 + exp(-g)) * u over a fused [rows, 2*inter] input
+//              (kernels/src/swiglu_kernel_cpu.cpp:20-24)
+#include "common.h"
+
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                             float* __restrict__ out, int hidden, int vocab) {
+    const int row = blockIdx.x;
+    int id = ids[row];
+    if (id < 0 || id >= vocab) id = 0;          // the host rejects such ids before the launch
+    const T* src = table + (size_t)id * hidden;
+    float* dst = out + (size_t)row * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32(src[i]);
+}
+
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+                                   const float* __restrict__ weight, T* __restrict__ out,
+                                   const int* __restrict__ rows, int n, float eps, int total_rows) {
+    __shared__ float scratch[16];
+    const int out_row = blockIdx.x;
+    int r = rows ? rows[out_row] : out_row;
+    if (r < 0 || r >= total_rows) r = 0;
+    float* x = resid + (size_t)r * n;
+    const T* d = delta ? delta + (size_t)r * n : nullptr;
+    const bool update = (rows == nullptr) && (d != nullptr);
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        float v = x[i];
+        if (d) v += to_f32(d[i]);
+        if (update) x[i] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)n + eps);
+    T* o = out + (size_t)out_row * n;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        float v = x[i];
+        if (d && !update) v += to_f32(d[i]);
+        from_f32(o + i, weight[i] * v * scale);
+    }
+}
+
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const size_t row = idx / inter;
+    const int col = (int)(idx - row * inter);
+    const float g = to_f32(gu[row * 2 * inter + col]);
+    const float u = to_f32(gu[row * 2 * inter + inter + col]);
+    from_f32(out + idx, g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int tli_embed(const void* table, const int* ids, float* out, int rows, int hidden,
+                         int vocab, int dtype, void* stream) {
+    if (rows <= 0) return 0;
+    if (hidden <= 0 || vocab <= 0) return tli_fail("embed: bad sizes hidden=%d vocab=%d", hidden, vocab);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TLI_F32)
+        embed_kernel<float><<<rows, 256, 0, s>>>((const float*)table, ids, out, hidden, vocab);
+    else if (dtype == TLI_BF16)
+        embed_kernel<bf16_t><<<rows, 256, 0, s>>>((const bf16_t*)table, ids, out, hidden, vocab);
+    else
+        return tli_fail("embed: unknown dtype %d", dtype);
+    return tli_check_launch("embed");
+}
+
+extern "C" int tli_add_rmsnorm(float* resid, const void* delta, const float* weight, void* out,
+                               const int* rows, int out_rows, int total_rows, int n, float eps,
+                               int dtype, void* stream) {
+    if (out_rows <= 0) return 0;
+    if (n <= 0) return tli_fail("add_rmsnorm: bad row size %d", n);
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = n >= 2048 ? 512 : 256;
+    if (dtype == TLI_F32)
+        add_rmsnorm_kernel<float><<<out_rows, threads, 0, s>>>(resid, (const float*)delta, weight,
+                                                             (float*)out, rows, n, eps, total_rows);
+    else if (dtype == TLI_BF16)
+        add_rmsnorm_kernel<bf16_t><<<out_rows, threads, 0, s>>>(resid, (const bf16_t*)delta, weight,
+                                                              (bf16_t*)out, rows, n, eps, total_rows);
+    else
+        return tli_fail("add_rmsnorm: unknown dtype %d", dtype);
+    return tli_check_launch("add_rmsnorm");
+}
+
+extern "C" int tli_swiglu(const void* gu, void* out, int rows, int inter, int dtype, void* stream) {
+    if (rows <= 0) return 0;
+    if (inter <= 0) return tli_fail("swiglu: bad size %d", inter);
+    hipStream_t s = (hipStream_t)stream;
+    const size_t total = (size_t)rows * inter;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    if (dtype == TLI_F32)
+        swiglu_kernel<float><<<blocks, 256, 0, s>>>((const float*)gu, (float*)out, inter, total);
+    else if (dtype == TLI_BF16)
+        swiglu_kernel<bf16_t><<<blocks, 256, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, inter, total);
+    else
+        return tli_fail("swiglu: unknown dtype %d", dtype);
+    return tli_check_launch("swiglu");
+}

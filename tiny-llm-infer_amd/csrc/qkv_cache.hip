@@ -1,0 +1,128 @@
+// Per-head norm of q and k, rotation, and the write of k and v into the paged
+// cache, in one pass over the fused projection output.
+//
+// For every row and head, in float32 (model/src/qwen3_paged_batch.cpp:160-227):
+//   q, k:  x <- w * x / sqrt(mean(x^2) + eps)  over the head      (if a norm is given)
+//          (x_i, x_{i+rd/2}) <- (x_i cos - x_{i+rd/2} sin, x_i sin + x_{i+rd/2} cos), i < rd/2
+//                                                 (kernels/src/rope_kernel_cpu.cpp:156-179)
+//   k, v -> cache[page = table[seq][pos / page_size]][kv head][pos % page_size][:]
+// q goes to its own [rows, heads*head_dim] buffer.  The cache layout differs from
+// the reference's [page][slot][kv_dim] (kernels/src/paged_attention_cuda.cu:58-67):
+// here the slots of one head in one page are contiguous.
+#include "common.h"
+
+#define QKV_MAX_HEAD_DIM 512
+#define QKV_WAVES 4
+
+template <typename T>
+__global__ void qkv_to_cache_kernel(
+    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const int* __restrict__ positions, const int* __restrict__ seq_of_row,
+    const int* __restrict__ tables, int table_width, int page_size, int num_pages,
+    int heads, int kv_heads, int head_dim,
+    const float* __restrict__ q_norm_w, float q_eps, const float* __restrict__ k_norm_w, float k_eps,
+    const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rotary_dim,
+    int table_positions, int write_cache) {
+    __shared__ float stage[QKV_WAVES][QKV_MAX_HEAD_DIM];
+    const int row = blockIdx.x;
+    const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE;
+    const int q_dim = heads * head_dim, kv_dim = kv_heads * head_dim;
+    const int stride = q_dim + 2 * kv_dim;
+    const int pos = positions[row];
+    const T* src_row = qkv + (size_t)row * stride;
+
+    // where this row's keys and values go
+    size_t cache_base = 0;
+    bool can_write = false;
+    if (write_cache) {
+        const int seq = seq_of_row[row];
+        const int page = tables[(size_t)seq * table_width + pos / page_size];
+        can_write = page >= 0 && page < num_pages;
+        cache_base = ((size_t)page * kv_heads * page_size + (size_t)(pos % page_size)) * head_dim;
+    }
+    const int half = rotary_dim / 2;
+    const float* cos_row = nullptr;
+    const float* sin_row = nullptr;
+    if (cos_table && pos >= 0 && pos < table_positions) {
+        cos_row = cos_table + (size_t)pos * half;
+        sin_row = sin_table + (size_t)pos * half;
+    }
+
+    float* x = stage[wave];
+    // heads 0..heads-1 are q, heads..heads+kv_heads-1 are k
+    for (int h = wave; h < heads + kv_heads; h += QKV_WAVES) {
+        const bool is_q = h < heads;
+        const T* src = src_row + (size_t)h * head_dim;     // q heads then k heads are contiguous
+        const float* nw = is_q ? q_norm_w : k_norm_w;
+        const float eps = is_q ? q_eps : k_eps;
+        float ss = 0.f;
+        for (int i = lane; i < head_dim; i += TLI_WAVE) {
+            const float v = to_f32(src[i]);
+            x[i] = v;
+            ss += v * v;
+        }
+        if (nw) {
+            ss = wave_sum(ss);
+            const float scale = 1.0f / sqrtf(ss / (float)head_dim + eps);
+            for (int i = lane; i < head_dim; i += TLI_WAVE) x[i] = nw[i] * x[i] * scale;
+        }
+        // lanes only touch the elements they wrote themselves until here; the
+        // rotation reads a partner element written by another lane of this wave
+        wave_lds_sync();
+        T* dst;
+        if (is_q) {
+            dst = q_out + (size_t)row * q_dim + (size_t)h * head_dim;
+        } else {
+            if (!can_write) continue;
+            dst = k_cache + cache_base + (size_t)(h - heads) * page_size * head_dim;
+        }
+        for (int i = lane; i < head_dim; i += TLI_WAVE) {
+            float v = x[i];
+            if (cos_row && i < rotary_dim) {
+                if (i < half) v = x[i] * cos_row[i] - x[i + half] * sin_row[i];
+                else v = x[i - half] * sin_row[i - half] + x[i] * cos_row[i - half];
+            }
+            from_f32(dst + i, v);
+        }
+        wave_lds_sync();
+    }
+    if (can_write) {
+        const T* vsrc = src_row + q_dim + kv_dim;
+        for (int i = threadIdx.x; i < kv_dim; i += blockDim.x) {
+            const int g = i / head_dim, d = i - g * head_dim;
+            v_cache[cache_base + (size_t)g * page_size * head_dim + d] = vsrc[i];
+        }
+    }
+}
+
+extern "C" int tli_qkv_to_cache(
+    const void* qkv, void* q_out, void* k_cache, void* v_cache, const int* positions,
+    const int* seq_of_row, const int* tables, int table_width, int page_size, int num_pages,
+    int rows, int heads, int kv_heads, int head_dim,
+    const float* q_norm_w, float q_eps, const float* k_norm_w, float k_eps,
+    const float* cos_table, const float* sin_table, int rotary_dim, int table_positions,
+    int write_cache, int dtype, void* stream) {
+    if (rows <= 0) return 0;
+    if (head_dim <= 0 || head_dim > QKV_MAX_HEAD_DIM)
+        return tli_fail("qkv_to_cache: head_dim %d is outside 1..%d", head_dim, QKV_MAX_HEAD_DIM);
+    if (heads <= 0 || kv_heads <= 0) return tli_fail("qkv_to_cache: bad head counts");
+    if (cos_table && (rotary_dim <= 0 || rotary_dim % 2 || rotary_dim > head_dim))
+        return tli_fail("qkv_to_cache: rotary_dim %d must be even and at most head_dim %d", rotary_dim, head_dim);
+    if (write_cache && (page_size <= 0 || table_width <= 0 || num_pages <= 0))
+        return tli_fail("qkv_to_cache: bad cache geometry");
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = QKV_WAVES * TLI_WAVE;
+    if (dtype == TLI_F32)
+        qkv_to_cache_kernel<float><<<rows, threads, 0, s>>>(
+            (const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache, positions, seq_of_row,
+            tables, table_width, page_size, num_pages, heads, kv_heads, head_dim, q_norm_w, q_eps,
+            k_norm_w, k_eps, cos_table, sin_table, rotary_dim, table_positions, write_cache);
+    else if (dtype == TLI_BF16)
+        qkv_to_cache_kernel<bf16_t><<<rows, threads, 0, s>>>(
+            (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, positions, seq_of_row,
+            tables, table_width, page_size, num_pages, heads, kv_heads, head_dim, q_norm_w, q_eps,
+            k_norm_w, k_eps, cos_table, sin_table, rotary_dim, table_positions, write_cache);
+    else
+        return tli_fail("qkv_to_cache: unknown dtype %d", dtype);
+    return tli_check_launch("qkv_to_cache");
+}

@@ -1,0 +1,69 @@
+// Sampling from float32 logits: arg-max, or Gumbel-max for a temperature.
+//
+// Greedy picks the largest logit, the lowest token id on ties
+// (engine/src/llm_engine.cpp:81-85; kernels/src/sampling_kernel_cuda.cu:25-27).
+// With temperature T > 1e-6 the score of token v is logit_v + T * (-log(-log u_v))
+// (kernels/src/sampling_kernel_cuda.cu:50-54).  The reference draws u from
+// Philox keyed by the thread index; here u_v is a hash of (seed, v) alone, so
+// the draw does not depend on the launch shape or on the batch.
+#include "common.h"
+
+#define SAMPLE_THREADS 1024
+
+__host__ __device__ inline uint32_t tli_mix32(uint32_t h) {
+    h ^= h >> 16; h *= 0x85ebca6bu; h ^= h >> 13; h *= 0xc2b2ae35u; h ^= h >> 16;
+    return h;
+}
+
+// uniform in (0, 1): 24 bits of a hash of (seed, token)
+__host__ __device__ inline float tli_uniform(uint32_t seed_lo, uint32_t seed_hi, uint32_t token) {
+    uint32_t h = tli_mix32(token ^ 0x9e3779b9u);
+    h = tli_mix32(h ^ seed_lo);
+    h = tli_mix32(h + seed_hi * 0x85ebca6bu + 0x27d4eb2fu);
+    return ((float)(h >> 8) + 0.5f) * (1.0f / 16777216.0f);
+}
+
+__global__ void sample_kernel(const float* __restrict__ logits, int vocab,
+                              const float* __restrict__ temperatures,
+                              const uint32_t* __restrict__ seeds, int* __restrict__ out) {
+    __shared__ float best_v[SAMPLE_THREADS / TLI_WAVE];
+    __shared__ int best_i[SAMPLE_THREADS / TLI_WAVE];
+    const int row = blockIdx.x;
+    const float* l = logits + (size_t)row * vocab;
+    const float temp = temperatures ? temperatures[row] : 0.f;
+    const uint32_t lo = seeds ? seeds[2 * row] : 0u, hi = seeds ? seeds[2 * row + 1] : 0u;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int t = threadIdx.x; t < vocab; t += blockDim.x) {
+        float s = l[t];
+        if (temp > 1.0e-6f) s += temp * -logf(-logf(tli_uniform(lo, hi, (uint32_t)t)));
+        if (s > bv || (s == bv && t < bi)) { bv = s; bi = t; }
+    }
+    for (int off = TLI_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, TLI_WAVE);
+        const int oi = __shfl_xor(bi, off, TLI_WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE;
+    if (lane == 0) { best_v[wave] = bv; best_i[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x / TLI_WAVE); ++w)
+            if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) { bv = best_v[w]; bi = best_i[w]; }
+        out[row] = (bi == 0x7fffffff) ? 0 : bi;
+    }
+}
+
+// temperatures: float [rows] or null (greedy); seeds: uint32 [rows][2] (low, high word) or null
+extern "C" int tli_sample(const float* logits, int rows, int vocab, const float* temperatures,
+                          const uint32_t* seeds, int* out, void* stream) {
+    if (rows <= 0) return 0;
+    if (vocab <= 0) return tli_fail("sample: bad vocabulary size %d", vocab);
+    sample_kernel<<<rows, SAMPLE_THREADS, 0, (hipStream_t)stream>>>(logits, vocab, temperatures, seeds, out);
+    return tli_check_launch("sample");
+}
+
+// the same draw on the host, for tests and for callers that hold logits there
+extern "C" float tli_sample_uniform(uint32_t seed_lo, uint32_t seed_hi, uint32_t token) {
+    return tli_uniform(seed_lo, seed_hi, token);
+}

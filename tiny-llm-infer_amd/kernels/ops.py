@@ -1,0 +1,247 @@
+"""The kernel library as the parts see it: hand-written HIP kernels for gfx950,
+called through a C ABI on torch tensors.  There is no CPU path and no
+fallback: without the library, or without a GPU, construction fails.
+
+Every wrapper checks on the host that shapes, dtypes and devices are what the
+kernel and its grid assume before anything is launched.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_void_p
+from typing import Optional, Tuple
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"kernels take float32 or bfloat16 tensors, not {dtype}")
+
+
+_LIB = None
+
+
+def load_library():
+    """Load (building it first if nothing is built) the shared library."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    path = build.find_library() or build.build_library()
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as exc:
+        raise KernelError(f"cannot load the kernel library {path}: {exc}") from None
+    lib.tli_last_error.restype = ctypes.c_char_p
+    P, I, F = c_void_p, c_int, c_float
+    sigs = {
+        "tli_abi_version": [],
+        "tli_embed": [P, P, P, I, I, I, I, P],
+        "tli_add_rmsnorm": [P, P, P, P, P, I, I, I, F, I, P],
+        "tli_swiglu": [P, P, I, I, I, P],
+        "tli_qkv_to_cache": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I, I, I, I, P],
+        "tli_attention_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
+        "tli_gemm_plain": [P, P, P, I, I, I, I, I, I, P],
+        "tli_sample": [P, I, I, P, P, P, P],
+    }
+    for name, args in sigs.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = c_int
+    lib.tli_sample_uniform.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32]
+    lib.tli_sample_uniform.restype = c_float
+    _LIB = lib
+    return lib
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+class HipOps:
+    name = "hip-gfx950"
+    MAX_HEAD_DIM = 512
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise KernelError(f"the kernels run on an AMD GPU ('cuda:N' in torch), not on '{device}'")
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible to torch; this engine has no CPU path")
+        self.lib = load_library()
+
+    # ---- helpers ----------------------------------------------------------
+    def _stream(self):
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    def _call(self, fn, *args):
+        if fn(*args) != 0:
+            raise KernelError(self.lib.tli_last_error().decode())
+
+    def _want(self, t: torch.Tensor, what: str, dtype=None, shape=None):
+        if t.device != self.device:
+            raise KernelError(f"{what} is on {t.device}, expected {self.device}")
+        if not t.is_contiguous():
+            raise KernelError(f"{what} must be contiguous")
+        if dtype is not None and t.dtype != dtype:
+            raise KernelError(f"{what} has dtype {t.dtype}, expected {dtype}")
+        if shape is not None and tuple(t.shape) != tuple(shape):
+            raise KernelError(f"{what} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+
+    # ---- limits that parts ask about at build time --------------------------
+    def check_attention_sizes(self, heads: int, kv_heads: int, head_dim: int) -> None:
+        if head_dim % 16 or not 16 <= head_dim <= self.MAX_HEAD_DIM:
+            raise KernelError(f"head_dim {head_dim} is not supported: the attention kernels take "
+                              f"multiples of 16 from 16 to {self.MAX_HEAD_DIM}")
+        if heads <= 0 or kv_heads <= 0 or heads % kv_heads:
+            raise KernelError(f"{heads} heads cannot be grouped over {kv_heads} kv heads")
+
+    def check_page_size(self, page_size: int) -> None:
+        if page_size <= 0 or page_size > 256 or page_size & (page_size - 1):
+            raise KernelError(f"page size {page_size} is not supported: powers of two up to 256")
+
+    # ---- ops ------------------------------------------------------------------
+    def embed(self, table: torch.Tensor, token_ids: torch.Tensor, num_rows: int) -> torch.Tensor:
+        vocab, hidden = table.shape
+        self._want(table, "embedding table")
+        self._want(token_ids, "token ids", torch.int32)
+        if token_ids.numel() < num_rows:
+            raise KernelError("fewer token ids than rows")
+        out = torch.empty((num_rows, hidden), dtype=torch.float32, device=self.device)
+        self._call(self.lib.tli_embed, table.data_ptr(), token_ids.data_ptr(), out.data_ptr(),
+                   num_rows, hidden, vocab, _dtype_code(table.dtype), self._stream())
+        return out
+
+    def add_rmsnorm(self, resid, delta, weight, eps, out_dtype, rows=None, num_rows=None):
+        total, n = resid.shape
+        self._want(resid, "residual", torch.float32)
+        self._want(weight, "norm weight", torch.float32, (n,))
+        if delta is not None:
+            self._want(delta, "residual delta", out_dtype, (total, n))
+        out_rows = total
+        if rows is not None:
+            self._want(rows, "row list", torch.int32)
+            out_rows = rows.numel() if num_rows is None else num_rows
+            if rows.numel() < out_rows:
+                raise KernelError("row list is shorter than the rows asked for")
+        out = torch.empty((out_rows, n), dtype=out_dtype, device=self.device)
+        self._call(self.lib.tli_add_rmsnorm, resid.data_ptr(), _ptr(delta), weight.data_ptr(),
+                   out.data_ptr(), _ptr(rows), out_rows, total, n, float(eps),
+                   _dtype_code(out_dtype), self._stream())
+        return out
+
+    def linear(self, x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
+        M, K = x.shape
+        N, K2 = w.shape
+        if K != K2:
+            raise KernelError(f"linear: input has {K} columns, the matrix {K2}")
+        self._want(x, "linear input")
+        self._want(w, "linear matrix")
+        if x.dtype != w.dtype:
+            raise KernelError(f"linear: input is {x.dtype}, the matrix {w.dtype}")
+        out_dtype = out_dtype or x.dtype
+        y = torch.empty((M, N), dtype=out_dtype, device=self.device)
+        self._call(self.lib.tli_gemm_plain, x.data_ptr(), w.data_ptr(), y.data_ptr(), M, N, K,
+                   _dtype_code(x.dtype), _dtype_code(w.dtype), _dtype_code(out_dtype), self._stream())
+        return y
+
+    def swiglu(self, gu: torch.Tensor) -> torch.Tensor:
+        rows, two = gu.shape
+        if two % 2:
+            raise KernelError("swiglu input must hold gate and up side by side")
+        self._want(gu, "swiglu input")
+        out = torch.empty((rows, two // 2), dtype=gu.dtype, device=self.device)
+        self._call(self.lib.tli_swiglu, gu.data_ptr(), out.data_ptr(), rows, two // 2,
+                   _dtype_code(gu.dtype), self._stream())
+        return out
+
+    def qkv_to_cache(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary):
+        T = step.num_rows
+        q_dim, kv_dim = heads * head_dim, kv_heads * head_dim
+        self._want(qkv, "qkv", None, (T, q_dim + 2 * kv_dim))
+        q = torch.empty((T, q_dim), dtype=qkv.dtype, device=self.device)
+        qw, qe = q_norm if q_norm is not None else (None, 0.0)
+        kw, ke = k_norm if k_norm is not None else (None, 0.0)
+        for w in (qw, kw):
+            if w is not None:
+                self._want(w, "head norm weight", torch.float32, (head_dim,))
+        cos = sin = None
+        rd = npos = 0
+        if rotary is not None:
+            cos, sin, rd = rotary
+            npos = cos.shape[0]
+            self._want(cos, "cos table", torch.float32, (npos, rd // 2))
+            self._want(sin, "sin table", torch.float32, (npos, rd // 2))
+            if step.max_seq_len > npos:
+                raise KernelError(f"a position reaches {step.max_seq_len}, the rotation table has {npos}")
+        write = 1 if (cache is not None and cache.writes) else 0
+        k_ptr = v_ptr = tab_ptr = None
+        width = page = pages = 0
+        if write:
+            kc, vc = cache.k, cache.v
+            g = cache.group
+            self._check_cache(kc, vc, g, kv_heads, head_dim, qkv.dtype, step)
+            k_ptr, v_ptr, tab_ptr = kc.data_ptr(), vc.data_ptr(), g.tables.data_ptr()
+            width, page, pages = g.table_width, g.page_size, kc.shape[0]
+        self._call(self.lib.tli_qkv_to_cache, qkv.data_ptr(), q.data_ptr(), k_ptr, v_ptr,
+                   step.positions.data_ptr(), step.seq_of_row.data_ptr(), tab_ptr, width, page, pages,
+                   T, heads, kv_heads, head_dim, _ptr(qw), float(qe), _ptr(kw), float(ke),
+                   _ptr(cos), _ptr(sin), rd, npos, write, _dtype_code(qkv.dtype), self._stream())
+        return q
+
+    def _check_cache(self, kc, vc, g, kv_heads, head_dim, dtype, step):
+        pages = kc.shape[0]
+        want = (pages, kv_heads, g.page_size, head_dim)
+        for t, what in ((kc, "key cache"), (vc, "value cache")):
+            self._want(t, what, dtype, want)
+        self._want(g.tables, "block tables", torch.int32, (step.num_seqs, g.table_width))
+        if (step.max_seq_len + g.page_size - 1) // g.page_size > g.table_width:
+            raise KernelError("a block table is narrower than its sequence needs")
+
+    def paged_attention(self, q, step, cache, heads, kv_heads, head_dim, scale, window):
+        T = step.num_rows
+        self._want(q, "queries", None, (T, heads * head_dim))
+        if cache is None:
+            raise KernelError("attention needs a cache layer")
+        kc, vc, g = cache.k, cache.v, cache.group
+        self._check_cache(kc, vc, g, kv_heads, head_dim, q.dtype, step)
+        out = torch.empty_like(q)
+        self._call(self.lib.tli_attention_plain, q.data_ptr(), out.data_ptr(), kc.data_ptr(),
+                   vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
+                   g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], T, heads, kv_heads,
+                   head_dim, float(scale), int(window or 0), _dtype_code(q.dtype), self._stream())
+        return out
+
+    def sample(self, logits: torch.Tensor, temperatures: Optional[torch.Tensor] = None,
+               seeds: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Token ids int32 [rows].  ``temperatures`` float32 [rows] (None: greedy);
+        ``seeds`` int64 [rows], one draw seed per row."""
+        rows, vocab = logits.shape
+        self._want(logits, "logits", torch.float32)
+        if temperatures is not None:
+            self._want(temperatures, "temperatures", torch.float32, (rows,))
+            if seeds is None:
+                raise KernelError("sampling with a temperature needs seeds")
+            self._want(seeds, "seeds", torch.int64, (rows,))
+        out = torch.empty((rows,), dtype=torch.int32, device=self.device)
+        self._call(self.lib.tli_sample, logits.data_ptr(), rows, vocab, _ptr(temperatures),
+                   _ptr(seeds) if temperatures is not None else None, out.data_ptr(), self._stream())
+        return out
+
+
+def sample_uniform(seed: int, token: int) -> float:
+    """The uniform number the sampling kernel draws for (seed, token)."""
+    lib = load_library()
+    seed &= (1 << 64) - 1
+    return float(lib.tli_sample_uniform(seed & 0xFFFFFFFF, seed >> 32, token))
