@@ -99,3 +99,47 @@ class CpuOps:
                 w = torch.softmax(s, dim=0)
                 out[r, h] = w @ vv[:, h // mul]
         return out.reshape(T, heads * head_dim).to(q.dtype)
+
+    # ---- sampling: the same hash and rule as csrc/sampling.hip, in Python ----
+    @staticmethod
+    def _mix32(h):
+        h &= 0xFFFFFFFF
+        h ^= h >> 16
+        h = (h * 0x85EBCA6B) & 0xFFFFFFFF
+        h ^= h >> 13
+        h = (h * 0xC2B2AE35) & 0xFFFFFFFF
+        h ^= h >> 16
+        return h
+
+    @classmethod
+    def uniform(cls, seed, token):
+        seed &= (1 << 64) - 1
+        lo, hi = seed & 0xFFFFFFFF, seed >> 32
+        h = cls._mix32(token ^ 0x9E3779B9)
+        h = cls._mix32(h ^ lo)
+        h = cls._mix32((h + hi * 0x85EBCA6B + 0x27D4EB2F) & 0xFFFFFFFF)
+        return ((h >> 8) + 0.5) / 16777216.0
+
+    def sample(self, logits, temperatures=None, seeds=None, top_p=None):
+        import math
+        out = []
+        for r in range(logits.shape[0]):
+            row = logits[r].double()
+            temp = 0.0 if temperatures is None else float(temperatures[r])
+            if temp <= 1e-6:
+                out.append(int(torch.argmax(row)))
+                continue
+            keep = torch.ones_like(row, dtype=torch.bool)
+            if top_p is not None and float(top_p[r]) < 1.0:
+                w = torch.exp((row - row.max()) / temp)
+                order = torch.argsort(w, descending=True)
+                csum = torch.cumsum(w[order], 0)
+                n = int((csum < float(top_p[r]) * w.sum()).sum()) + 1
+                keep[:] = False
+                keep[order[:n]] = True
+            seed = int(seeds[r])
+            g = torch.tensor([-math.log(-math.log(self.uniform(seed, t))) for t in range(row.numel())],
+                             dtype=torch.float64)
+            score = torch.where(keep, row + temp * g, torch.full_like(row, -float("inf")))
+            out.append(int(torch.argmax(score)))
+        return torch.tensor(out, dtype=torch.int32)

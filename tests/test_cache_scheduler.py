@@ -1,0 +1,247 @@
+"""The cache manager (no page lost, held twice or freed twice, under random
+orders of requests; windows give pages back) and the scheduler's decisions
+(decode first, portions under the token budget, preemption when pages run
+out).  No GPU."""
+import random
+
+import pytest
+
+from tiny_llm_infer_amd.cache import CacheFull, CacheManager, CacheNeed, PageError, PagePool
+from tiny_llm_infer_amd.engine.scheduler import Scheduler, SchedulerConfig, SchedulerError
+from tiny_llm_infer_amd.engine.sequence import Sequence, Status
+from tiny_llm_infer_amd.sampling.params import SamplingParams
+
+FULL = CacheNeed(2, 16, None)
+WIN = CacheNeed(2, 16, 20)
+
+
+# --------------------------------------------------------------------- pages --
+def test_pool_hands_out_the_lowest_free_page_and_refuses_double_release():
+    pool = PagePool(4)
+    assert [pool.take() for _ in range(3)] == [0, 1, 2]
+    pool.release(1)
+    assert pool.take() == 1
+    pool.release(0)
+    with pytest.raises(PageError):
+        pool.release(0)
+    with pytest.raises(PageError):
+        pool.release(9)
+    assert pool.take() == 0 and pool.take() == 3
+    with pytest.raises(PageError):
+        pool.take()
+    pool.check()
+
+
+def test_groups_have_pages_of_their_own():
+    m = CacheManager([FULL, WIN, FULL, None, WIN], page_size=8, num_pages=10, max_requests=2)
+    assert [g.cache_layers for g in m.groups] == [[0, 2], [1, 4]]
+    m.admit("a")
+    m.reserve("a", 20)
+    assert m.free_pages() == [7, 7]
+    assert m.get("a").tables[0] == [0, 1, 2] and m.get("a").tables[1] == [0, 1, 2]
+    m.release("a")
+    assert m.free_pages() == [10, 10]
+    m.check()
+
+
+def test_window_pages_are_given_back_when_passed():
+    m = CacheManager([FULL, WIN], page_size=8, num_pages=64, max_requests=1)
+    m.admit("a")
+    m.reserve("a", 50)
+    m.advance("a", 50)
+    # the next query is at 50 and reads 31..50: blocks 0..2 (slots 0..23) are passed
+    assert m.get("a").tables[1][:4] == [-1, -1, -1, 3]
+    assert m.get("a").tables[0][:4] == [0, 1, 2, 3]
+    held = 64 - m.free_pages()[1]
+    assert held == 4
+    for n in range(51, 200):
+        m.reserve("a", n)
+        m.advance("a", n)
+        live = [p for p in m.get("a").tables[1] if p >= 0]
+        assert len(live) <= 20 // 8 + 2          # the window, not the history
+        first = (n - 20 + 1) // 8
+        assert all(p < 0 for p in m.get("a").tables[1][:first])
+        assert all(p >= 0 for p in m.get("a").tables[1][first:(n + 7) // 8])
+    m.check()
+    m.release("a")
+    assert m.free_pages() == [64, 64]
+
+
+def test_reserve_is_all_or_nothing():
+    m = CacheManager([FULL, WIN], page_size=8, num_pages=3, max_requests=2)
+    m.admit("a")
+    m.admit("b")
+    m.reserve("a", 16)
+    assert not m.can_reserve("b", 17)
+    with pytest.raises(CacheFull):
+        m.reserve("b", 17)
+    assert m.free_pages() == [1, 1] and m.get("b").tables == [[], []]
+    m.reserve("b", 8)
+    with pytest.raises(ValueError):
+        m.advance("b", 9)                         # more than was reserved
+    with pytest.raises(CacheFull):
+        m.admit("c")                              # no slot
+    m.check()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_lose_no_page(seed):
+    rng = random.Random(seed)
+    m = CacheManager([FULL, WIN, FULL, WIN], page_size=4, num_pages=40, max_requests=5)
+    live = {}
+    taken_slots = set()
+    for it in range(600):
+        r = rng.random()
+        if r < 0.2 and len(live) < 5:
+            key = f"q{it}"
+            rc = m.admit(key)
+            assert rc.slot not in taken_slots
+            taken_slots.add(rc.slot)
+            live[key] = 0
+        elif r < 0.85 and live:
+            key = rng.choice(list(live))
+            n = live[key] + rng.choice([1, 1, 1, 2, 5, 9, 17])
+            if m.can_reserve(key, n):
+                m.reserve(key, n)
+                m.advance(key, n)
+                live[key] = n
+            else:
+                with pytest.raises(CacheFull):
+                    m.reserve(key, n)
+        elif live:
+            key = rng.choice(list(live))
+            taken_slots.discard(m.get(key).slot)
+            m.release(key)
+            del live[key]
+        m.check()
+        # every token a later query may read is held
+        for key, n in live.items():
+            rc = m.get(key)
+            for gi, g in enumerate(m.groups):
+                lo = 0 if g.need.window is None else max(0, n - g.need.window + 1)
+                for pos in range(lo, n):
+                    assert rc.tables[gi][pos // 4] >= 0
+    for key in list(live):
+        m.release(key)
+    m.check()
+    assert m.free_pages() == [40, 40]
+    assert m.pages_taken_total == m.pages_returned_total > 80      # pages were used again
+
+
+# ----------------------------------------------------------------- scheduler --
+def _seq(i, n, max_tokens=4):
+    return Sequence(i, list(range(n)), n, SamplingParams(max_tokens=max_tokens, ignore_eos=True))
+
+
+def _run(sched, plan, token=1):
+    """Pretend the model ran: advance the cache and post-process."""
+    for item in plan.sequences:
+        s = item.sequence
+        sched.cache.reserve(s.request_id, item.token_start + item.token_count)
+        sched.cache.advance(s.request_id, item.token_start + item.token_count)
+    return sched.postprocess(plan, [token if i.samples else None for i in plan.sequences], lambda t: False)
+
+
+def test_prompts_are_cut_to_the_token_budget_one_portion_a_step():
+    cache = CacheManager([FULL], page_size=8, num_pages=100, max_requests=4)
+    s = Scheduler(SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=24), cache)
+    a, b = _seq(1, 50), _seq(2, 10)
+    s.add(a)
+    s.add(b)
+    p = s.schedule()
+    assert [(i.sequence.request_id, i.token_start, i.token_count, i.is_prefill) for i in p.sequences] == \
+        [(1, 0, 24, True)]
+    _run(s, p)
+    p = s.schedule()          # b is now first in the queue, a went to the back
+    assert [(i.sequence.request_id, i.token_start, i.token_count) for i in p.sequences] == \
+        [(2, 0, 10), (1, 24, 14)]
+    assert [i.samples for i in p.sequences] == [True, False]
+    _run(s, p)
+    assert b.status == Status.RUNNING and b.size == 11
+    p = s.schedule()          # decode first, then the rest of a's prompt
+    assert [(i.sequence.request_id, i.token_start, i.token_count, i.is_prefill) for i in p.sequences] == \
+        [(2, 10, 1, False), (1, 38, 12, True)]
+    assert p.num_tokens == 13
+    _run(s, p)
+    p = s.schedule()
+    assert [(i.sequence.request_id, i.is_prefill) for i in p.sequences] == [(2, False), (1, False)]
+
+
+def test_max_num_seqs_limits_a_step_and_running_requests_take_turns():
+    cache = CacheManager([FULL], page_size=8, num_pages=100, max_requests=8)
+    s = Scheduler(SchedulerConfig(max_num_seqs=2, max_num_batched_tokens=100), cache)
+    for i in range(1, 4):
+        s.add(_seq(i, 5, max_tokens=10))
+    p = s.schedule()
+    assert [i.sequence.request_id for i in p.sequences] == [1, 2]
+    _run(s, p)
+    p = s.schedule()          # two running requests fill the step; 3 waits
+    assert [i.sequence.request_id for i in p.sequences] == [1, 2]
+    _run(s, p)
+
+
+def test_requests_finish_at_max_tokens_or_eos_and_give_everything_back():
+    cache = CacheManager([FULL, WIN], page_size=8, num_pages=10, max_requests=2)
+    s = Scheduler(SchedulerConfig(2, 64), cache)
+    a = Sequence(1, [5, 6, 7], 3, SamplingParams(max_tokens=3))
+    b = Sequence(2, [5, 6], 2, SamplingParams(max_tokens=50))
+    s.add(a)
+    s.add(b)
+    done = []
+    for step in range(3):
+        p = s.schedule()
+        for item in p.sequences:
+            cache.reserve(item.sequence.request_id, item.token_start + item.token_count)
+            cache.advance(item.sequence.request_id, item.token_start + item.token_count)
+        # b draws the end-of-sequence token 99 in the second step
+        toks = [99 if (i.sequence is b and step == 1) else 1 for i in p.sequences]
+        done += s.postprocess(p, toks, lambda t: t == 99)
+    assert [d.request_id for d in done] == [2, 1]
+    assert b.completion_tokens == [1, 99] and a.completion_tokens == [1, 1, 1]
+    assert s.is_finished() and cache.free_pages() == [10, 10] and cache.free_slots() == 2
+    cache.check()
+
+
+def test_when_pages_run_out_the_request_is_preempted_and_computed_again():
+    cache = CacheManager([FULL], page_size=4, num_pages=4, max_requests=4)
+    s = Scheduler(SchedulerConfig(4, 64), cache)
+    a, b = _seq(1, 7, max_tokens=8), _seq(2, 7, max_tokens=8)
+    s.add(a)
+    s.add(b)
+    _run(s, s.schedule())                       # both prompts: 2 pages each, pool full
+    assert cache.free_pages() == [0]
+    p = s.schedule()                            # both decode at position 7: still fits
+    assert len(p.sequences) == 2
+    _run(s, p)
+    p = s.schedule()                            # position 8 needs a third page: a is preempted,
+    assert s.num_preemptions == 1               # its pages let b go on
+    assert [(i.sequence.request_id, i.is_prefill) for i in p.sequences] == [(2, False)]
+    assert a.status == Status.WAITING and not a.admitted and a.preemptions == 1
+    assert s.waiting[0] is a
+    _run(s, p)
+    # b runs to its end; then a is admitted again and recomputes prompt + generated tokens
+    while b.status != Status.FINISHED:
+        _run(s, s.schedule())
+    p = s.schedule()
+    assert [(i.sequence.request_id, i.token_start, i.token_count, i.is_prefill) for i in p.sequences] == \
+        [(1, 0, 9, True)]
+    while not s.is_finished():
+        _run(s, s.schedule())
+    assert a.completion_size == 8 and b.completion_size == 8
+    assert cache.free_pages() == [4]
+    cache.check()
+
+
+def test_a_prompt_larger_than_the_pool_is_an_error_and_a_stuck_queue_too():
+    cache = CacheManager([FULL], page_size=4, num_pages=2, max_requests=2)
+    s = Scheduler(SchedulerConfig(2, 64), cache)
+    s.add(_seq(1, 9))
+    with pytest.raises(SchedulerError, match="more KV blocks"):
+        s.schedule()
+    cache = CacheManager([FULL], page_size=4, num_pages=2, max_requests=2)
+    cache.admit("someone else")
+    cache.reserve("someone else", 8)
+    s = Scheduler(SchedulerConfig(2, 64), cache)
+    s.add(_seq(1, 5))
+    with pytest.raises(SchedulerError, match="could not make progress"):
+        s.schedule()

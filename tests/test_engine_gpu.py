@@ -1,0 +1,138 @@
+"""Generation through the entry points on the GPU: the Python engine and the
+command line, greedy against the plain implementation, the BASELINE workloads
+of the two tiny configurations, and top-p sampling against a plain version."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3
+from cpu_ops import CpuOps
+from helpers import TINY, random_prompt
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _engine(folder, name, dtype, **kw):
+    from tiny_llm_infer_amd.engine.llm_engine import LLMEngine
+    args = dict(dtype=dtype, device="cuda:0", max_model_len=128, page_size=TINY[name]["page_size"],
+                num_kv_blocks=64, max_num_seqs=4, max_num_batched_tokens=24)
+    args.update(kw)
+    return LLMEngine.from_folder(folder, **args)
+
+
+def test_greedy_generation_float32_equals_plain(model_folders):
+    from tiny_llm_infer_amd.sampling.params import SamplingParams
+    folder = model_folders["A"]
+    cfg, w = plain_qwen3.read_model(folder)
+    prompts = [random_prompt(256, n, 40 + n) for n in (5, 17, 33)]
+    want = [plain_qwen3.greedy(cfg, w, p, 16) for p in prompts]
+    eng = _engine(folder, "A", "float32")
+    got = eng.generate(prompts, SamplingParams(max_tokens=16, ignore_eos=True))
+    assert [r.token_ids for r in got] == want
+    small = _engine(folder, "A", "float32", num_kv_blocks=9)       # preemption and recompute
+    got = small.generate(prompts, SamplingParams(max_tokens=16, ignore_eos=True))
+    assert [r.token_ids for r in got] == want and small.scheduler.num_preemptions > 0
+    small.runner.cache.check()
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_greedy_generation_bfloat16_follows_plain(model_folders, name):
+    """In bfloat16 a near-tie may fall the other way, so each generated token
+    is checked against the plain logits for the engine's own prefix: it must be
+    the plain arg-max or within the rounding margin of it."""
+    from tiny_llm_infer_amd.sampling.params import SamplingParams
+    folder = model_folders[name]
+    cfg, w = plain_qwen3.read_model(folder)
+    vocab = TINY[name]["vocab_size"]
+    prompts = [random_prompt(vocab, n, 90 + n) for n in (3, 21, 40)]
+    eng = _engine(folder, name, "bfloat16")
+    got = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
+    same = 0
+    for p, r in zip(prompts, got):
+        logits = plain_qwen3.forward(cfg, w, p + r.token_ids[:-1])[len(p) - 1:]
+        for t, row in zip(r.token_ids, logits):
+            margin = 2.5e-2 * float(row.abs().max())
+            assert float(row.max() - row[t]) <= 2 * margin
+            same += int(t == int(row.argmax()))
+    assert same >= 30          # of 36
+
+
+def test_temperature_workload_of_configuration_b(model_folders):
+    """Five requests with prompts of 1..40 tokens, 12 tokens each at temperature
+    0.7 with fixed seeds, page 16, budget 32: the tokens are those a plain
+    sampler draws from the engine's own float32 logits, and do not depend on
+    the batch."""
+    from tiny_llm_infer_amd.sampling.params import SamplingParams
+    folder = model_folders["B"]
+    prompts = [random_prompt(384, n, 70 + n) for n in (1, 9, 40, 23, 14)]
+    params = [SamplingParams(max_tokens=12, temperature=0.7, ignore_eos=True, seed=100 + i)
+              for i in range(5)]
+    eng = _engine(folder, "B", "float32", max_num_batched_tokens=32)
+    together = eng.generate(prompts, params)
+    alone = [_engine(folder, "B", "float32", max_num_batched_tokens=32).generate([p], [s])[0]
+             for p, s in zip(prompts, params)]
+    assert [r.token_ids for r in together] == [r.token_ids for r in alone]
+    # the same engine logic on the CPU stand-in draws the same tokens
+    from tiny_llm_infer_amd.engine.llm_engine import LLMEngine
+    cpu = LLMEngine.from_folder(folder, dtype="float32", device="cpu", max_model_len=128, page_size=16,
+                                num_kv_blocks=64, max_num_seqs=4, max_num_batched_tokens=32, ops=CpuOps())
+    ref = cpu.generate(prompts, params)
+    agree = sum(a == b for r, c in zip(together, ref) for a, b in zip(r.token_ids, c.token_ids))
+    assert agree >= 55         # of 60; a draw on a near-tie may differ between float32 libraries
+
+
+def test_top_p_kernel_against_plain():
+    from tiny_llm_infer_amd.kernels.ops import HipOps
+    ops = HipOps("cuda:0")
+    rows, vocab = 6, 500
+    g = torch.Generator().manual_seed(2)
+    logits = torch.randn(rows, vocab, generator=g) * 3
+    temps = torch.tensor([0.7, 1.0, 0.0, 0.5, 2.0, 1.0])
+    top_p = torch.tensor([0.9, 0.5, 0.3, 1.0, 0.05, 1e-6])
+    seeds = torch.arange(1, rows + 1, dtype=torch.int64) * 104729
+    got = ops.sample(logits.cuda(), temps.cuda(), seeds.cuda(), top_p=top_p.cuda()).cpu().tolist()
+    want = CpuOps().sample(logits, temps, seeds, top_p).tolist()
+    assert got == want
+    assert got[5] == int(logits[5].argmax())        # a vanishing top_p keeps the best token only
+
+
+def test_command_line_infer(model_folders):
+    folder = model_folders["A"]
+    cfg, w = plain_qwen3.read_model(folder)
+    prompts = [random_prompt(256, 7, 1), random_prompt(256, 19, 2)]
+    want = [plain_qwen3.greedy(cfg, w, p, 5) for p in prompts]
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "model_main"), "--infer", "--model", folder,
+           "--dtype", "float32", "--max-new-tokens", "5", "--max-seq-len", "64", "--num-kv-blocks", "16",
+           "--page-size", "8", "--ignore-eos"]
+    for p in prompts:
+        cmd += ["--prompt-ids", ",".join(map(str, p))]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = [list(map(int, l.split())) for l in proc.stdout.strip().split("\n")]
+    assert lines == want
+    # usage errors exit with 2
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "model_main"), "--infer", "--model", folder],
+                         stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=600)
+    assert bad.returncode == 2
+
+
+def test_command_line_bench(model_folders):
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "model_main"), "--bench", "--model", model_folders["B"],
+           "--num-seqs", "3", "--min-input-len", "4", "--max-input-len", "9", "--min-output-len", "3",
+           "--max-output-len", "5", "--warmup", "1", "--repeats", "2", "--max-seq-len", "64"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    out = proc.stdout.strip().split("\n")
+    assert out[0].startswith("run=0 output_tokens=") and "output_tokens_per_second=" in out[-1]
+    assert out[-1].startswith("aggregate_runs=2")
+
+
+def test_the_library_is_needed():
+    from tiny_llm_infer_amd.kernels.ops import HipOps, KernelError
+    with pytest.raises(KernelError):
+        HipOps("cpu")

@@ -1,0 +1,84 @@
+"""The engine end to end on the CPU stand-in kernels: greedy generation equals
+the plain implementation token for token, also when the pool is so small that
+requests are preempted and computed again; temperature sampling does not
+depend on the batch."""
+import pytest
+
+import plain_qwen3
+from cpu_ops import CpuOps
+from helpers import TINY, random_prompt
+from tiny_llm_infer_amd.engine.llm_engine import LLMEngine
+from tiny_llm_infer_amd.sampling.params import SamplingParams
+
+
+def _engine(folder, name, **kw):
+    args = dict(dtype="float32", device="cpu", max_model_len=128, page_size=TINY[name]["page_size"],
+                num_kv_blocks=64, max_num_seqs=4, max_num_batched_tokens=24, ops=CpuOps())
+    args.update(kw)
+    return LLMEngine.from_folder(folder, **args)
+
+
+def test_greedy_generation_matches_plain(model_folders):
+    """BASELINE workload of configuration A: prompts of 5/17/33 tokens, 16
+    greedy tokens each, page 8, budget 24."""
+    folder = model_folders["A"]
+    cfg, w = plain_qwen3.read_model(folder)
+    prompts = [random_prompt(256, n, 40 + n) for n in (5, 17, 33)]
+    want = [plain_qwen3.greedy(cfg, w, p, 16) for p in prompts]
+    eng = _engine(folder, "A")
+    got = eng.generate(prompts, SamplingParams(max_tokens=16, ignore_eos=True))
+    assert [r.token_ids for r in got] == want
+    assert eng.total_generated_tokens == 48
+    eng.runner.cache.check()
+    assert eng.runner.cache.free_pages() == [64]
+    # a pool too small for all three at once: preemption, same tokens
+    small = _engine(folder, "A", num_kv_blocks=9)
+    got = small.generate(prompts, SamplingParams(max_tokens=16, ignore_eos=True))
+    assert [r.token_ids for r in got] == want
+    assert small.scheduler.num_preemptions > 0 and sum(r.preemptions for r in got) > 0
+    small.runner.cache.check()
+
+
+def test_admission_checks(model_folders):
+    eng = _engine(model_folders["A"], "A", max_model_len=32)
+    with pytest.raises(ValueError, match="at least one token"):
+        eng.add_request([], SamplingParams())
+    with pytest.raises(ValueError, match="exceeds max_model_len"):
+        eng.add_request([1] * 33, SamplingParams(max_tokens=1))
+    with pytest.raises(ValueError, match="completion exceeds"):
+        eng.add_request([1] * 30, SamplingParams(max_tokens=4))
+    with pytest.raises(ValueError, match="greater than zero"):
+        eng.add_request([1], SamplingParams(max_tokens=0))
+    with pytest.raises(ValueError, match="top_p"):
+        eng.add_request([1], SamplingParams(top_p=0.0))
+    with pytest.raises(ValueError, match="vocabulary"):
+        eng.add_request([256], SamplingParams(max_tokens=4))
+    eng.add_request([1] * 30, SamplingParams(max_tokens=3))     # exactly fits: 30 + 3 - 1 = 32
+
+
+def test_eos_stops_a_request(model_folders):
+    folder = model_folders["A"]
+    cfg, w = plain_qwen3.read_model(folder)
+    prompt = random_prompt(256, 12, 5)
+    free_run = plain_qwen3.greedy(cfg, w, prompt, 8)
+    eng = _engine(folder, "A")
+    eng.eos_token_ids = {free_run[3]}
+    cut = free_run.index(free_run[3]) + 1
+    assert eng.generate([prompt], SamplingParams(max_tokens=8))[0].token_ids == free_run[:cut]
+    assert eng.generate([prompt], SamplingParams(max_tokens=8, ignore_eos=True))[0].token_ids == free_run
+
+
+def test_temperature_tokens_do_not_depend_on_the_batch(model_folders):
+    """Configuration B's workload: temperature 0.7 with fixed seeds; a request
+    gives the same tokens alone and among others (and under top_p)."""
+    folder = model_folders["B"]
+    prompts = [random_prompt(384, n, 70 + n) for n in (1, 9, 40, 23, 14)]
+    params = [SamplingParams(max_tokens=12, temperature=0.7, ignore_eos=True, seed=100 + i,
+                             top_p=1.0 if i % 2 else 0.9) for i in range(5)]
+    eng = _engine(folder, "B", max_num_batched_tokens=32)
+    together = eng.generate(prompts, params)
+    alone = [_engine(folder, "B", max_num_batched_tokens=32).generate([p], [s])[0]
+             for p, s in zip(prompts, params)]
+    assert [r.token_ids for r in together] == [r.token_ids for r in alone]
+    greedy = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
+    assert [r.token_ids for r in greedy] != [r.token_ids for r in together]

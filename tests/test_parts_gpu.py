@@ -1,0 +1,236 @@
+"""Each part alone on the GPU against the plain implementation's function for
+it, and a toy mixer with state of its own that is registered, built and
+stepped from this test file without a change to the framework."""
+import math
+
+import pytest
+import torch
+
+import plain_qwen3 as P
+from test_kernels_gpu import DEV, close, make_step, rnd
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def envs():
+    from tiny_llm_infer_amd.engine.loading import make_env
+    return {dt: make_env(dt, DEV, max_model_len=256) for dt in DTYPES}
+
+
+def _weights(decls, dtype, seed=0):
+    from tiny_llm_infer_amd.weights import random_tensors
+    return {n: t.to(DEV) for n, t in random_tensors(decls, seed, dtype)}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_part(envs, dtype):
+    from tiny_llm_infer_amd.config import PartSpec
+    from tiny_llm_infer_amd.parts import build_part
+    part = build_part("norm", PartSpec("rmsnorm", {"size": 72, "eps": 2e-5}, {"weight": "n.w"}))
+    w = _weights(part.tensors(), dtype)
+    part.load(w, envs[dtype])
+    resid = rnd((6, 72), torch.float32, 1, 2.0)
+    delta = rnd((6, 72), dtype, 2)
+    r = resid.to(DEV)
+    out = part.forward(r, delta.to(DEV))
+    total = resid.double() + delta.double()
+    close(out, P.rmsnorm(total, w["n.w"].cpu().double(), 2e-5), dtype, "rmsnorm part")
+    assert torch.allclose(r.cpu().double(), total, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_part_tables(envs, dtype):
+    from tiny_llm_infer_amd.config import PartSpec
+    from tiny_llm_infer_amd.parts import build_part
+    part = build_part("position", PartSpec("rope_neox", {"head_dim": 48, "theta": 50000.0,
+                                                          "max_positions": 200}))
+    part.load({}, envs[dtype])
+    cos, sin, rd = part.rotary()
+    assert rd == 48 and cos.shape == (200, 24)
+    ang = P.rope_angles(48, 50000.0, list(range(200)))
+    assert torch.allclose(cos.cpu().double(), torch.cos(torch.from_numpy(ang).double()), atol=1e-7)
+    assert torch.allclose(sin.cpu().double(), torch.sin(torch.from_numpy(ang).double()), atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu_part(envs, dtype):
+    from tiny_llm_infer_amd.config import PartSpec
+    from tiny_llm_infer_amd.parts import build_part
+    part = build_part("ffn", PartSpec("swiglu", {"hidden_size": 80, "intermediate_size": 112},
+                                      {"gate": "g", "up": "u", "down": "d"}))
+    w = _weights(part.tensors(), dtype)
+    part.load(w, envs[dtype])
+    x = rnd((9, 80), dtype, 3)
+    f = {k: v.cpu().double() for k, v in w.items()}
+    want = P.linear(P.swiglu(P.linear(x.double(), f["g"]), P.linear(x.double(), f["u"])), f["d"])
+    close(part.forward(x.to(DEV), None), want, dtype, "swiglu part")
+
+
+def _attention_spec(heads, kv, hd, hidden, window, theta=1e4, eps=1e-6):
+    from tiny_llm_infer_amd.config import PartSpec
+    norm = lambda n: PartSpec("rmsnorm", {"size": hd, "eps": eps}, {"weight": n})
+    return PartSpec("paged_attention",
+                    {"hidden_size": hidden, "num_heads": heads, "num_kv_heads": kv, "head_dim": hd,
+                     "scale": hd ** -0.5, "window": window},
+                    {"q": "q", "k": "k", "v": "v", "o": "o"},
+                    {"position": PartSpec("rope_neox", {"head_dim": hd, "theta": theta, "max_positions": 256}),
+                     "q_norm": norm("qn"), "k_norm": norm("kn")})
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [None, 7])
+def test_attention_part_whole_sequence(envs, dtype, window):
+    """One whole sequence through the attention part in one step equals the
+    plain attention block."""
+    from tiny_llm_infer_amd.parts import build_part
+    heads, kv, hd, hidden, T = 6, 2, 32, 80, 45
+    part = build_part("mixer", _attention_spec(heads, kv, hd, hidden, window))
+    w = _weights(part.tensors(), dtype, seed=4)
+    part.load(w, envs[dtype])
+    assert part.cache_need().window == window
+    step, tables, pos, seq = make_step([T], [T], 16, 5, 0, kv, hd, dtype, window)
+    x = rnd((T, hidden), dtype, 5)
+    out = part.forward(x.to(DEV), step)
+    f = {("self." + k + ("_proj.weight" if k in "qkvo" else "")): v.cpu().double() for k, v in w.items()}
+    f["self.q_norm.weight"], f["self.k_norm.weight"] = f.pop("self.qn"), f.pop("self.kn")
+    cfg = dict(num_attention_heads=heads, num_key_value_heads=kv, head_dim=hd, hidden_size=hidden,
+               rms_norm_eps=1e-6, rope_theta=1e4)
+    want = P.attention_block(x.double(), f, "self.", cfg, list(range(T)), window)
+    close(out, want, dtype, "attention part")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_prenorm_block(envs, dtype):
+    from tiny_llm_infer_amd.config import PartSpec
+    from tiny_llm_infer_amd.parts import build_part
+    heads, kv, hd, hidden, inter, T = 4, 4, 16, 48, 64, 20
+    mixer = build_part("mixer", _attention_spec(heads, kv, hd, hidden, None))
+    ffn = build_part("ffn", PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": inter},
+                                     {"gate": "g", "up": "u", "down": "d"}))
+    norms = {"mixer": build_part("norm", PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6}, {"weight": "n1"})),
+             "ffn": build_part("norm", PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6}, {"weight": "n2"}))}
+    block = build_part("block", PartSpec("prenorm"), mixer, ffn, norms)
+    w = _weights(block.tensors(), dtype, seed=6)
+    block.load(w, envs[dtype])
+    step, *_ = make_step([T], [T], 8, 4, 0, kv, hd, dtype)
+    h0 = rnd((T, hidden), torch.float32, 7)
+    resid = h0.to(DEV)
+    pending = block.forward(resid, None, step)
+    f = {k: v.cpu().double() for k, v in w.items()}
+    att = {"s.q_proj.weight": f["q"], "s.k_proj.weight": f["k"], "s.v_proj.weight": f["v"],
+           "s.o_proj.weight": f["o"], "s.q_norm.weight": f["qn"], "s.k_norm.weight": f["kn"]}
+    cfg = dict(num_attention_heads=heads, num_key_value_heads=kv, head_dim=hd, hidden_size=hidden,
+               rms_norm_eps=1e-6, rope_theta=1e4)
+    h = h0.double()
+    r = h + P.attention_block(P.rmsnorm(h, f["n1"], 1e-6), att, "s.", cfg, list(range(T)), None)
+    m = P.rmsnorm(r, f["n2"], 1e-6)
+    d = P.linear(P.swiglu(P.linear(m, f["g"]), P.linear(m, f["u"])), f["d"])
+    close(resid, r, dtype, "residual after the mixer")     # the second sum is still owed
+    close(pending, d, dtype, "what the block owes the residual")
+
+
+# ------------------------------------------------------------------ toy mixer --
+def test_toy_mixer_with_state_of_its_own(tmp_path):
+    """A mixer defined here, keeping a running sum per request in a state slot:
+    y_t = W . mean(x_0..x_t).  It is registered, built into a model of a toy
+    architecture and stepped in several cuts through the framework's runner,
+    cache manager and replay, none of which is changed for it."""
+    import json
+
+    import numpy as np
+
+    from helpers import collect, trace_mixed, trace_portions, trace_whole
+    from tiny_llm_infer_amd import register_architecture
+    from tiny_llm_infer_amd.cache import StateNeed
+    from tiny_llm_infer_amd.config import BlockSpec, JsonReader, LayerCall, ModelSpec, PartSpec
+    from tiny_llm_infer_amd.engine.loading import load_model, write_random_model
+    from tiny_llm_infer_amd.engine.replay import Replayer
+    from tiny_llm_infer_amd.engine.runner import ModelRunner
+    from tiny_llm_infer_amd.parts import Mixer, register_part
+    from tiny_llm_infer_amd.weights import TensorDecl
+
+    class RunningMean(Mixer):
+        def __init__(self, spec):
+            super().__init__(spec)
+            self.n = spec.params["size"]
+
+        def tensors(self):
+            return [TensorDecl(self.spec.names["w"], (self.n, self.n))]
+
+        def load(self, weights, env):
+            super().load(weights, env)
+            self.w = weights[self.spec.names["w"]].float()
+
+        def state_need(self):
+            return StateNeed((self.n,), torch.float32)
+
+        def forward(self, x, step):
+            out = torch.empty_like(x)
+            for i in range(step.num_seqs):
+                r0, r1 = step.h_row_start[i], step.h_row_start[i + 1]
+                slot, start = step.h_slots[i], step.h_seq_start[i]
+                if start == 0:
+                    step.state[slot].zero_()          # a slot may have served another request
+                cum = step.state[slot] + torch.cumsum(x[r0:r1].float(), 0)
+                step.state[slot] = cum[-1]
+                count = torch.arange(start + 1, start + 1 + (r1 - r0), device=x.device)[:, None]
+                out[r0:r1] = ((cum / count) @ self.w.t()).to(x.dtype)
+            return out
+
+    register_part("mixer", "running_mean", RunningMean, replace=True)
+
+    class ToyConfig:
+        def __init__(self, d):
+            r = JsonReader(d)
+            self.size, self.inter = r.integer("size"), r.integer("inter")
+            self.layers, self.vocab = r.integer("layers"), r.integer("vocab")
+            self.d = d
+
+        def to_dict(self):
+            return self.d
+
+    def toy_spec(c):
+        rms = lambda n: PartSpec("rmsnorm", {"size": c.size, "eps": 1e-6}, {"weight": n})
+        blocks = tuple(BlockSpec(
+            "prenorm", PartSpec("running_mean", {"size": c.size}, {"w": f"l{i}.mix"}),
+            PartSpec("swiglu", {"hidden_size": c.size, "intermediate_size": c.inter},
+                     {"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}),
+            {"mixer": rms(f"l{i}.n1"), "ffn": rms(f"l{i}.n2")}) for i in range(c.layers))
+        return ModelSpec("ToyStateLM", c.size, c.vocab, 4096,
+                         PartSpec("token_embedding", {"vocab_size": c.vocab, "hidden_size": c.size}, {"weight": "emb"}),
+                         blocks, tuple(LayerCall(i) for i in range(c.layers)), rms("norm"),
+                         PartSpec("linear_head", {"vocab_size": c.vocab, "hidden_size": c.size, "tied": True},
+                                  {"weight": "emb"}))
+
+    register_architecture("ToyStateLM", lambda d, origin: ToyConfig(d), toy_spec, replace=True)
+    cfg = {"architectures": ["ToyStateLM"], "size": 40, "inter": 56, "layers": 2, "vocab": 97}
+    folder = write_random_model(str(tmp_path / "toy"), "ToyStateLM", ToyConfig(cfg), seed=3)
+
+    # the plain version of the toy, whole sequences
+    w = {k: v for k, v in P.read_safetensors(str(tmp_path / "toy" / "model.safetensors")).items()}
+
+    def plain(ids):
+        h = w["emb"][torch.tensor(ids)]
+        for i in range(2):
+            n = P.rmsnorm(h, w[f"l{i}.n1"], 1e-6)
+            mean = torch.cumsum(n, 0) / torch.arange(1, len(ids) + 1, dtype=torch.float64)[:, None]
+            r = h + mean @ w[f"l{i}.mix"].t()
+            m = P.rmsnorm(r, w[f"l{i}.n2"], 1e-6)
+            h = r + P.linear(P.swiglu(P.linear(m, w[f"l{i}.g"]), P.linear(m, w[f"l{i}.u"])), w[f"l{i}.d"])
+        return P.linear(P.rmsnorm(h, w["norm"], 1e-6), w["emb"]).numpy()
+
+    rng = np.random.default_rng(0)
+    reqs = {f"t{i}": rng.integers(0, 97, n).tolist() for i, n in enumerate([30, 51, 9, 44, 27])}
+    want = {k: plain(v) for k, v in reqs.items()}
+    model, _ = load_model(folder, "float32", DEV)
+    assert model.cache_needs() == [] and all(s is not None for s in model.state_needs())
+    for steps in (trace_whole(reqs), trace_portions(reqs, 2), trace_mixed(reqs, 256, seed=5)):
+        runner = ModelRunner(model, model.env, page_size=16, num_pages=16, max_requests=4,
+                             max_batch_tokens=256)
+        rp = Replayer(runner)
+        got = collect(steps, {s["step"]: rp.run_step(s) for s in steps})
+        for k in reqs:
+            assert np.abs(got[k] - want[k]).max() <= 2e-5 * max(1.0, np.abs(want[k]).max())
+        assert runner.cache.free_slots() == 4

@@ -25,18 +25,51 @@ __host__ __device__ inline float tli_uniform(uint32_t seed_lo, uint32_t seed_hi,
 
 __global__ void sample_kernel(const float* __restrict__ logits, int vocab,
                               const float* __restrict__ temperatures,
-                              const uint32_t* __restrict__ seeds, int* __restrict__ out) {
+                              const uint32_t* __restrict__ seeds, const float* __restrict__ top_p,
+                              int* __restrict__ out) {
     __shared__ float best_v[SAMPLE_THREADS / TLI_WAVE];
     __shared__ int best_i[SAMPLE_THREADS / TLI_WAVE];
+    __shared__ float red[16];
     const int row = blockIdx.x;
     const float* l = logits + (size_t)row * vocab;
     const float temp = temperatures ? temperatures[row] : 0.f;
+    const bool draw = temp > 1.0e-6f;
     const uint32_t lo = seeds ? seeds[2 * row] : 0u, hi = seeds ? seeds[2 * row + 1] : 0u;
+
+    // top-p: the smallest logit that is kept.  A token is kept if the weights
+    // exp((l - max)/T) of all tokens strictly above it sum to less than
+    // top_p * total (engine/src/llm_engine.cpp:118-141: tokens are taken in
+    // descending order until the running sum reaches top_p * total).
+    float cutoff = -INFINITY;
+    if (draw && top_p && top_p[row] < 1.0f) {
+        float mx = -INFINITY, mn = INFINITY;
+        for (int t = threadIdx.x; t < vocab; t += blockDim.x) { mx = fmaxf(mx, l[t]); mn = fminf(mn, l[t]); }
+        mx = block_max(mx, red);
+        mn = -block_max(-mn, red);
+        const float inv_t = 1.0f / temp;
+        float total = 0.f;
+        for (int t = threadIdx.x; t < vocab; t += blockDim.x) total += expf((l[t] - mx) * inv_t);
+        total = block_sum(total, red);
+        const float theta = top_p[row] * total;
+        float below = mn - 1.0f, above = mx;       // f(below) >= theta, f(above) = 0 < theta
+        for (int it = 0; it < 64; ++it) {
+            const float mid = below + (above - below) * 0.5f;
+            if (!(mid > below && mid < above)) break;
+            float f = 0.f;
+            for (int t = threadIdx.x; t < vocab; t += blockDim.x)
+                if (l[t] > mid) f += expf((l[t] - mx) * inv_t);
+            f = block_sum(f, red);
+            if (f < theta) above = mid; else below = mid;
+        }
+        cutoff = above;
+    }
+
     float bv = -INFINITY;
     int bi = 0x7fffffff;
     for (int t = threadIdx.x; t < vocab; t += blockDim.x) {
         float s = l[t];
-        if (temp > 1.0e-6f) s += temp * -logf(-logf(tli_uniform(lo, hi, (uint32_t)t)));
+        if (s < cutoff) continue;
+        if (draw) s += temp * -logf(-logf(tli_uniform(lo, hi, (uint32_t)t)));
         if (s > bv || (s == bv && t < bi)) { bv = s; bi = t; }
     }
     for (int off = TLI_WAVE / 2; off > 0; off >>= 1) {
@@ -45,6 +78,7 @@ __global__ void sample_kernel(const float* __restrict__ logits, int vocab,
         if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
     }
     const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE;
+    __syncthreads();
     if (lane == 0) { best_v[wave] = bv; best_i[wave] = bi; }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -54,12 +88,15 @@ __global__ void sample_kernel(const float* __restrict__ logits, int vocab,
     }
 }
 
-// temperatures: float [rows] or null (greedy); seeds: uint32 [rows][2] (low, high word) or null
+// temperatures: float [rows] or null (greedy); seeds: uint32 [rows][2] (low, high word) or null;
+// top_p: float [rows] or null (1 everywhere)
 extern "C" int tli_sample(const float* logits, int rows, int vocab, const float* temperatures,
-                          const uint32_t* seeds, int* out, void* stream) {
+                          const uint32_t* seeds, const float* top_p, int* out, void* stream) {
     if (rows <= 0) return 0;
     if (vocab <= 0) return tli_fail("sample: bad vocabulary size %d", vocab);
-    sample_kernel<<<rows, SAMPLE_THREADS, 0, (hipStream_t)stream>>>(logits, vocab, temperatures, seeds, out);
+    if (temperatures && !seeds) return tli_fail("sample: temperatures need seeds");
+    sample_kernel<<<rows, SAMPLE_THREADS, 0, (hipStream_t)stream>>>(logits, vocab, temperatures, seeds,
+                                                                     top_p, out);
     return tli_check_launch("sample");
 }
 

@@ -171,7 +171,7 @@ class ModelRunner:
         totals = [s + c for s, c in zip(starts, counts)]
         rows, seqs = sum(counts), len(entries)
         wanted = sum(len(e.want) for e in entries)
-        width = _pow2_at_least(max((t + page - 1) // page for t in totals))
+        width = _pow2_at_least(max(max((len(tab) for tab in rc.tables), default=1) for rc in rcs))
         lay = self.inputs.layout(rows, seqs, wanted, width)
         buf = self.inputs.begin()
         row_start = [0]

@@ -1,0 +1,179 @@
+"""The scheduler: which requests run in the next step and with how many tokens.
+
+The policy is the reference's (engine/src/scheduler.cpp:40-121):
+
+1. Decode first.  Every running request, in round-robin order, gets one token
+   while ``max_num_seqs`` and the token budget ``max_num_batched_tokens`` allow.
+   A running request that needs a page when none is free is preempted: all it
+   holds is given back, it goes to the FRONT of the waiting queue and is later
+   computed again from its prompt and everything it has generated.
+2. Then prompts.  Waiting requests, in order, each get at most one portion per
+   step, cut to the budget that is left.  A request is admitted only when the
+   pages for all its current tokens are free (and a state slot); otherwise it
+   goes to the back of the queue.  A prompt that needs more pages than the pool
+   owns is an error.
+3. If nothing could be scheduled while work remains, that is an error.
+
+After the step (engine/src/scheduler.cpp:123-159) a request whose portion
+reached its last token, or that decoded, takes its sampled token; it finishes
+on an end-of-sequence token (unless ``ignore_eos``) or at ``max_tokens``, and
+gives back what it holds.
+"""
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Callable, Deque, List, Optional, Sequence as Seq
+
+from ..cache.manager import CacheFull, CacheManager
+from .sequence import Sequence, Status
+
+
+class SchedulerError(RuntimeError):
+    pass
+
+
+@dataclass
+class SchedulerConfig:
+    max_num_seqs: int = 16
+    max_num_batched_tokens: int = 1024
+
+
+@dataclass
+class ScheduledSequence:
+    sequence: Sequence
+    token_start: int
+    token_count: int
+    is_prefill: bool
+
+    @property
+    def samples(self) -> bool:
+        """Does this item end at the request's last token (so a token is sampled)?"""
+        return (not self.is_prefill) or self.token_start + self.token_count == self.sequence.size
+
+
+@dataclass
+class BatchPlan:
+    sequences: List[ScheduledSequence] = field(default_factory=list)
+    num_tokens: int = 0
+
+
+class Scheduler:
+    def __init__(self, config: SchedulerConfig, cache: CacheManager):
+        if config.max_num_seqs <= 0 or config.max_num_batched_tokens <= 0:
+            raise ValueError("max_num_seqs and max_num_batched_tokens must be positive")
+        self.config = config
+        self.cache = cache
+        self.waiting: Deque[Sequence] = deque()
+        self.running: Deque[Sequence] = deque()
+        self.num_preemptions = 0
+
+    def add(self, sequence: Sequence) -> None:
+        if sequence.size == 0:
+            raise ValueError("A scheduled request must contain at least one token.")
+        self.waiting.append(sequence)
+
+    def is_finished(self) -> bool:
+        return not self.waiting and not self.running
+
+    # ---- pages ------------------------------------------------------------
+    def _preempt(self, seq: Sequence) -> None:
+        if seq.admitted:
+            self.cache.release(seq.request_id)
+            seq.admitted = False
+        seq.status = Status.WAITING
+        seq.num_cached_tokens = 0
+        seq.num_scheduled_tokens = 0
+        seq.preemptions += 1
+        self.num_preemptions += 1
+        self.waiting.appendleft(seq)
+
+    def _pages_for_whole_pool(self, size: int) -> bool:
+        page = self.cache.page_size
+        return (size + page - 1) // page <= self.cache.num_pages
+
+    def _admit(self, seq: Sequence) -> bool:
+        if self.cache.free_slots() == 0:
+            return False
+        self.cache.admit(seq.request_id)
+        if not self.cache.can_reserve(seq.request_id, seq.size):
+            self.cache.release(seq.request_id)
+            return False
+        self.cache.reserve(seq.request_id, seq.size)
+        seq.admitted = True
+        seq.num_cached_tokens = 0
+        return True
+
+    # ---- one step's plan -----------------------------------------------------
+    def schedule(self) -> BatchPlan:
+        plan = BatchPlan()
+        budget = self.config.max_num_batched_tokens
+        tokens = 0
+        for _ in range(len(self.running)):
+            if len(plan.sequences) >= self.config.max_num_seqs or tokens >= budget:
+                break
+            seq = self.running.popleft()
+            if not self.cache.can_reserve(seq.request_id, seq.size):
+                self._preempt(seq)
+                continue
+            self.cache.reserve(seq.request_id, seq.size)
+            seq.num_scheduled_tokens = 1
+            plan.sequences.append(ScheduledSequence(seq, seq.size - 1, 1, False))
+            self.running.append(seq)
+            tokens += 1
+
+        for _ in range(len(self.waiting)):
+            if len(plan.sequences) >= self.config.max_num_seqs or tokens >= budget:
+                break
+            seq = self.waiting.popleft()
+            if not seq.admitted and not self._admit(seq):
+                if not self._pages_for_whole_pool(seq.size):
+                    raise SchedulerError("The prompt requires more KV blocks than the engine owns.")
+                self.waiting.append(seq)
+                continue
+            remaining = seq.size - seq.num_cached_tokens
+            if remaining <= 0:
+                raise SchedulerError("A waiting prompt has no uncached tokens to schedule.")
+            count = min(remaining, budget - tokens)
+            seq.num_scheduled_tokens = count
+            plan.sequences.append(ScheduledSequence(seq, seq.num_cached_tokens, count, True))
+            tokens += count
+            if seq.num_cached_tokens + count == seq.size:
+                seq.status = Status.RUNNING
+                self.running.append(seq)
+            else:
+                self.waiting.append(seq)
+        plan.num_tokens = tokens
+        if not plan.sequences and not self.is_finished():
+            raise SchedulerError("The scheduler could not make progress with the available KV blocks.")
+        return plan
+
+    # ---- after the step --------------------------------------------------------
+    def postprocess(self, plan: BatchPlan, sampled: Seq[Optional[int]],
+                    is_eos: Callable[[int], bool]) -> List[Sequence]:
+        """``sampled[i]`` is the token of plan item i, None where nothing was
+        sampled.  Returns the requests that finished."""
+        if len(sampled) != len(plan.sequences):
+            raise SchedulerError("The model runner returned the wrong number of sampled tokens.")
+        finished = []
+        for item, token in zip(plan.sequences, sampled):
+            seq = item.sequence
+            seq.num_cached_tokens += seq.num_scheduled_tokens
+            seq.num_scheduled_tokens = 0
+            if item.is_prefill and seq.num_cached_tokens < seq.size:
+                continue
+            if token is None or token < 0:
+                raise SchedulerError("The model runner did not return a token for a completed step.")
+            seq.token_ids.append(int(token))
+            seq.num_sampled += 1
+            stopped = (not seq.sampling.ignore_eos) and is_eos(int(token))
+            if stopped or seq.completion_size >= seq.sampling.max_tokens:
+                seq.status = Status.FINISHED
+                self.cache.release(seq.request_id)
+                seq.admitted = False
+                try:
+                    self.running.remove(seq)
+                except ValueError:
+                    pass
+                finished.append(seq)
+        return finished

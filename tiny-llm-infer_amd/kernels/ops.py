@@ -53,7 +53,7 @@ def load_library():
         "tli_qkv_to_cache": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I, I, I, I, P],
         "tli_attention_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
         "tli_gemm_plain": [P, P, P, I, I, I, I, I, I, P],
-        "tli_sample": [P, I, I, P, P, P, P],
+        "tli_sample": [P, I, I, P, P, P, P, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -224,9 +224,9 @@ class HipOps:
         return out
 
     def sample(self, logits: torch.Tensor, temperatures: Optional[torch.Tensor] = None,
-               seeds: Optional[torch.Tensor] = None) -> torch.Tensor:
+               seeds: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Token ids int32 [rows].  ``temperatures`` float32 [rows] (None: greedy);
-        ``seeds`` int64 [rows], one draw seed per row."""
+        ``seeds`` int64 [rows], one draw seed per row; ``top_p`` float32 [rows] or None."""
         rows, vocab = logits.shape
         self._want(logits, "logits", torch.float32)
         if temperatures is not None:
@@ -234,9 +234,12 @@ class HipOps:
             if seeds is None:
                 raise KernelError("sampling with a temperature needs seeds")
             self._want(seeds, "seeds", torch.int64, (rows,))
+        if top_p is not None:
+            self._want(top_p, "top_p", torch.float32, (rows,))
         out = torch.empty((rows,), dtype=torch.int32, device=self.device)
         self._call(self.lib.tli_sample, logits.data_ptr(), rows, vocab, _ptr(temperatures),
-                   _ptr(seeds) if temperatures is not None else None, out.data_ptr(), self._stream())
+                   _ptr(seeds) if temperatures is not None else None,
+                   _ptr(top_p) if temperatures is not None else None, out.data_ptr(), self._stream())
         return out
 
 
