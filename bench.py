@@ -1,0 +1,170 @@
+"""Serving benchmark on one MI355X: decode tokens a second of a Qwen3-8B-shaped
+model with random bfloat16 weights (BASELINE.json configs[2]), plus the prefill
+of one 2,048-token prompt and decode at batch 1 and 64.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+
+A step is one decode step of the engine (schedule, run the batch, sample,
+post-process).  One JSON line is printed.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12            # bytes/s, MI355X HBM3E
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_size=4096,
+                intermediate_size=12288, num_hidden_layers=36, num_attention_heads=32,
+                num_key_value_heads=8, head_dim=128, vocab_size=151936, max_position_embeddings=40960,
+                rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False)
+
+
+def weight_bytes(cfg, layers, elem=2):
+    H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    Q = cfg["num_attention_heads"] * cfg["head_dim"]
+    KV = cfg["num_key_value_heads"] * cfg["head_dim"]
+    per_layer = (Q + 2 * KV) * H + H * Q + 3 * I * H
+    return (layers * per_layer + V * H) * elem       # what a decode step reads (embedding rows aside)
+
+
+def kv_bytes_per_token(cfg, layers, elem=2):
+    return 2 * layers * cfg["num_key_value_heads"] * cfg["head_dim"] * elem
+
+
+def step_flops(cfg, layers, rows, ctx_sum, wanted):
+    """2*rows*params for the matrices, 4*heads*head_dim per (row, key) for attention."""
+    H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    Q = cfg["num_attention_heads"] * cfg["head_dim"]
+    KV = cfg["num_key_value_heads"] * cfg["head_dim"]
+    per_layer = (Q + 2 * KV) * H + H * Q + 3 * I * H
+    return 2.0 * rows * layers * per_layer + 4.0 * Q * ctx_sum * layers + 2.0 * wanted * V * H
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0: all)")
+    ap.add_argument("--prompt-len", type=int, default=128)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py runs on one GPU only; --gpus {args.gpus} is not supported (single-GPU engine)")
+        return 2
+
+    import random
+
+    import torch
+
+    from tiny_llm_infer_amd.config import Qwen3Config
+    from tiny_llm_infer_amd.engine.llm_engine import LLMEngine
+    from tiny_llm_infer_amd.engine.loading import random_model
+    from tiny_llm_infer_amd.sampling.params import SamplingParams
+
+    cfg_json = dict(QWEN3_8B)
+    full_layers = cfg_json["num_hidden_layers"]
+    layers = args.layers or full_layers
+    cfg_json["num_hidden_layers"] = layers
+    cfg = Qwen3Config.from_dict(cfg_json)
+    elem = 2 if args.dtype == "bfloat16" else 4
+    dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
+    t0 = time.time()
+    model = random_model("Qwen3ForCausalLM", cfg, args.seed, args.dtype, "cuda:0", args.context)
+    torch.cuda.synchronize()
+    print(f"[bench] model with {layers} layers on the device in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+
+    page = 16
+    max_batch = max(64, args.batch)
+    budget = max(args.prefill_tokens, 2048)
+    pages = max_batch * ((args.prompt_len + args.steps + args.warmup + 64 + page - 1) // page) \
+        + (args.prefill_tokens + page - 1) // page + 8
+    engine = LLMEngine.from_model(model, max_model_len=args.context, page_size=page, num_kv_blocks=pages,
+                                  max_num_seqs=max_batch, max_num_batched_tokens=budget)
+    rng = random.Random(args.seed)
+    vocab = cfg.vocab_size
+
+    def decode_run(batch, steps, warmup):
+        """Prefill ``batch`` prompts, then time ``steps`` decode steps."""
+        params = SamplingParams(max_tokens=steps + warmup + 1, temperature=0.0, ignore_eos=True)
+        for _ in range(batch):
+            engine.add_request([rng.randrange(vocab) for _ in range(args.prompt_len)], params)
+        while engine.scheduler.waiting:
+            engine.step()
+        for _ in range(warmup):
+            engine.step()
+        ctx0 = sum(s.size for s in engine.scheduler.running)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            engine.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        ctx1 = sum(s.size for s in engine.scheduler.running)
+        while not engine.is_finished():
+            engine.step()
+        return dt, (ctx0 + ctx1) / 2.0
+
+    dt, ctx_tokens = decode_run(args.batch, args.steps, args.warmup)
+    ms_step = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    step_bytes = weight_bytes(cfg_json, layers, elem) + ctx_tokens * kv_bytes_per_token(cfg_json, layers, elem)
+    achieved = step_bytes / (dt / args.steps)
+
+    # prefill of one prompt in one step
+    def prefill_once():
+        engine.add_request([rng.randrange(vocab) for _ in range(args.prefill_tokens)],
+                           SamplingParams(max_tokens=1, ignore_eos=True))
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        engine.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        assert engine.is_finished()
+        return dt
+    prefill_once()
+    pre = min(prefill_once() for _ in range(3))
+    T = args.prefill_tokens
+    pre_flops = step_flops(cfg_json, layers, T, T * (T + 1) / 2.0, 1)
+
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            d, _ = decode_run(b, min(args.steps, 32), 4)
+            points[f"decode_b{b}"] = round(b * min(args.steps, 32) / d, 2)
+
+    out = {
+        "metric": "decode tok/s @ batch 8 (Qwen3-8B shape, bf16, random weights)",
+        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": dkey, "data": "synthetic",
+        "config": {"model": "Qwen3-8B shape, random weights", "global_batch": args.batch,
+                   "seq_len": args.context, "parallelism": "single GPU", "layers": layers,
+                   "layers_of_config": full_layers, "hidden_size": cfg.hidden_size,
+                   "intermediate_size": cfg.intermediate_size, "heads": cfg.num_attention_heads,
+                   "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                   "vocab_size": cfg.vocab_size, "prompt_len": args.prompt_len,
+                   "page_size": page, "prefill_tokens": T},
+        "prefill": {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
+                    "frac": round(pre_flops / pre / MFMA_PEAK[dkey], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4)},
+        "points": points,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

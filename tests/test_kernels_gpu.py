@@ -105,6 +105,35 @@ def test_linear(ops, dtype, mnk):
           scale=float(want.abs().max()) * (1.0 if dtype == torch.float32 else 0.05))
 
 
+SKINNY = [(1, 4096, 4096), (8, 6144, 4096), (8, 4096, 12288), (16, 301, 80), (17, 1000, 264),
+          (33, 24576, 512), (64, 130, 4096), (5, 151936, 128), (48, 70, 8)]
+
+
+@pytest.mark.parametrize("mnk", SKINNY)
+@pytest.mark.parametrize("out", [torch.bfloat16, torch.float32])
+def test_skinny_linear_against_plain_kernel_and_reference(ops, mnk, out):
+    """The weight-streaming MFMA kernel for up to 64 rows, beside the plain tiled kernel."""
+    M, N, K = mnk
+    x, w = rnd((M, K), torch.bfloat16, 7), rnd((N, K), torch.bfloat16, 8, 0.05)
+    xd, wd = x.to(DEV), w.to(DEV)
+    got = ops.linear(xd, wd, out_dtype=out)
+    plain = ops.linear_plain(xd, wd, out_dtype=out)
+    want = x.double() @ w.double().t()
+    scale = float(want.abs().max())
+    # float32 out: only the order of the float32 additions differs
+    bound = 2e-5 * scale * (K ** 0.5) / 8 + 1e-6 if out == torch.float32 else 1.2e-2 * scale
+    assert float((got.double().cpu() - want).abs().max()) <= bound
+    assert float((plain.double().cpu() - want).abs().max()) <= bound
+
+
+def test_library_linear_for_many_rows(ops):
+    x, w = rnd((300, 264), torch.bfloat16, 1), rnd((130, 264), torch.bfloat16, 2, 0.05)
+    close(ops.linear(x.to(DEV), w.to(DEV)), x.double() @ w.double().t(), torch.bfloat16, "library product")
+    y32 = ops.linear(x.to(DEV), w.to(DEV), out_dtype=torch.float32)       # float32 out, 64 rows at a time
+    assert y32.dtype == torch.float32
+    close(y32, x.double() @ w.double().t(), torch.float32, "float32 logits for many rows", scale=5.0)
+
+
 def test_linear_rows_do_not_depend_on_the_batch(ops):
     """float32: a row's product is bit-identical whatever else is in the batch."""
     x, w = rnd((70, 100), torch.float32, 9), rnd((130, 100), torch.float32, 10)

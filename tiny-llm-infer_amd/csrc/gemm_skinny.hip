@@ -1,0 +1,151 @@
+// Matrix product for few rows (decode): y[M,N] = x[M,K] . W[N,K]^T, M <= 64,
+// bfloat16 inputs, float32 accumulation on the matrix cores, bfloat16 or
+// float32 output.  The work is streaming W from HBM once; everything is laid
+// out so that each lane's global loads are 64 contiguous bytes of one W row and
+// land directly in the MFMA operand registers (no LDS staging of W).
+//
+// The reference multiplies a single row with a hand GEMV and more rows with a
+// library call (kernels/src/matmul_kernel_cuda.cu:72-91); this kernel covers
+// both for up to 64 rows.
+//
+// v_mfma_f32_16x16x32_bf16 computes D[16x16] += A[16x32] B[32x16]; lane l holds
+// A[l%16][(l/16)*8 .. +8], B[(l/16)*8 .. +8][l%16] and D[(l/16)*4 .. +4][l%16].
+// Here A is a tile of W (16 output columns n), B is x^T (16 rows m), so a lane
+// ends with y[m = l%16][n = (l/16)*4 .. +4].  The 32 k-slots of one MFMA may be
+// any 32 values of k as long as A and B agree: lane group c = l/16 takes the 32
+// consecutive k  [kb + 32c, kb + 32c + 32)  of a 128-wide step, 8 per MFMA.
+//
+// A workgroup owns 16*RT output columns; its waves take the 128-wide k steps in
+// turn and their partial sums are added through LDS in wave order, so the
+// result does not depend on the launch.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+union Pack16 {
+    uint4 u;
+    bf16x8 v;
+};
+
+__device__ __forceinline__ uint4 load16_or_zero(const bf16_t* p, bool ok) {
+    return ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
+}
+
+template <int RT, int MT, int WAVES, typename TO>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* __restrict__ y,
+                   int M, int N, int K) {
+    __shared__ float red[WAVES][RT * MT][64][4];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int r = lane % 16, c = lane / 16;
+    const int n_base = blockIdx.x * (16 * RT);
+
+    f32x4 acc[RT][MT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[t][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    const bf16_t* w_row[RT];
+    bool w_ok[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        const int n = n_base + t * 16 + r;
+        w_ok[t] = n < N;
+        w_row[t] = w + (size_t)(w_ok[t] ? n : 0) * K;
+    }
+    const bf16_t* x_row[MT];
+    bool x_ok[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int row = m * 16 + r;
+        x_ok[m] = row < M;
+        x_row[m] = x + (size_t)(x_ok[m] ? row : 0) * K;
+    }
+
+    for (int kb = wave * 128; kb < K; kb += WAVES * 128) {
+        const int k = kb + c * 32;
+        Pack16 a[RT][4], b[MT][4];
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                a[t][j].u = load16_or_zero(w_row[t] + k + j * 8, w_ok[t] && (k + j * 8 < K));
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                b[m][j].u = load16_or_zero(x_row[m] + k + j * 8, x_ok[m] && (k + j * 8 < K));
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int t = 0; t < RT; ++t)
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+                    acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][j].v, b[m][j].v, acc[t][m], 0, 0, 0);
+    }
+
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave][t * MT + m][lane][i] = acc[t][m][i];
+    __syncthreads();
+    // tiles are shared out over the waves; each sums the partials in wave order
+    for (int tile = wave; tile < RT * MT; tile += WAVES) {
+        const int t = tile / MT, m = tile % MT;
+        float s[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int wv = 0; wv < WAVES; ++wv)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[i] += red[wv][tile][lane][i];
+        const int row = m * 16 + r;
+        const int n0 = n_base + t * 16 + c * 4;
+        if (row < M) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (n0 + i < N) from_f32(y + (size_t)row * N + n0 + i, s[i]);
+        }
+    }
+}
+
+template <int RT, int MT, int WAVES>
+static int launch_skinny(const bf16_t* x, const bf16_t* w, void* y, int M, int N, int K, int y_dtype,
+                         hipStream_t s) {
+    const int blocks = (N + 16 * RT - 1) / (16 * RT);
+    if (y_dtype == TLI_BF16)
+        gemm_skinny_kernel<RT, MT, WAVES, bf16_t><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
+    else
+        gemm_skinny_kernel<RT, MT, WAVES, float><<<blocks, WAVES * 64, 0, s>>>(x, w, (float*)y, M, N, K);
+    return tli_check_launch("gemm_skinny");
+}
+
+template <int MT>
+static int pick_skinny(const bf16_t* x, const bf16_t* w, void* y, int M, int N, int K, int y_dtype,
+                       hipStream_t s) {
+    // narrow outputs: one 16-column tile per workgroup and 8 waves over k, so that
+    // even N = 4096 gives 256 workgroups; wide outputs share x over more columns
+    const long tiles = (N + 15) / 16;
+    if (tiles >= 4096 && MT <= 2) return launch_skinny<4, MT, 4>(x, w, y, M, N, K, y_dtype, s);
+    if (tiles >= 1024) return launch_skinny<2, MT, 8>(x, w, y, M, N, K, y_dtype, s);
+    return launch_skinny<1, MT, 8>(x, w, y, M, N, K, y_dtype, s);
+}
+
+extern "C" int tli_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K,
+                                    int y_dtype, void* stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 64) return tli_fail("gemm_skinny: %d rows, at most 64", M);
+    if (K <= 0 || K % 8) return tli_fail("gemm_skinny: K = %d must be a positive multiple of 8", K);
+    if (y_dtype != TLI_BF16 && y_dtype != TLI_F32) return tli_fail("gemm_skinny: bad output dtype %d", y_dtype);
+    if (((uintptr_t)x | (uintptr_t)w) & 15) return tli_fail("gemm_skinny: operands must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    const bf16_t* xp = (const bf16_t*)x;
+    const bf16_t* wp = (const bf16_t*)w;
+    switch ((M + 15) / 16) {
+        case 1: return pick_skinny<1>(xp, wp, y, M, N, K, y_dtype, s);
+        case 2: return pick_skinny<2>(xp, wp, y, M, N, K, y_dtype, s);
+        case 3: return pick_skinny<3>(xp, wp, y, M, N, K, y_dtype, s);
+        default: return pick_skinny<4>(xp, wp, y, M, N, K, y_dtype, s);
+    }
+}

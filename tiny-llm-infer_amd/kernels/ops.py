@@ -53,6 +53,7 @@ def load_library():
         "tli_qkv_to_cache": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I, I, I, I, P],
         "tli_attention_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
         "tli_gemm_plain": [P, P, P, I, I, I, I, I, I, P],
+        "tli_gemm_skinny_bf16": [P, P, P, I, I, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P],
     }
     for name, args in sigs.items():
@@ -72,6 +73,7 @@ def _ptr(t: Optional[torch.Tensor]):
 class HipOps:
     name = "hip-gfx950"
     MAX_HEAD_DIM = 512
+    SKINNY_ROWS = 64
 
     def __init__(self, device):
         self.device = torch.device(device)
@@ -150,6 +152,33 @@ class HipOps:
         self._want(w, "linear matrix")
         if x.dtype != w.dtype:
             raise KernelError(f"linear: input is {x.dtype}, the matrix {w.dtype}")
+        out_dtype = out_dtype or x.dtype
+        y = torch.empty((M, N), dtype=out_dtype, device=self.device)
+        if M == 0:
+            return y
+        if x.dtype == torch.bfloat16 and K % 8 == 0:
+            if M <= self.SKINNY_ROWS or out_dtype == torch.float32:
+                # few rows (decode), or float32 logits: the weight-streaming MFMA kernel,
+                # 64 rows at a time
+                for m0 in range(0, M, self.SKINNY_ROWS):
+                    m1 = min(M, m0 + self.SKINNY_ROWS)
+                    self._call(self.lib.tli_gemm_skinny_bf16, x[m0:m1].data_ptr(), w.data_ptr(),
+                               y[m0:m1].data_ptr(), m1 - m0, N, K, _dtype_code(out_dtype), self._stream())
+                return y
+            # many rows (prefill): the library's matrix product, as the reference
+            # uses its library for more than one row (kernels/src/matmul_kernel_cuda.cu:84-91)
+            torch.matmul(x, w.t(), out=y)
+            return y
+        self._call(self.lib.tli_gemm_plain, x.data_ptr(), w.data_ptr(), y.data_ptr(), M, N, K,
+                   _dtype_code(x.dtype), _dtype_code(w.dtype), _dtype_code(out_dtype), self._stream())
+        return y
+
+    def linear_plain(self, x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
+        """The plain tiled kernel for any sizes and dtypes: the reference beside the tuned ones."""
+        M, K = x.shape
+        N = w.shape[0]
+        self._want(x, "linear input")
+        self._want(w, "linear matrix", x.dtype, (N, K))
         out_dtype = out_dtype or x.dtype
         y = torch.empty((M, N), dtype=out_dtype, device=self.device)
         self._call(self.lib.tli_gemm_plain, x.data_ptr(), w.data_ptr(), y.data_ptr(), M, N, K,
