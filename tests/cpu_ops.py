@@ -74,7 +74,7 @@ class CpuOps:
             assert (pages >= 0).all(), "a row writes to a page that is not held"
             slots = pos % page
             cache.k[pages, :, slots] = k.to(cache.k.dtype)
-            cache.v[pages, :, slots] = v.to(cache.v.dtype)
+            cache.v[pages, :, :, slots] = v.to(cache.v.dtype)        # values are kept transposed
         return q.reshape(T, qd).to(qkv.dtype)
 
     def paged_attention(self, q, step, cache, heads, kv_heads, head_dim, scale, window):
@@ -93,7 +93,7 @@ class CpuOps:
             pages = tables[seq_l[r], idx // page].long()
             assert (pages >= 0).all(), "a row reads a page that is not held"
             kk = cache.k[pages, :, idx % page].to(torch.float32)     # [n, kv, d]
-            vv = cache.v[pages, :, idx % page].to(torch.float32)
+            vv = cache.v[pages, :, :, idx % page].to(torch.float32)
             for h in range(heads):
                 s = (kk[:, h // mul] @ qf[r, h]) * scale
                 w = torch.softmax(s, dim=0)

@@ -170,7 +170,7 @@ def make_step(seq_lens, new_counts, page, num_pages, seed, kv_heads, head_dim, d
         seq += [i] * c
         row_start.append(len(pos))
     k = torch.zeros((1, num_pages, kv_heads, page, head_dim), dtype=dtype, device=DEV)
-    v = torch.zeros_like(k)
+    v = torch.zeros((1, num_pages, kv_heads, head_dim, page), dtype=dtype, device=DEV)
     # garbage in every slot: pages not held and slots not yet written must never be read
     k.normal_(0, 50.0)
     v.normal_(0, 50.0)
@@ -196,7 +196,7 @@ def fill_cache(step, tables, seq_lens, kv_heads, head_dim, dtype, seed, std=1.0)
         for t in range(n):
             p = int(tables[i, t // page])
             step.cache.k[p, :, t % page] = kk[t].to(DEV)
-            step.cache.v[p, :, t % page] = vv[t].to(DEV)
+            step.cache.v[p, :, :, t % page] = vv[t].to(DEV)
         ks.append(kk)
         vs.append(vv)
     return ks, vs
@@ -225,12 +225,31 @@ ATT_CASES = [
     (8, 8, 64, 16, [130, 257], [130, 2], 19),
     (6, 3, 256, 16, [90], [7], 64),
     (32, 8, 128, 16, [513], [2], None),
+    # one row per sequence (decode), long enough for the keys to be split over workgroups
+    (32, 8, 128, 16, [1500, 40, 129, 1, 640], [1, 1, 1, 1, 1], None),
+    (8, 8, 64, 16, [130, 257], [1, 1], 19),
+    (5, 1, 48, 32, [300, 64], [1, 1], 100),
+    (32, 1, 32, 8, [70, 3], [1, 1], None),        # 32 heads on one kv head: two head tiles
+    (32, 1, 32, 4, [70], [9], None),
+    (6, 2, 80, 16, [200, 31], [200, 31], None),   # 3 heads a group: columns do not fill the tile
+    (16, 2, 112, 64, [333], [100], 150),
 ]
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dtype", DTYPES + ["bfloat16-plain"])
 @pytest.mark.parametrize("case", ATT_CASES)
 def test_paged_attention(ops, dtype, case):
+    """float32: the plain kernel.  bfloat16: the MFMA kernels (decode when every
+    sequence brings one row, prefill otherwise), and the plain kernel beside them."""
+    ops.force_plain = dtype == "bfloat16-plain"
+    dtype = torch.bfloat16 if isinstance(dtype, str) else dtype
+    try:
+        _paged_attention_case(ops, dtype, case)
+    finally:
+        ops.force_plain = False
+
+
+def _paged_attention_case(ops, dtype, case):
     heads, kv_heads, hd, page, seq_lens, new_counts, window = case
     num_pages = sum((n + page - 1) // page for n in seq_lens) + 5
     step, tables, pos, seq = make_step(seq_lens, new_counts, page, num_pages, 3, kv_heads, hd, dtype, window)
@@ -329,7 +348,7 @@ def test_qkv_to_cache(ops, dtype, case):
     for r in range(T):
         p, slot = int(tables[seq[r], pos[r] // page]), pos[r] % page
         close(step.cache.k[p, :, slot], kk[r], dtype, "k in cache")
-        assert torch.equal(step.cache.v[p, :, slot].cpu(), qkv[r, qd + kd:].reshape(kv_heads, hd))
+        assert torch.equal(step.cache.v[p, :, :, slot].cpu(), qkv[r, qd + kd:].reshape(kv_heads, hd))
         written[p, slot] = True
     # nothing else in the cache was touched
     untouched = ~written[:, None, :, None].expand_as(before_k.cpu())

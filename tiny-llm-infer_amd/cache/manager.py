@@ -10,8 +10,10 @@ window of all tokens still to come; every group gives all of a request's pages
 back when the request ends.  (The reference has one group and no window:
 model/src/qwen3_kv_cache.cpp:14-44, engine/src/block_manager.cpp.)
 
-Page layout on the device: ``[cache layer in group, page, kv head, slot, head_dim]``
-so that the slots of one head in one page are contiguous.  The block table of a
+Page layout on the device: keys ``[cache layer in group, page, kv head, slot,
+head_dim]``, values ``[cache layer in group, page, kv head, head_dim, slot]``, so
+that one head's part of a page is contiguous and each matrix-core operand is
+contiguous along the index it is contracted over.  The block table of a
 request maps ``position // page_size`` to a page id, -1 where no page is held.
 """
 from __future__ import annotations

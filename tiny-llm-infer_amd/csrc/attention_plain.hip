@@ -68,8 +68,8 @@ __global__ void attention_plain_kernel(
                 const int page = table[tt / page_size];
                 if (page < 0 || page >= num_pages) continue;
                 const T* vp = v_cache + (size_t)page * page_stride +
-                              ((size_t)g * page_size + (tt % page_size)) * head_dim;
-                a += p_s[j] * to_f32(vp[d]);
+                              (size_t)g * page_size * head_dim + (tt % page_size);
+                a += p_s[j] * to_f32(vp[(size_t)d * page_size]);
             }
             if (half == 0) acc0 = a; else acc1 = a;
         }

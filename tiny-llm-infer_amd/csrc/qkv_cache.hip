@@ -5,7 +5,8 @@
 //   q, k:  x <- w * x / sqrt(mean(x^2) + eps)  over the head      (if a norm is given)
 //          (x_i, x_{i+rd/2}) <- (x_i cos - x_{i+rd/2} sin, x_i sin + x_{i+rd/2} cos), i < rd/2
 //                                                 (kernels/src/rope_kernel_cpu.cpp:156-179)
-//   k, v -> cache[page = table[seq][pos / page_size]][kv head][pos % page_size][:]
+//   k -> keys[page = table[seq][pos / page_size]][kv head][pos % page_size][:]
+//   v -> values[page][kv head][:][pos % page_size]      (values are kept transposed)
 // q goes to its own [rows, heads*head_dim] buffer.  The cache layout differs from
 // the reference's [page][slot][kv_dim] (kernels/src/paged_attention_cuda.cu:58-67):
 // here the slots of one head in one page are contiguous.
@@ -32,13 +33,14 @@ __global__ void qkv_to_cache_kernel(
     const T* src_row = qkv + (size_t)row * stride;
 
     // where this row's keys and values go
-    size_t cache_base = 0;
+    size_t cache_base = 0, v_base = 0;
     bool can_write = false;
     if (write_cache) {
         const int seq = seq_of_row[row];
         const int page = tables[(size_t)seq * table_width + pos / page_size];
         can_write = page >= 0 && page < num_pages;
         cache_base = ((size_t)page * kv_heads * page_size + (size_t)(pos % page_size)) * head_dim;
+        v_base = (size_t)page * kv_heads * head_dim * page_size + (size_t)(pos % page_size);
     }
     const int half = rotary_dim / 2;
     const float* cos_row = nullptr;
@@ -90,7 +92,7 @@ __global__ void qkv_to_cache_kernel(
         const T* vsrc = src_row + q_dim + kv_dim;
         for (int i = threadIdx.x; i < kv_dim; i += blockDim.x) {
             const int g = i / head_dim, d = i - g * head_dim;
-            v_cache[cache_base + (size_t)g * page_size * head_dim + d] = vsrc[i];
+            v_cache[v_base + ((size_t)g * head_dim + d) * page_size] = vsrc[i];
         }
     }
 }

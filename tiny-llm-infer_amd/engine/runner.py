@@ -106,9 +106,11 @@ class ModelRunner:
         self.cache = CacheManager(model.cache_needs(), page_size, num_pages, max_requests)
         self.group_tensors = []
         for g in self.cache.groups:
-            shape = (len(g.cache_layers), num_pages, g.need.num_kv_heads, page_size, g.need.head_dim)
-            k = torch.zeros(shape, dtype=env.dtype, device=env.device)
-            v = torch.zeros(shape, dtype=env.dtype, device=env.device)
+            n, heads, hd = len(g.cache_layers), g.need.num_kv_heads, g.need.head_dim
+            # keys [.., slot, head_dim]; values transposed [.., head_dim, slot]: both are
+            # then contiguous along the index the matrix cores contract over
+            k = torch.zeros((n, num_pages, heads, page_size, hd), dtype=env.dtype, device=env.device)
+            v = torch.zeros((n, num_pages, heads, hd, page_size), dtype=env.dtype, device=env.device)
             self.group_tensors.append((k, v))
         self.states: List[Optional[torch.Tensor]] = []
         for need in model.state_needs():

@@ -54,6 +54,8 @@ def load_library():
         "tli_attention_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
         "tli_gemm_plain": [P, P, P, I, I, I, I, I, I, P],
         "tli_gemm_skinny_bf16": [P, P, P, I, I, I, I, P],
+        "tli_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
+        "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P],
     }
     for name, args in sigs.items():
@@ -74,6 +76,7 @@ class HipOps:
     name = "hip-gfx950"
     MAX_HEAD_DIM = 512
     SKINNY_ROWS = 64
+    DECODE_WORKGROUPS = 512      # aim of the decode attention's key splitting
 
     def __init__(self, device):
         self.device = torch.device(device)
@@ -82,6 +85,7 @@ class HipOps:
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible to torch; this engine has no CPU path")
         self.lib = load_library()
+        self.force_plain = False     # tests: run the plain attention kernel for bfloat16 too
 
     # ---- helpers ----------------------------------------------------------
     def _stream(self):
@@ -231,9 +235,8 @@ class HipOps:
 
     def _check_cache(self, kc, vc, g, kv_heads, head_dim, dtype, step):
         pages = kc.shape[0]
-        want = (pages, kv_heads, g.page_size, head_dim)
-        for t, what in ((kc, "key cache"), (vc, "value cache")):
-            self._want(t, what, dtype, want)
+        self._want(kc, "key cache", dtype, (pages, kv_heads, g.page_size, head_dim))
+        self._want(vc, "value cache", dtype, (pages, kv_heads, head_dim, g.page_size))
         self._want(g.tables, "block tables", torch.int32, (step.num_seqs, g.table_width))
         if (step.max_seq_len + g.page_size - 1) // g.page_size > g.table_width:
             raise KernelError("a block table is narrower than its sequence needs")
@@ -246,10 +249,37 @@ class HipOps:
         kc, vc, g = cache.k, cache.v, cache.group
         self._check_cache(kc, vc, g, kv_heads, head_dim, q.dtype, step)
         out = torch.empty_like(q)
+        if q.dtype == torch.bfloat16 and head_dim <= 256 and g.page_size >= 4 and not self.force_plain:
+            if step.max_rows_per_seq == 1:
+                return self._attention_decode(q, out, step, kc, vc, g, heads, kv_heads, head_dim, scale, window)
+            self._call(self.lib.tli_attention_prefill_bf16, q.data_ptr(), out.data_ptr(), kc.data_ptr(),
+                       vc.data_ptr(), step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs,
+                       T, g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], heads, kv_heads,
+                       head_dim, float(scale), int(window or 0), self._stream())
+            return out
         self._call(self.lib.tli_attention_plain, q.data_ptr(), out.data_ptr(), kc.data_ptr(),
                    vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
                    g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], T, heads, kv_heads,
                    head_dim, float(scale), int(window or 0), _dtype_code(q.dtype), self._stream())
+        return out
+
+    def _attention_decode(self, q, out, step, kc, vc, g, heads, kv_heads, head_dim, scale, window):
+        """One row per sequence.  The keys are split over workgroups when the
+        batch alone would leave most of the 256 compute units idle."""
+        T = step.num_rows
+        reach = step.max_seq_len if not window else min(step.max_seq_len, window + 32)
+        groups = T * kv_heads * ((heads // kv_heads + 15) // 16)
+        splits = max(1, min((self.DECODE_WORKGROUPS + groups - 1) // groups, (reach + 127) // 128, 64))
+        per_split = ((reach + splits - 1) // splits + 127) // 128 * 128
+        splits = (reach + per_split - 1) // per_split
+        partial = None
+        if splits > 1:
+            partial = torch.empty((T * heads * splits * (head_dim + 2),), dtype=torch.float32,
+                                  device=self.device)
+        self._call(self.lib.tli_attention_decode_bf16, q.data_ptr(), out.data_ptr(), _ptr(partial),
+                   kc.data_ptr(), vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
+                   g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], T, heads, kv_heads,
+                   head_dim, float(scale), int(window or 0), splits, per_split, self._stream())
         return out
 
     def sample(self, logits: torch.Tensor, temperatures: Optional[torch.Tensor] = None,

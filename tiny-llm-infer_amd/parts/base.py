@@ -37,7 +37,7 @@ class BuildEnv:
 class GroupView:
     """One cache group as a step sees it."""
     k: torch.Tensor               # [layers in group, pages, kv heads, page_size, head_dim]
-    v: torch.Tensor
+    v: torch.Tensor               # [layers in group, pages, kv heads, head_dim, page_size]
     tables: torch.Tensor          # int32 [sequences in step, table width], -1 where no page
     table_width: int
     page_size: int
