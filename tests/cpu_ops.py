@@ -33,6 +33,7 @@ class CpuOps:
         return (weight * x * scale).to(out_dtype)
 
     def linear(self, x, w, out_dtype=None):
+        w = getattr(w, "w", w)
         y = x.to(torch.float32) @ w.to(torch.float32).t()
         return y.to(out_dtype or x.dtype)
 

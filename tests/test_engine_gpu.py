@@ -136,3 +136,45 @@ def test_the_library_is_needed():
     from tiny_llm_infer_amd.kernels.ops import HipOps, KernelError
     with pytest.raises(KernelError):
         HipOps("cpu")
+
+
+def test_recorded_decode_steps_equal_eager_ones(model_folders):
+    """Decode steps are replayed from a recorded HIP graph.  Every replay is
+    compared with the same step run eagerly on a second runner, with eager work
+    (prefill of new requests, steps of other shapes) and synchronisation between
+    the replays, and while requests come and go so that pages and slots change."""
+    from tiny_llm_infer_amd.engine.loading import load_model
+    from tiny_llm_infer_amd.engine.runner import ModelRunner, StepEntry
+    name = "B"
+    model, _ = load_model(model_folders[name], "bfloat16", "cuda:0")
+    make = lambda: ModelRunner(model, model.env, page_size=16, num_pages=40, max_requests=4,
+                               max_batch_tokens=256)
+    fast, slow = make(), make()
+    assert fast.use_graphs
+    slow.use_graphs = False
+    rng = np.random.default_rng(1)
+    live = {}
+    compared = 0
+    for it in range(60):
+        if len(live) < 3 and rng.random() < 0.4:
+            key = f"r{it}"
+            prompt = rng.integers(0, 384, int(rng.integers(2, 50))).tolist()
+            for r in (fast, slow):
+                r.admit(key)
+                r.step([StepEntry(key, prompt, [])])          # eager work between replays
+            live[key] = len(prompt)
+        if not live:
+            continue
+        entries = [StepEntry(k, [int(rng.integers(0, 384))], [0]) for k in live]
+        a = fast.step(entries).clone()
+        torch.cuda.synchronize()
+        b = slow.step(entries)
+        assert torch.equal(a, b), f"replay {it} differs from the eager step"
+        compared += 1
+        for k in list(live):
+            live[k] += 1
+            if live[k] > 70 or rng.random() < 0.05:
+                fast.release(k)
+                slow.release(k)
+                del live[k]
+    assert compared > 30 and fast.graph_replays == compared and len(fast.graphs) >= 3

@@ -118,6 +118,12 @@ def test_skinny_linear_against_plain_kernel_and_reference(ops, mnk, out):
     xd, wd = x.to(DEV), w.to(DEV)
     got = ops.linear(xd, wd, out_dtype=out)
     plain = ops.linear_plain(xd, wd, out_dtype=out)
+
+    class Both:                      # the matrix with its decode layout, as the parts hold it
+        w = wd
+        tiled = ops.tile_matrix(wd)
+    streamed = ops.linear(xd, Both, out_dtype=out)
+    assert torch.equal(streamed, got)          # same additions in the same order, other addresses
     want = x.double() @ w.double().t()
     scale = float(want.abs().max())
     # float32 out: only the order of the float32 additions differs
@@ -182,7 +188,8 @@ def make_step(seq_lens, new_counts, page, num_pages, seed, kv_heads, head_dim, d
                     slots=i32(list(range(len(seq_lens)))), sample_rows=i32([0]),
                     h_row_start=row_start, h_seq_start=[n - c for n, c in zip(seq_lens, new_counts)],
                     h_seq_len=list(seq_lens), h_slots=list(range(len(seq_lens))),
-                    max_rows_per_seq=max(new_counts), max_seq_len=max(seq_lens), groups=[g])
+                    max_rows_per_seq=max(new_counts), max_seq_len=max(seq_lens),
+                    reach=max(128, 1 << (max(seq_lens) - 1).bit_length()), groups=[g])
     step.cache = LayerCache(g, 0, True)
     return step, tables, pos, seq
 

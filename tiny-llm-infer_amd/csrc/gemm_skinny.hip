@@ -32,7 +32,7 @@ __device__ __forceinline__ uint4 load16_or_zero(const bf16_t* p, bool ok) {
     return ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
 }
 
-template <int RT, int MT, int WAVES, typename TO>
+template <int RT, int MT, int WAVES, typename TO, bool TILED = false>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* __restrict__ y,
                    int M, int N, int K) {
@@ -54,6 +54,9 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
         const int n = n_base + t * 16 + r;
         w_ok[t] = n < N;
         w_row[t] = w + (size_t)(w_ok[t] ? n : 0) * K;
+        if (TILED)   // blocks of 16 rows x 128 k = 4 KiB, stored [j][lane][8]: one load instruction
+                     // of a wave reads 1 KiB in a row
+            w_row[t] = w + ((size_t)(blockIdx.x * RT + t) * ((K + 127) / 128)) * 2048 + lane * 8;
     }
     const bf16_t* x_row[MT];
     bool x_ok[MT];
@@ -64,26 +67,43 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
         x_row[m] = x + (size_t)(x_ok[m] ? row : 0) * K;
     }
 
-    for (int kb = wave * 128; kb < K; kb += WAVES * 128) {
+    // two-stage pipeline: the loads of the next 128-wide step are issued before the
+    // MFMAs of the current one, so a wave keeps 4*(RT+MT) 16-byte loads in flight
+    Pack16 a[2][RT][4], b[2][MT][4];
+    auto load_step = [&](int buf, int kb) {
         const int k = kb + c * 32;
-        Pack16 a[RT][4], b[MT][4];
 #pragma unroll
         for (int t = 0; t < RT; ++t)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                a[t][j].u = load16_or_zero(w_row[t] + k + j * 8, w_ok[t] && (k + j * 8 < K));
+                a[buf][t][j].u = TILED ? *reinterpret_cast<const uint4*>(w_row[t] + (size_t)(kb / 128) * 2048 + j * 512)
+                                       : load16_or_zero(w_row[t] + k + j * 8, w_ok[t] && (k + j * 8 < K));
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                b[m][j].u = load16_or_zero(x_row[m] + k + j * 8, x_ok[m] && (k + j * 8 < K));
+                b[buf][m][j].u = load16_or_zero(x_row[m] + k + j * 8, x_ok[m] && (k + j * 8 < K));
+    };
+    auto mma_step = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int t = 0; t < RT; ++t)
 #pragma unroll
                 for (int m = 0; m < MT; ++m)
-                    acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][j].v, b[m][j].v, acc[t][m], 0, 0, 0);
+                    acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[buf][t][j].v, b[buf][m][j].v,
+                                                                        acc[t][m], 0, 0, 0);
+    };
+    int kb = wave * 128;
+    if (kb < K) load_step(0, kb);
+    for (; kb < K; kb += 2 * WAVES * 128) {
+        const int k1 = kb + WAVES * 128;
+        if (k1 < K) load_step(1, k1);
+        mma_step(0);
+        if (k1 < K) {
+            if (k1 + WAVES * 128 < K) load_step(0, k1 + WAVES * 128);
+            mma_step(1);
+        }
     }
 
 #pragma unroll
@@ -112,28 +132,46 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
 
 template <int RT, int MT, int WAVES>
 static int launch_skinny(const bf16_t* x, const bf16_t* w, void* y, int M, int N, int K, int y_dtype,
-                         hipStream_t s) {
+                         bool tiled, hipStream_t s) {
     const int blocks = (N + 16 * RT - 1) / (16 * RT);
-    if (y_dtype == TLI_BF16)
-        gemm_skinny_kernel<RT, MT, WAVES, bf16_t><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
-    else
-        gemm_skinny_kernel<RT, MT, WAVES, float><<<blocks, WAVES * 64, 0, s>>>(x, w, (float*)y, M, N, K);
+    if (tiled) {
+        if (y_dtype == TLI_BF16)
+            gemm_skinny_kernel<RT, MT, WAVES, bf16_t, true><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
+        else
+            gemm_skinny_kernel<RT, MT, WAVES, float, true><<<blocks, WAVES * 64, 0, s>>>(x, w, (float*)y, M, N, K);
+    } else {
+        if (y_dtype == TLI_BF16)
+            gemm_skinny_kernel<RT, MT, WAVES, bf16_t, false><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
+        else
+            gemm_skinny_kernel<RT, MT, WAVES, float, false><<<blocks, WAVES * 64, 0, s>>>(x, w, (float*)y, M, N, K);
+    }
     return tli_check_launch("gemm_skinny");
 }
 
 template <int MT>
 static int pick_skinny(const bf16_t* x, const bf16_t* w, void* y, int M, int N, int K, int y_dtype,
-                       hipStream_t s) {
-    // narrow outputs: one 16-column tile per workgroup and 8 waves over k, so that
-    // even N = 4096 gives 256 workgroups; wide outputs share x over more columns
+                       bool tiled, hipStream_t s, int cfg) {
+    // cfg 0: by shape.  Narrow outputs get one 16-column tile per workgroup so that
+    // even N = 4096 gives 256 workgroups; wide outputs share x over two tiles.
     const long tiles = (N + 15) / 16;
-    if (tiles >= 4096 && MT <= 2) return launch_skinny<4, MT, 4>(x, w, y, M, N, K, y_dtype, s);
-    if (tiles >= 1024) return launch_skinny<2, MT, 8>(x, w, y, M, N, K, y_dtype, s);
-    return launch_skinny<1, MT, 8>(x, w, y, M, N, K, y_dtype, s);
+    if (cfg == 0) cfg = tiles <= 256 ? 18 : (tiles < 1024 ? 28 : 24);
+    switch (cfg) {
+        case 14: return launch_skinny<1, MT, 4>(x, w, y, M, N, K, y_dtype, tiled, s);
+        case 18: return launch_skinny<1, MT, 8>(x, w, y, M, N, K, y_dtype, tiled, s);
+        case 24: return launch_skinny<2, MT, 4>(x, w, y, M, N, K, y_dtype, tiled, s);
+        case 28: return launch_skinny<2, MT, 8>(x, w, y, M, N, K, y_dtype, tiled, s);
+        default: return tli_fail("gemm_skinny: unknown configuration %d", cfg);
+    }
 }
 
+// y[M,N] = x[M,K] . W^T.  `tiled` = 0: w is W[N,K] row-major.  `tiled` = 1: w is the
+// same matrix in blocks of 16 rows x 128 columns, zero-padded to whole blocks, stored
+// [row block][column block][j = 0..3][lane = 16*c + r][8] with element
+// W[16*row block + r][128*column block + 32*c + 8*j + e]: every load instruction of
+// a wave then reads 1 KiB in a row.  cfg 0 picks the launch shape; other values
+// (row tiles * 10 + waves) force one, for measurements.
 extern "C" int tli_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K,
-                                    int y_dtype, void* stream) {
+                                    int y_dtype, int tiled, int cfg, void* stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64) return tli_fail("gemm_skinny: %d rows, at most 64", M);
     if (K <= 0 || K % 8) return tli_fail("gemm_skinny: K = %d must be a positive multiple of 8", K);
@@ -143,9 +181,9 @@ extern "C" int tli_gemm_skinny_bf16(const void* x, const void* w, void* y, int M
     const bf16_t* xp = (const bf16_t*)x;
     const bf16_t* wp = (const bf16_t*)w;
     switch ((M + 15) / 16) {
-        case 1: return pick_skinny<1>(xp, wp, y, M, N, K, y_dtype, s);
-        case 2: return pick_skinny<2>(xp, wp, y, M, N, K, y_dtype, s);
-        case 3: return pick_skinny<3>(xp, wp, y, M, N, K, y_dtype, s);
-        default: return pick_skinny<4>(xp, wp, y, M, N, K, y_dtype, s);
+        case 1: return pick_skinny<1>(xp, wp, y, M, N, K, y_dtype, tiled != 0, s, cfg);
+        case 2: return pick_skinny<2>(xp, wp, y, M, N, K, y_dtype, tiled != 0, s, cfg);
+        case 3: return pick_skinny<3>(xp, wp, y, M, N, K, y_dtype, tiled != 0, s, cfg);
+        default: return pick_skinny<4>(xp, wp, y, M, N, K, y_dtype, tiled != 0, s, cfg);
     }
 }

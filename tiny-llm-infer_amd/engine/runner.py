@@ -120,6 +120,15 @@ class ModelRunner:
         self.inputs = StepInputs(env.device, max_batch_tokens, max_requests,
                                  len(self.cache.groups), max_width)
         self.steps_run = 0
+        # Decode steps (one token for every request, every logit wanted) launch the same
+        # kernels with the same arguments whenever (requests, table width, reach) agree:
+        # their launch sequence is recorded once as a HIP graph and replayed.
+        parts = [model.embedding, model.final_norm, model.head] + list(model.blocks)
+        self.use_graphs = (env.device.type == "cuda" and env.dtype == torch.bfloat16
+                           and all(p.replayable for p in parts))
+        self.graphs = {}
+        self.graph_pool = None
+        self.graph_replays = 0
 
     # ---- requests ---------------------------------------------------------
     def admit(self, key: Hashable):
@@ -215,7 +224,8 @@ class ModelRunner:
             slots=dev[lay["slots"]], sample_rows=dev[lay["sample_rows"]],
             h_row_start=row_start, h_seq_start=starts, h_seq_len=totals,
             h_slots=[rc.slot for rc in rcs], max_rows_per_seq=max(counts),
-            max_seq_len=max(totals), groups=groups)
+            max_seq_len=max(totals), reach=max(128, 1 << (max(totals) - 1).bit_length()),
+            groups=groups)
 
     def forward(self, step: StepView, num_wanted: int) -> Optional[torch.Tensor]:
         """Run the model over a packed step; float32 logits [wanted, vocab] or None."""
@@ -239,6 +249,25 @@ class ModelRunner:
         x = model.final_norm.forward(resid, pending, rows=step.sample_rows, num_rows=num_wanted)
         return model.head.forward(x)
 
+    def _replay(self, view: StepView, wanted: int) -> torch.Tensor:
+        """A decode step through its recorded launch sequence.  The step's inputs
+        already lie in the device buffer whose layout depends on the key alone."""
+        key = (view.num_seqs, view.groups[0].table_width if view.groups else 0, view.reach)
+        entry = self.graphs.get(key)
+        if entry is None:
+            self.forward(view, wanted)                 # once eagerly: anything lazy happens now
+            torch.cuda.synchronize(self.env.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self.graph_pool):
+                out = self.forward(view, wanted)
+            if self.graph_pool is None:
+                self.graph_pool = graph.pool()
+            entry = (graph, out)
+            self.graphs[key] = entry
+        entry[0].replay()
+        self.graph_replays += 1
+        return entry[1]
+
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Run one batch.  Pages are reserved for every entry first; if the pool
         cannot hold the batch, CacheFull is raised and no token has been run."""
@@ -257,7 +286,10 @@ class ModelRunner:
             self.cache.reserve(e.key, self.cache.get(e.key).num_tokens + len(e.tokens))
         view = self._pack(entries)
         wanted = sum(len(e.want) for e in entries)
-        logits = self.forward(view, wanted)
+        if self.use_graphs and view.max_rows_per_seq == 1 and wanted == len(entries):
+            logits = self._replay(view, wanted)
+        else:
+            logits = self.forward(view, wanted)
         for e in entries:
             self.cache.advance(e.key, self.cache.get(e.key).num_tokens + len(e.tokens))
         self.steps_run += 1

@@ -53,7 +53,7 @@ def load_library():
         "tli_qkv_to_cache": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I, I, I, I, P],
         "tli_attention_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
         "tli_gemm_plain": [P, P, P, I, I, I, I, I, I, P],
-        "tli_gemm_skinny_bf16": [P, P, P, I, I, I, I, P],
+        "tli_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, I, P],
         "tli_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
         "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P],
@@ -86,6 +86,7 @@ class HipOps:
             raise KernelError("no GPU is visible to torch; this engine has no CPU path")
         self.lib = load_library()
         self.force_plain = False     # tests: run the plain attention kernel for bfloat16 too
+        self.skinny_cfg = 0          # measurements: force a launch shape of the weight-streaming kernel
 
     # ---- helpers ----------------------------------------------------------
     def _stream(self):
@@ -147,7 +148,28 @@ class HipOps:
                    _dtype_code(out_dtype), self._stream())
         return out
 
-    def linear(self, x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
+    def tile_matrix(self, w: torch.Tensor) -> Optional[torch.Tensor]:
+        """The decode layout of a bfloat16 matrix W[N,K]: blocks of 16 rows x 128
+        columns, zero-padded to whole blocks, stored [row block][column block][j][lane][8]
+        with lane = 16*c + r holding W[16*row block + r][128*column block + 32*c + 8*j + e].
+        A wave of the weight-streaming kernel then reads 4 KiB in a row per block, in the
+        order its MFMA operands want.  None if the matrix cannot use that kernel."""
+        N, K = w.shape
+        if w.dtype != torch.bfloat16 or K % 8:
+            return None
+        n16, k128 = (N + 15) // 16 * 16, (K + 127) // 128 * 128
+        if (n16, k128) != (N, K):
+            padded = torch.zeros((n16, k128), dtype=w.dtype, device=w.device)
+            padded[:N, :K] = w
+            w = padded
+        t = w.view(n16 // 16, 16, k128 // 128, 4, 4, 8)          # [nb, r, kb, c, j, e]
+        return t.permute(0, 2, 4, 3, 1, 5).contiguous()           # [nb, kb, j, c, r, e]
+
+    def linear(self, x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None):
+        """y = x W^T.  ``w`` is a [N, K] tensor or a ``Matrix`` (row-major tensor plus
+        its decode layout)."""
+        tiled = getattr(w, "tiled", None)
+        w = getattr(w, "w", w)
         M, K = x.shape
         N, K2 = w.shape
         if K != K2:
@@ -164,10 +186,12 @@ class HipOps:
             if M <= self.SKINNY_ROWS or out_dtype == torch.float32:
                 # few rows (decode), or float32 logits: the weight-streaming MFMA kernel,
                 # 64 rows at a time
+                wp = w if tiled is None else tiled
                 for m0 in range(0, M, self.SKINNY_ROWS):
                     m1 = min(M, m0 + self.SKINNY_ROWS)
-                    self._call(self.lib.tli_gemm_skinny_bf16, x[m0:m1].data_ptr(), w.data_ptr(),
-                               y[m0:m1].data_ptr(), m1 - m0, N, K, _dtype_code(out_dtype), self._stream())
+                    self._call(self.lib.tli_gemm_skinny_bf16, x[m0:m1].data_ptr(), wp.data_ptr(),
+                               y[m0:m1].data_ptr(), m1 - m0, N, K, _dtype_code(out_dtype),
+                               0 if tiled is None else 1, self.skinny_cfg, self._stream())
                 return y
             # many rows (prefill): the library's matrix product, as the reference
             # uses its library for more than one row (kernels/src/matmul_kernel_cuda.cu:84-91)
@@ -267,7 +291,7 @@ class HipOps:
         """One row per sequence.  The keys are split over workgroups when the
         batch alone would leave most of the 256 compute units idle."""
         T = step.num_rows
-        reach = step.max_seq_len if not window else min(step.max_seq_len, window + 32)
+        reach = step.reach if not window else min(step.reach, (window + 31) // 32 * 32 + 32)
         groups = T * kv_heads * ((heads // kv_heads + 15) // 16)
         splits = max(1, min((self.DECODE_WORKGROUPS + groups - 1) // groups, (reach + 127) // 128, 64))
         per_split = ((reach + splits - 1) // splits + 127) // 128 * 128

@@ -23,6 +23,8 @@ from .linear import as_matrix, fuse_rows
 
 
 class PagedAttention(Mixer):
+    replayable = True
+
     def __init__(self, spec):
         super().__init__(spec)
         p = spec.params

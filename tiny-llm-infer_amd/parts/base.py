@@ -81,6 +81,8 @@ class StepView:
     h_slots: List[int] = field(default_factory=list)
     max_rows_per_seq: int = 1
     max_seq_len: int = 1
+    reach: int = 1                # max_seq_len rounded up to a power of two: launches are shaped by
+                                  # this, so that steps of like shape launch alike (and can be replayed)
     groups: List[GroupView] = field(default_factory=list)
     # filled by the runner for the layer call that is running
     cache: Optional[LayerCache] = None
@@ -88,6 +90,10 @@ class StepView:
 
 
 class Part:
+    # True if forward() looks at nothing on the host but the step's shape (rows,
+    # sequences, table width, reach): then a recorded launch sequence can be replayed
+    replayable = False
+
     def __init__(self, spec: PartSpec):
         self.spec = spec
 

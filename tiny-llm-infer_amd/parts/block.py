@@ -15,6 +15,7 @@ from .base import Block, BuildEnv, StepView, register_part
 class PreNormBlock(Block):
     def __init__(self, spec, mixer, ffn, norms):
         super().__init__(spec)
+        self.replayable = all(p.replayable for p in (mixer, ffn, *norms.values()))
         self.mixer = mixer
         self.ffn = ffn
         self.norm_mixer = norms["mixer"]

@@ -16,6 +16,8 @@ from .linear import as_matrix
 
 
 class TokenEmbedding(Part):
+    replayable = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.vocab = int(spec.params["vocab_size"])
@@ -27,7 +29,7 @@ class TokenEmbedding(Part):
 
     def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
         super().load(weights, env)
-        self.table = as_matrix(weights[self.name], env)
+        self.table = weights[self.name].to(env.dtype).contiguous()      # rows are gathered: row-major only
 
     def forward(self, token_ids: torch.Tensor, num_rows: int) -> torch.Tensor:
         """Rows of the table as a float32 residual stream [rows, hidden]."""
@@ -35,6 +37,8 @@ class TokenEmbedding(Part):
 
 
 class LinearHead(Part):
+    replayable = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.vocab = int(spec.params["vocab_size"])
@@ -47,7 +51,7 @@ class LinearHead(Part):
     def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv, share_with=None) -> None:
         super().load(weights, env)
         if share_with is not None and share_with.name == self.name:
-            self.weight = share_with.table          # tied: one matrix on the device
+            self.weight = as_matrix(share_with.table, env)     # tied: the row-major copy is shared
         else:
             self.weight = as_matrix(weights[self.name], env)
 

@@ -14,6 +14,8 @@ from .linear import as_matrix, fuse_rows
 
 
 class SwiGLU(FeedForward):
+    replayable = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.hidden = int(spec.params["hidden_size"])

@@ -13,6 +13,8 @@ from .base import BuildEnv, Norm, register_part
 
 
 class RMSNorm(Norm):
+    replayable = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.size = int(spec.params["size"])
