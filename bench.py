@@ -58,6 +58,7 @@ def main():
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiles)")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -133,8 +134,11 @@ def main():
         dt = time.perf_counter() - t
         assert engine.is_finished()
         return dt
-    prefill_once()
-    pre = min(prefill_once() for _ in range(3))
+    if args.no_prefill:
+        pre = float("nan")
+    else:
+        prefill_once()
+        pre = min(prefill_once() for _ in range(3))
     T = args.prefill_tokens
     pre_flops = step_flops(cfg_json, layers, T, T * (T + 1) / 2.0, 1)
 

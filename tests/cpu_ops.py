@@ -37,6 +37,9 @@ class CpuOps:
         y = x.to(torch.float32) @ w.to(torch.float32).t()
         return y.to(out_dtype or x.dtype)
 
+    def linear_swiglu(self, x, m):
+        return self.swiglu(self.linear(x, m))
+
     def swiglu(self, gu):
         inter = gu.shape[1] // 2
         g, u = gu[:, :inter].to(torch.float32), gu[:, inter:].to(torch.float32)

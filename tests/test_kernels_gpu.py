@@ -132,6 +132,24 @@ def test_skinny_linear_against_plain_kernel_and_reference(ops, mnk, out):
     assert float((plain.double().cpu() - want).abs().max()) <= bound
 
 
+@pytest.mark.parametrize("mki", [(1, 64, 32), (8, 4096, 12288), (33, 96, 160), (64, 264, 1008)])
+def test_gated_product_writes_the_activation(ops, mki):
+    """gate and up interleaved in the decode layout: one pass, silu(g)*u in the epilogue."""
+    from tiny_llm_infer_amd.engine.loading import make_env
+    from tiny_llm_infer_amd.parts.linear import GatedMatrix
+    M, K, I = mki
+    env = make_env(torch.bfloat16, DEV)
+    gate, up = rnd((I, K), torch.bfloat16, 3, 0.05), rnd((I, K), torch.bfloat16, 4, 0.05)
+    x = rnd((M, K), torch.bfloat16, 5)
+    m = GatedMatrix(gate.to(DEV), up.to(DEV), env)
+    assert m.gated is not None
+    got = ops.linear_swiglu(x.to(DEV), m)
+    g, u = x.double() @ gate.double().t(), x.double() @ up.double().t()
+    close(got, torch.nn.functional.silu(g) * u, torch.bfloat16, "gated product")
+    two_pass = ops.swiglu(ops.linear(x.to(DEV), m.w))
+    close(two_pass, torch.nn.functional.silu(g) * u, torch.bfloat16, "stacked product, then activation")
+
+
 def test_library_linear_for_many_rows(ops):
     x, w = rnd((300, 264), torch.bfloat16, 1), rnd((130, 264), torch.bfloat16, 2, 0.05)
     close(ops.linear(x.to(DEV), w.to(DEV)), x.double() @ w.double().t(), torch.bfloat16, "library product")

@@ -47,6 +47,89 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
     }
 }
 
+// The same with the row held in registers: n % 4 == 0 and n <= 4 * blockDim.x * IT.
+// Each thread owns IT groups of 4 consecutive elements, read and written once.
+__device__ __forceinline__ void load4(const float* p, float v[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void load4(const bf16_t* p, float v[4]) {
+    const uint2 t = *reinterpret_cast<const uint2*>(p);
+    v[0] = bf16_to_f32((bf16_t)(t.x & 0xffffu)); v[1] = bf16_to_f32((bf16_t)(t.x >> 16));
+    v[2] = bf16_to_f32((bf16_t)(t.y & 0xffffu)); v[3] = bf16_to_f32((bf16_t)(t.y >> 16));
+}
+__device__ __forceinline__ void store4(float* p, const float v[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store4(bf16_t* p, const float v[4]) {
+    uint2 t;
+    t.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+    t.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+    *reinterpret_cast<uint2*>(p) = t;
+}
+
+template <typename T, int IT>
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+                                       const float* __restrict__ weight, T* __restrict__ out,
+                                       const int* __restrict__ rows, int n, float eps, int total_rows) {
+    __shared__ float scratch[16];
+    const int out_row = blockIdx.x;
+    int r = rows ? rows[out_row] : out_row;
+    if (r < 0 || r >= total_rows) r = 0;
+    float* x = resid + (size_t)r * n;
+    const T* d = delta ? delta + (size_t)r * n : nullptr;
+    const bool update = (rows == nullptr) && (d != nullptr);
+    float v[IT][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const int i = (threadIdx.x + it * blockDim.x) * 4;
+        if (i < n) {
+            load4(x + i, v[it]);
+            if (d) {
+                float dv[4];
+                load4(d + i, dv);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[it][e] += dv[e];
+                if (update) store4(x + i, v[it]);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ss += v[it][e] * v[it][e];
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)n + eps);
+    T* o = out + (size_t)out_row * n;
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const int i = (threadIdx.x + it * blockDim.x) * 4;
+        if (i < n) {
+            float w[4], y[4];
+            load4(weight + i, w);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) y[e] = w[e] * v[it][e] * scale;
+            store4(o + i, y);
+        }
+    }
+}
+
+template <typename T>
+static void launch_add_rmsnorm(float* resid, const T* delta, const float* weight, T* out, const int* rows,
+                               int out_rows, int total_rows, int n, float eps, hipStream_t s) {
+    const int groups = n / 4;
+    if (n % 4 == 0 && groups <= 4096) {
+        int threads = groups <= 1024 ? (groups + 63) / 64 * 64 : 1024;
+        if (groups <= 1024)
+            add_rmsnorm_vec_kernel<T, 1><<<out_rows, threads, 0, s>>>(resid, delta, weight, out, rows, n, eps, total_rows);
+        else if (groups <= 2048)
+            add_rmsnorm_vec_kernel<T, 2><<<out_rows, threads, 0, s>>>(resid, delta, weight, out, rows, n, eps, total_rows);
+        else
+            add_rmsnorm_vec_kernel<T, 4><<<out_rows, threads, 0, s>>>(resid, delta, weight, out, rows, n, eps, total_rows);
+        return;
+    }
+    add_rmsnorm_kernel<T><<<out_rows, n >= 2048 ? 512 : 256, 0, s>>>(resid, delta, weight, out, rows, n, eps, total_rows);
+}
+
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -78,13 +161,12 @@ extern "C" int tli_add_rmsnorm(float* resid, const void* delta, const float* wei
     if (out_rows <= 0) return 0;
     if (n <= 0) return tli_fail("add_rmsnorm: bad row size %d", n);
     hipStream_t s = (hipStream_t)stream;
-    const int threads = n >= 2048 ? 512 : 256;
     if (dtype == TLI_F32)
-        add_rmsnorm_kernel<float><<<out_rows, threads, 0, s>>>(resid, (const float*)delta, weight,
-                                                             (float*)out, rows, n, eps, total_rows);
+        launch_add_rmsnorm<float>(resid, (const float*)delta, weight, (float*)out, rows, out_rows,
+                                  total_rows, n, eps, s);
     else if (dtype == TLI_BF16)
-        add_rmsnorm_kernel<bf16_t><<<out_rows, threads, 0, s>>>(resid, (const bf16_t*)delta, weight,
-                                                              (bf16_t*)out, rows, n, eps, total_rows);
+        launch_add_rmsnorm<bf16_t>(resid, (const bf16_t*)delta, weight, (bf16_t*)out, rows, out_rows,
+                                   total_rows, n, eps, s);
     else
         return tli_fail("add_rmsnorm: unknown dtype %d", dtype);
     return tli_check_launch("add_rmsnorm");

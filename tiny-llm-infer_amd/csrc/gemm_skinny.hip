@@ -32,7 +32,7 @@ __device__ __forceinline__ uint4 load16_or_zero(const bf16_t* p, bool ok) {
     return ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
 }
 
-template <int RT, int MT, int WAVES, typename TO, bool TILED = false>
+template <int RT, int MT, int WAVES, typename TO, bool TILED = false, bool GATED = false>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* __restrict__ y,
                    int M, int N, int K) {
@@ -113,6 +113,30 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
 #pragma unroll
             for (int i = 0; i < 4; ++i) red[wave][t * MT + m][lane][i] = acc[t][m][i];
     __syncthreads();
+    if (GATED) {
+        // row tiles come in pairs (gate rows, up rows of the same 16 outputs): the
+        // epilogue writes silu(gate) * up, N/2 columns (kernels/src/swiglu_kernel_cpu.cpp:20-24)
+        const int n_out = N / 2;
+        for (int pair = wave; pair < (RT / 2) * MT; pair += WAVES) {
+            const int tp = pair / MT, m = pair % MT;
+            float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int wv = 0; wv < WAVES; ++wv)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    g[i] += red[wv][(2 * tp) * MT + m][lane][i];
+                    u[i] += red[wv][(2 * tp + 1) * MT + m][lane][i];
+                }
+            const int row = m * 16 + r;
+            const int n0 = (blockIdx.x * (RT / 2) + tp) * 16 + c * 4;
+            if (row < M) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n0 + i < n_out)
+                        from_f32(y + (size_t)row * n_out + n0 + i, g[i] / (1.0f + expf(-g[i])) * u[i]);
+            }
+        }
+        return;
+    }
     // tiles are shared out over the waves; each sums the partials in wave order
     for (int tile = wave; tile < RT * MT; tile += WAVES) {
         const int t = tile / MT, m = tile % MT;
@@ -132,9 +156,11 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
 
 template <int RT, int MT, int WAVES>
 static int launch_skinny(const bf16_t* x, const bf16_t* w, void* y, int M, int N, int K, int y_dtype,
-                         bool tiled, hipStream_t s) {
+                         int tiled, hipStream_t s) {
     const int blocks = (N + 16 * RT - 1) / (16 * RT);
-    if (tiled) {
+    if (tiled == 2) {       // gated: pairs of row tiles, silu(gate)*up written as bfloat16
+        gemm_skinny_kernel<RT, MT, WAVES, bf16_t, true, true><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
+    } else if (tiled) {
         if (y_dtype == TLI_BF16)
             gemm_skinny_kernel<RT, MT, WAVES, bf16_t, true><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
         else
@@ -150,11 +176,12 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, void* y, int M, int N
 
 template <int MT>
 static int pick_skinny(const bf16_t* x, const bf16_t* w, void* y, int M, int N, int K, int y_dtype,
-                       bool tiled, hipStream_t s, int cfg) {
+                       int tiled, hipStream_t s, int cfg) {
     // cfg 0: by shape.  Narrow outputs get one 16-column tile per workgroup so that
     // even N = 4096 gives 256 workgroups; wide outputs share x over two tiles.
     const long tiles = (N + 15) / 16;
     if (cfg == 0) cfg = tiles <= 256 ? 18 : (tiles < 1024 ? 28 : 24);
+    if (tiled == 2 && cfg < 20) cfg = 24;          // gated needs pairs of row tiles
     switch (cfg) {
         case 14: return launch_skinny<1, MT, 4>(x, w, y, M, N, K, y_dtype, tiled, s);
         case 18: return launch_skinny<1, MT, 8>(x, w, y, M, N, K, y_dtype, tiled, s);
@@ -168,7 +195,9 @@ static int pick_skinny(const bf16_t* x, const bf16_t* w, void* y, int M, int N, 
 // same matrix in blocks of 16 rows x 128 columns, zero-padded to whole blocks, stored
 // [row block][column block][j = 0..3][lane = 16*c + r][8] with element
 // W[16*row block + r][128*column block + 32*c + 8*j + e]: every load instruction of
-// a wave then reads 1 KiB in a row.  cfg 0 picks the launch shape; other values
+// a wave then reads 1 KiB in a row.  `tiled` = 2: tiled, and the 16-row blocks alternate
+// between a gate matrix and an up matrix (block 2t: gate rows 16t.., block 2t+1: up rows
+// 16t..); N counts both, y is [M, N/2] bfloat16 = silu(x.gate^T) * (x.up^T).  cfg 0 picks the launch shape; other values
 // (row tiles * 10 + waves) force one, for measurements.
 extern "C" int tli_gemm_skinny_bf16(const void* x, const void* w, void* y, int M, int N, int K,
                                     int y_dtype, int tiled, int cfg, void* stream) {
@@ -176,14 +205,17 @@ extern "C" int tli_gemm_skinny_bf16(const void* x, const void* w, void* y, int M
     if (M > 64) return tli_fail("gemm_skinny: %d rows, at most 64", M);
     if (K <= 0 || K % 8) return tli_fail("gemm_skinny: K = %d must be a positive multiple of 8", K);
     if (y_dtype != TLI_BF16 && y_dtype != TLI_F32) return tli_fail("gemm_skinny: bad output dtype %d", y_dtype);
+    if (tiled < 0 || tiled > 2) return tli_fail("gemm_skinny: bad layout code %d", tiled);
+    if (tiled == 2 && (N % 32 || y_dtype != TLI_BF16))
+        return tli_fail("gemm_skinny: a gated product needs N %% 32 == 0 and bfloat16 output");
     if (((uintptr_t)x | (uintptr_t)w) & 15) return tli_fail("gemm_skinny: operands must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xp = (const bf16_t*)x;
     const bf16_t* wp = (const bf16_t*)w;
     switch ((M + 15) / 16) {
-        case 1: return pick_skinny<1>(xp, wp, y, M, N, K, y_dtype, tiled != 0, s, cfg);
-        case 2: return pick_skinny<2>(xp, wp, y, M, N, K, y_dtype, tiled != 0, s, cfg);
-        case 3: return pick_skinny<3>(xp, wp, y, M, N, K, y_dtype, tiled != 0, s, cfg);
-        default: return pick_skinny<4>(xp, wp, y, M, N, K, y_dtype, tiled != 0, s, cfg);
+        case 1: return pick_skinny<1>(xp, wp, y, M, N, K, y_dtype, tiled, s, cfg);
+        case 2: return pick_skinny<2>(xp, wp, y, M, N, K, y_dtype, tiled, s, cfg);
+        case 3: return pick_skinny<3>(xp, wp, y, M, N, K, y_dtype, tiled, s, cfg);
+        default: return pick_skinny<4>(xp, wp, y, M, N, K, y_dtype, tiled, s, cfg);
     }
 }

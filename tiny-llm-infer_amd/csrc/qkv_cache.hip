@@ -51,8 +51,19 @@ __global__ void qkv_to_cache_kernel(
     }
 
     float* x = stage[wave];
-    // heads 0..heads-1 are q, heads..heads+kv_heads-1 are k
-    for (int h = wave; h < heads + kv_heads; h += QKV_WAVES) {
+    // units 0..heads-1 are q heads, heads..heads+kv_heads-1 are k heads, then the v heads;
+    // a workgroup takes QKV_WAVES consecutive units, one a wave
+    const int h = blockIdx.y * QKV_WAVES + wave;
+    if (h >= heads + 2 * kv_heads) return;
+    if (h >= heads + kv_heads) {
+        if (!can_write) return;
+        const int g = h - heads - kv_heads;
+        const T* vsrc = src_row + q_dim + kv_dim + (size_t)g * head_dim;
+        for (int d = lane; d < head_dim; d += TLI_WAVE)
+            v_cache[v_base + ((size_t)g * head_dim + d) * page_size] = vsrc[d];
+        return;
+    }
+    {
         const bool is_q = h < heads;
         const T* src = src_row + (size_t)h * head_dim;     // q heads then k heads are contiguous
         const float* nw = is_q ? q_norm_w : k_norm_w;
@@ -75,7 +86,7 @@ __global__ void qkv_to_cache_kernel(
         if (is_q) {
             dst = q_out + (size_t)row * q_dim + (size_t)h * head_dim;
         } else {
-            if (!can_write) continue;
+            if (!can_write) return;
             dst = k_cache + cache_base + (size_t)(h - heads) * page_size * head_dim;
         }
         for (int i = lane; i < head_dim; i += TLI_WAVE) {
@@ -85,14 +96,6 @@ __global__ void qkv_to_cache_kernel(
                 else v = x[i - half] * sin_row[i - half] + x[i] * cos_row[i - half];
             }
             from_f32(dst + i, v);
-        }
-        wave_lds_sync();
-    }
-    if (can_write) {
-        const T* vsrc = src_row + q_dim + kv_dim;
-        for (int i = threadIdx.x; i < kv_dim; i += blockDim.x) {
-            const int g = i / head_dim, d = i - g * head_dim;
-            v_cache[v_base + ((size_t)g * head_dim + d) * page_size] = vsrc[i];
         }
     }
 }
@@ -114,13 +117,16 @@ extern "C" int tli_qkv_to_cache(
         return tli_fail("qkv_to_cache: bad cache geometry");
     hipStream_t s = (hipStream_t)stream;
     const int threads = QKV_WAVES * TLI_WAVE;
+    const int units = heads + 2 * kv_heads;
+    if ((units + QKV_WAVES - 1) / QKV_WAVES > 65535) return tli_fail("qkv_to_cache: too many heads");
+    dim3 grid(rows, (units + QKV_WAVES - 1) / QKV_WAVES);
     if (dtype == TLI_F32)
-        qkv_to_cache_kernel<float><<<rows, threads, 0, s>>>(
+        qkv_to_cache_kernel<float><<<grid, threads, 0, s>>>(
             (const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache, positions, seq_of_row,
             tables, table_width, page_size, num_pages, heads, kv_heads, head_dim, q_norm_w, q_eps,
             k_norm_w, k_eps, cos_table, sin_table, rotary_dim, table_positions, write_cache);
     else if (dtype == TLI_BF16)
-        qkv_to_cache_kernel<bf16_t><<<rows, threads, 0, s>>>(
+        qkv_to_cache_kernel<bf16_t><<<grid, threads, 0, s>>>(
             (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, positions, seq_of_row,
             tables, table_width, page_size, num_pages, heads, kv_heads, head_dim, q_norm_w, q_eps,
             k_norm_w, k_eps, cos_table, sin_table, rotary_dim, table_positions, write_cache);

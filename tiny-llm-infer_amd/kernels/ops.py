@@ -213,6 +213,20 @@ class HipOps:
                    _dtype_code(x.dtype), _dtype_code(w.dtype), _dtype_code(out_dtype), self._stream())
         return y
 
+    def linear_swiglu(self, x: torch.Tensor, m) -> torch.Tensor:
+        """silu(x gate^T) * (x up^T) for a ``GatedMatrix``.  Few rows: one pass of
+        the weight-streaming kernel over the interleaved layout, the activation in
+        its epilogue.  Otherwise the stacked product, then the activation."""
+        M, K = x.shape
+        gated = getattr(m, "gated", None)
+        if gated is not None and 0 < M <= self.SKINNY_ROWS and x.dtype == torch.bfloat16:
+            self._want(x, "linear input", torch.bfloat16, (M, m.w.shape[1]))
+            y = torch.empty((M, m.inter), dtype=x.dtype, device=self.device)
+            self._call(self.lib.tli_gemm_skinny_bf16, x.data_ptr(), gated.data_ptr(), y.data_ptr(), M,
+                       2 * m.inter, K, BF16, 2, self.skinny_cfg if self.skinny_cfg >= 20 else 0, self._stream())
+            return y
+        return self.swiglu(self.linear(x, m))
+
     def swiglu(self, gu: torch.Tensor) -> torch.Tensor:
         rows, two = gu.shape
         if two % 2:

@@ -26,6 +26,28 @@ class Matrix:
         return self.w.shape
 
 
+class GatedMatrix(Matrix):
+    """A gate matrix and an up matrix that read the same input, for
+    silu(x gate^T) * (x up^T).  ``w`` stacks them ([gate; up], one product for many
+    rows, the activation in a pass of its own); ``gated`` is the decode layout with
+    the 16-row blocks of gate and up alternating, so that the weight-streaming
+    kernel holds both sums of an output and writes the activation itself."""
+
+    def __init__(self, gate: torch.Tensor, up: torch.Tensor, env: BuildEnv):
+        super().__init__(torch.cat([gate.to(env.dtype), up.to(env.dtype)], dim=0), env, decode_layout=False)
+        self.inter = gate.shape[0]
+        self.gated = None
+        tile = getattr(env.ops, "tile_matrix", None)
+        if tile is not None and self.inter % 16 == 0 and env.dtype == torch.bfloat16:
+            k = gate.shape[1]
+            pairs = torch.stack([self.w[:self.inter].view(-1, 16, k), self.w[self.inter:].view(-1, 16, k)], dim=1)
+            self.gated = tile(pairs.reshape(2 * self.inter, k))
+            if self.gated is None:          # the kernel cannot take this width: plain decode layout
+                self.tiled = tile(self.w)
+        elif tile is not None:
+            self.tiled = tile(self.w)
+
+
 def as_matrix(t: torch.Tensor, env: BuildEnv) -> Matrix:
     """A loaded matrix ready for products."""
     return Matrix(t, env)

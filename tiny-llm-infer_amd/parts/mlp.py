@@ -10,7 +10,7 @@ import torch
 
 from ..weights.loader import TensorDecl
 from .base import BuildEnv, FeedForward, StepView, register_part
-from .linear import as_matrix, fuse_rows
+from .linear import GatedMatrix, as_matrix
 
 
 class SwiGLU(FeedForward):
@@ -30,13 +30,12 @@ class SwiGLU(FeedForward):
     def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
         super().load(weights, env)
         n = self.spec.names
-        self.w_gate_up = fuse_rows([weights[n["gate"]], weights[n["up"]]], env)
+        self.w_gate_up = GatedMatrix(weights[n["gate"]], weights[n["up"]], env)
         self.w_down = as_matrix(weights[n["down"]], env)
 
     def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
         ops = self.env.ops
-        gu = ops.linear(x, self.w_gate_up)
-        return ops.linear(ops.swiglu(gu), self.w_down)
+        return ops.linear(ops.linear_swiglu(x, self.w_gate_up), self.w_down)
 
 
 register_part("ffn", "swiglu", SwiGLU)
