@@ -59,6 +59,7 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiles)")
+    ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement (for profiles)")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -117,7 +118,10 @@ def main():
             engine.step()
         return dt, (ctx0 + ctx1) / 2.0
 
-    dt, ctx_tokens = decode_run(args.batch, args.steps, args.warmup)
+    if args.no_decode:
+        dt, ctx_tokens = float("nan"), 0.0
+    else:
+        dt, ctx_tokens = decode_run(args.batch, args.steps, args.warmup)
     ms_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     step_bytes = weight_bytes(cfg_json, layers, elem) + ctx_tokens * kv_bytes_per_token(cfg_json, layers, elem)

@@ -261,17 +261,18 @@ ATT_CASES = [
 ]
 
 
-@pytest.mark.parametrize("dtype", DTYPES + ["bfloat16-plain"])
+@pytest.mark.parametrize("dtype", DTYPES + ["bfloat16-plain", "bfloat16-direct", "bfloat16-lds1", "bfloat16-lds2"])
 @pytest.mark.parametrize("case", ATT_CASES)
 def test_paged_attention(ops, dtype, case):
     """float32: the plain kernel.  bfloat16: the MFMA kernels (decode when every
     sequence brings one row, prefill otherwise), and the plain kernel beside them."""
     ops.force_plain = dtype == "bfloat16-plain"
+    ops.prefill_direct = {"bfloat16-direct": 1, "bfloat16-lds1": 2, "bfloat16-lds2": 3}.get(dtype, 0)
     dtype = torch.bfloat16 if isinstance(dtype, str) else dtype
     try:
         _paged_attention_case(ops, dtype, case)
     finally:
-        ops.force_plain = False
+        ops.force_plain, ops.prefill_direct = False, 0
 
 
 def _paged_attention_case(ops, dtype, case):

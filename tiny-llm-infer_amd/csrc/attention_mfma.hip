@@ -78,12 +78,82 @@ __device__ __forceinline__ void tile_load_q(Tile<NJ, ND>& t, const bf16_t* q_hea
     }
 }
 
-// Process the 32 keys t0 .. t0+31 (t0 a multiple of 32).
-template <int NJ, int ND>
-__device__ __forceinline__ void tile_step(Tile<NJ, ND>& t, const CacheView& cv, int t0, float scale) {
-    const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
-    // ---- scores: two 16-key tiles --------------------------------------
+// Scores, softmax update and output accumulation of one column tile for 32 keys
+// whose fragments are given.  Row 4c+i of score tile u (and k-slot 4u+i of lane
+// group c in the output MFMA) is the key  key_c0 + u*u_stride + i.
+// The running maximum is kept in units of log2: scores are multiplied by
+// scale*log2(e) and exponentials are exp2 (one v_exp_f32 each).  MASK = false
+// skips the comparison with lo..pos when the caller knows every key is seen by
+// every live column.
+template <int NJ, int ND, bool MASK>
+__device__ __forceinline__ void tile_consume(Tile<NJ, ND>& t, const Frag (&ka)[2][NJ], const Frag (&vt)[ND],
+                                             int key_c0, int u_stride, float scale_log2) {
+    // ---- scores ------------------------------------------------------------
     f32x4 s[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        s[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+            s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[u][j].v, t.q[j].v, s[u], 0, 0, 0);
+    }
+    // ---- softmax over this column -------------------------------------------
+    float p[2][4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float v = s[u][i] * scale_log2;
+            if (MASK) {
+                const int key = key_c0 + u * u_stride + i;
+                v = (key >= t.lo && key <= t.pos) ? v : -INFINITY;
+            } else if (t.pos < 0) {
+                v = -INFINITY;                                   // an idle column
+            }
+            p[u][i] = v;
+            mx = fmaxf(mx, v);
+        }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(t.m, mx);
+    const float base = (m_new == -INFINITY) ? 0.f : m_new;      // nothing seen yet: all p become 0
+    const float corr = __builtin_amdgcn_exp2f(t.m - base);      // exp2(-inf) = 0 on the first block
+    float sum = 0.f;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            p[u][i] = __builtin_amdgcn_exp2f(p[u][i] - base);
+            sum += p[u][i];
+        }
+    Frag pb;
+    pb.u = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
+                      pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    t.l = t.l * corr + sum;
+    t.m = m_new;
+    // ---- output ----------------------------------------------------------------
+    // the accumulators are rescaled only if some column's maximum moved
+    if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) t.acc[dt][i] *= corr;
+    }
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt)
+        t.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt].v, pb.v, t.acc[dt], 0, 0, 0);
+}
+
+// Process the 32 keys t0 .. t0+31 (t0 a multiple of 32) for CT column tiles that
+// share the key and value fragments (one load from the cache, CT times the MFMAs).
+template <int NJ, int ND, int CT>
+__device__ __forceinline__ void tiles_step(Tile<NJ, ND> (&tiles)[CT], const CacheView& cv, int t0, float scale) {
+    const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
+    // ---- key fragments: two 16-key tiles -----------------------------------
+    Frag ka[2][NJ];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
         const int key = t0 + u * 16 + r;                       // the key this lane loads as an A row
@@ -91,16 +161,13 @@ __device__ __forceinline__ void tile_step(Tile<NJ, ND>& t, const CacheView& cv, 
         const bool ok = page >= 0 && page < cv.num_pages;
         const bf16_t* kp = cv.k + (((size_t)(ok ? page : 0) * cv.kv_heads + cv.kv_head) * cv.page_size +
                                    (key & (cv.page_size - 1))) * cv.head_dim;
-        s[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             const int d = c * 8 * NJ + j * 8;
-            Frag a;
-            a.u = (ok && d < cv.head_dim) ? *reinterpret_cast<const uint4*>(kp + d) : make_uint4(0, 0, 0, 0);
-            s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, t.q[j].v, s[u], 0, 0, 0);
+            ka[u][j].u = (ok && d < cv.head_dim) ? *reinterpret_cast<const uint4*>(kp + d) : make_uint4(0, 0, 0, 0);
         }
     }
-    // ---- values: issue the loads before the softmax arithmetic ----------------
+    // ---- value fragments: issued before the softmax arithmetic ------------------
     // lane (dim r of tile dt, group c) takes keys t0+4c..+3 and t0+16+4c..+3
     Frag vt[ND];
     {
@@ -119,44 +186,14 @@ __device__ __forceinline__ void tile_step(Tile<NJ, ND>& t, const CacheView& cv, 
             vt[dt].h[1] = ok_b ? *reinterpret_cast<const uint2*>(vb + off) : make_uint2(0, 0);
         }
     }
-    // ---- softmax over this column -----------------------------------------
-    float p[2][4];
-    float mx = -INFINITY;
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int key = t0 + u * 16 + 4 * c + i;
-            const bool seen = key >= t.lo && key <= t.pos;
-            p[u][i] = seen ? s[u][i] * scale : -INFINITY;
-            mx = fmaxf(mx, p[u][i]);
-        }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(t.m, mx);
-    const float base = (m_new == -INFINITY) ? 0.f : m_new;      // nothing seen yet: all p become 0
-    const float corr = __expf(t.m - base);                       // exp(-inf) = 0 on the first block
-    Frag pb;
-    float sum = 0.f;
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const bf16_t rounded = f32_to_bf16(__expf(p[u][i] - base));
-            pb.e[u * 4 + i] = rounded;
-            sum += bf16_to_f32(rounded);           // the sum uses what the matrix core will multiply
-        }
-    sum += __shfl_xor(sum, 16, 64);
-    sum += __shfl_xor(sum, 32, 64);
-    t.l = t.l * corr + sum;
-    t.m = m_new;
-    // ---- output --------------------------------------------------------------
-#pragma unroll
-    for (int dt = 0; dt < ND; ++dt) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) t.acc[dt][i] *= corr;
-        t.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt].v, pb.v, t.acc[dt], 0, 0, 0);
-    }
+    for (int ct = 0; ct < CT; ++ct) tile_consume<NJ, ND, true>(tiles[ct], ka, vt, t0 + 4 * c, 16, scale);
+}
+
+template <int NJ, int ND>
+__device__ __forceinline__ void tile_step(Tile<NJ, ND>& t, const CacheView& cv, int t0, float scale) {
+    Tile<NJ, ND> (&one)[1] = reinterpret_cast<Tile<NJ, ND>(&)[1]>(t);
+    tiles_step<NJ, ND, 1>(one, cv, t0, scale);
 }
 
 // --------------------------------------------------------------------- decode --
@@ -211,7 +248,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     float m = t.m;
     for (int w = 0; w < 3; ++w) m = fmaxf(m, lds[((size_t)w * 64 + lane) * stride]);
     const float base = (m == -INFINITY) ? 0.f : m;
-    float f = __expf(t.m - base);
+    float f = __builtin_amdgcn_exp2f(t.m - base);
     float l = t.l * f;
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt)
@@ -219,7 +256,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
         for (int i = 0; i < 4; ++i) t.acc[dt][i] *= f;
     for (int w = 0; w < 3; ++w) {
         const float* src = lds + ((size_t)w * 64 + lane) * stride;
-        f = __expf(src[0] - base);
+        f = __builtin_amdgcn_exp2f(src[0] - base);
         l += src[1] * f;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt)
@@ -238,7 +275,8 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
             *reinterpret_cast<uint2*>(o + dt * 16 + 4 * c) = packed;
         }
     } else {
-        // partial[row][head][split][head_dim + 2]: unnormalised sum, then maximum and sum of weights
+        // partial[row][head][split][head_dim + 2]: unnormalised sum, then maximum (in units of log2)
+        // and sum of weights
         float* dst = partial + (((size_t)row * heads + head) * splits + split) * (head_dim + 2);
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt)
@@ -261,14 +299,14 @@ __global__ void attention_merge_splits_kernel(const float* __restrict__ partial,
     float l = 0.f;
     for (int s = 0; s < splits; ++s) {
         const float* p = src + (size_t)s * (head_dim + 2);
-        l += p[head_dim + 1] * __expf(p[head_dim] - base);
+        l += p[head_dim + 1] * __builtin_amdgcn_exp2f(p[head_dim] - base);
     }
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
         float a = 0.f;
         for (int s = 0; s < splits; ++s) {
             const float* p = src + (size_t)s * (head_dim + 2);
-            a += p[d] * __expf(p[head_dim] - base);
+            a += p[d] * __builtin_amdgcn_exp2f(p[head_dim] - base);
         }
         out[((size_t)row * heads + head) * head_dim + d] = f32_to_bf16(a * inv);
     }
@@ -276,8 +314,10 @@ __global__ void attention_merge_splits_kernel(const float* __restrict__ partial,
 
 // -------------------------------------------------------------------- prefill --
 // grid (row blocks upper bound, kv_heads * head_tiles); 256 threads.
-// A wave owns `rq` consecutive rows of one sequence x min(group, 16) heads.
-template <int NJ, int ND>
+// A wave owns CT column tiles; a tile is `rq` consecutive rows of one sequence x
+// min(group, 16) heads; the wave's tiles are consecutive in the sequence and share
+// every key and value fragment they load.
+template <int NJ, int ND, int CT>
 __global__ void __launch_bounds__(256)
 attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                          const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
@@ -290,7 +330,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     const int head_tiles = (group + 15) / 16;
     const int kv_head = blockIdx.y / head_tiles, head_tile = blockIdx.y % head_tiles;
     const int heads_here = min(16, group - head_tile * 16);
-    const int rows_per_block = 4 * rq;
+    const int rows_per_wave = CT * rq, rows_per_block = 4 * rows_per_wave;
     // which sequence and which of its row blocks is this workgroup's?
     int block = blockIdx.x, seq = 0, first_row = 0, n_rows = 0;
     for (; seq < num_seqs; ++seq) {
@@ -301,42 +341,258 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         block -= blocks;
     }
     if (seq >= num_seqs) return;
-    const int local0 = block * rows_per_block + wave * rq;    // this wave's first row in the sequence's portion
+    const int local0 = block * rows_per_block + wave * rows_per_wave;   // this wave's first row in the portion
     if (local0 >= n_rows) return;
-    const int my_rows = min(rq, n_rows - local0);
-    // column r = (row r / heads_here, head r % heads_here)
+    const int wave_rows = min(rows_per_wave, n_rows - local0);
+    const int start = seq_start[seq];
+    // column r of tile ct = (row ct*rq + r / heads_here, head r % heads_here)
     const int col_row = r / heads_here, col_head = head_tile * 16 + r % heads_here;
-    const bool live = col_row < my_rows;
-    const int row = first_row + local0 + (live ? col_row : 0);
     const int head = kv_head * group + col_head;
-    const int pos = seq_start[seq] + local0 + col_row;
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
 
     CacheView cv{k_cache, v_cache, tables + (size_t)seq * table_width, table_width, page_size, page_shift,
                  num_pages, kv_heads, head_dim, kv_head};
-    Tile<NJ, ND> t;
-    tile_init(t);
-    t.pos = live ? pos : -1;
-    t.lo = live ? lo : 0;
-    tile_load_q(t, q + ((size_t)row * heads + head) * head_dim, head_dim, live);
-
-    const int first_pos = seq_start[seq] + local0, last_pos = first_pos + my_rows - 1;
-    const int wave_lo = window > 0 ? max(0, first_pos - window + 1) : 0;
-    for (int t0 = (wave_lo / 32) * 32; t0 <= last_pos; t0 += 32) tile_step(t, cv, t0, scale);
-
-    if (!live) return;
-    const float inv = t.l > 0.f ? 1.0f / t.l : 0.f;
-    bf16_t* o = out + ((size_t)row * heads + head) * head_dim;
+    Tile<NJ, ND> t[CT];
+    bool live[CT];
+    int row[CT];
 #pragma unroll
-    for (int dt = 0; dt < ND; ++dt) {
-        uint2 packed;
-        packed.x = (uint32_t)f32_to_bf16(t.acc[dt][0] * inv) | ((uint32_t)f32_to_bf16(t.acc[dt][1] * inv) << 16);
-        packed.y = (uint32_t)f32_to_bf16(t.acc[dt][2] * inv) | ((uint32_t)f32_to_bf16(t.acc[dt][3] * inv) << 16);
-        *reinterpret_cast<uint2*>(o + dt * 16 + 4 * c) = packed;
+    for (int ct = 0; ct < CT; ++ct) {
+        const int local = ct * rq + col_row;
+        live[ct] = col_row < rq && local < wave_rows;
+        row[ct] = first_row + local0 + (live[ct] ? local : 0);
+        const int pos = start + local0 + local;
+        tile_init(t[ct]);
+        t[ct].pos = live[ct] ? pos : -1;
+        t[ct].lo = live[ct] ? (window > 0 ? max(0, pos - window + 1) : 0) : 0;
+        tile_load_q(t[ct], q + ((size_t)row[ct] * heads + head) * head_dim, head_dim, live[ct]);
+    }
+
+    const int first_pos = start + local0, last_pos = first_pos + wave_rows - 1;
+    const int wave_lo = window > 0 ? max(0, first_pos - window + 1) : 0;
+    for (int t0 = (wave_lo / 32) * 32; t0 <= last_pos; t0 += 32) tiles_step<NJ, ND, CT>(t, cv, t0, scale);
+
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        if (!live[ct]) continue;
+        const float inv = t[ct].l > 0.f ? 1.0f / t[ct].l : 0.f;
+        bf16_t* o = out + ((size_t)row[ct] * heads + head) * head_dim;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) {
+            uint2 packed;
+            packed.x = (uint32_t)f32_to_bf16(t[ct].acc[dt][0] * inv) | ((uint32_t)f32_to_bf16(t[ct].acc[dt][1] * inv) << 16);
+            packed.y = (uint32_t)f32_to_bf16(t[ct].acc[dt][2] * inv) | ((uint32_t)f32_to_bf16(t[ct].acc[dt][3] * inv) << 16);
+            *reinterpret_cast<uint2*>(o + dt * 16 + 4 * c) = packed;
+        }
+    }
+}
+
+// ------------------------------------------------- prefill through LDS --
+// The same work as attention_prefill_kernel, but the workgroup's four waves share
+// every block of KB keys: it is loaded once from the cache into LDS (the next
+// block's loads are in flight while the current one is computed) and each wave
+// takes its MFMA fragments from there.  Within a 32-key step, row 4c+i of score
+// tile u is the key 8c + 4u + i, so the 8 k-slots of lane group c in the output
+// MFMA are the 8 consecutive keys 8c..8c+7: one 16-byte read of a value row.
+// The head size is ND*16 at compile time.  Needs page_size >= 8.
+//
+// Keys past the end of a sequence's pages are read from page 0 instead (no
+// branches in the loads) and masked: the pools hold finite numbers only (they are
+// zero-initialised and written by kernels), so a masked weight of exactly 0 times
+// such a value is 0.
+template <int NJ, int ND, int CT, int KB>
+__device__ __forceinline__ void prefill_lds_block(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int* __restrict__ row_start,
+    const int* __restrict__ seq_start, int num_seqs, const int* __restrict__ tables, int table_width,
+    int page_size, int page_shift, int num_pages, int heads, int kv_heads, float scale_log2, int window,
+    int rq, int block) {
+    constexpr int HD = ND * 16;
+    constexpr int K_PITCH = HD + 8;                   // elements per key row in LDS
+    constexpr int V_PITCH = KB + 8;                   // elements per value (dim) row in LDS
+    constexpr int K_CHUNKS = KB * HD / 8, V_CHUNKS = HD * KB / 8;      // 16-byte chunks of a block
+    constexpr int MAXC = (K_CHUNKS + 255) / 256;
+    extern __shared__ uint4 lds_raw[];
+    bf16_t* ks = reinterpret_cast<bf16_t*>(lds_raw);  // [KB][K_PITCH]
+    bf16_t* vs = ks + KB * K_PITCH;                   // [HD][V_PITCH]
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
+    const int group = heads / kv_heads;
+    const int head_tiles = (group + 15) / 16;
+    const int kv_head = blockIdx.y / head_tiles, head_tile = blockIdx.y % head_tiles;
+    const int heads_here = min(16, group - head_tile * 16);
+    const int rows_per_wave = CT * rq, rows_per_block = 4 * rows_per_wave;
+    int seq = 0, first_row = 0, n_rows = 0;
+    for (; seq < num_seqs; ++seq) {
+        first_row = row_start[seq];
+        n_rows = row_start[seq + 1] - first_row;
+        const int blocks = (n_rows + rows_per_block - 1) / rows_per_block;
+        if (block < blocks) break;
+        block -= blocks;
+    }
+    if (seq >= num_seqs) return;                      // the whole workgroup leaves together
+    const int start = seq_start[seq];
+    const int block0 = block * rows_per_block;        // first row of the workgroup in the portion
+    const int block_rows = min(rows_per_block, n_rows - block0);
+    const int local0 = block0 + wave * rows_per_wave;
+    const int wave_rows = max(0, min(rows_per_wave, n_rows - local0));
+    const int col_row = r / heads_here, col_head = head_tile * 16 + r % heads_here;
+    const int head = kv_head * group + col_head;
+    const int* table = tables + (size_t)seq * table_width;
+
+    Tile<NJ, ND> t[CT];
+    bool live[CT];
+    int row[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int local = ct * rq + col_row;
+        live[ct] = col_row < rq && local < wave_rows;
+        row[ct] = first_row + (live[ct] ? local0 + local : 0);
+        const int pos = start + local0 + local;
+        tile_init(t[ct]);
+        t[ct].pos = live[ct] ? pos : -1;
+        t[ct].lo = live[ct] ? (window > 0 ? max(0, pos - window + 1) : 0) : 0;
+        tile_load_q(t[ct], q + ((size_t)row[ct] * heads + head) * HD, HD, live[ct]);
+    }
+    // keys the workgroup walks, and those this wave needs
+    const int wg_first = start + block0, wg_last = wg_first + block_rows - 1;
+    const int wg_lo = window > 0 ? max(0, wg_first - window + 1) : 0;
+    const int wave_first = start + local0, wave_last = wave_first + wave_rows - 1;
+    const int wave_lo = window > 0 ? max(0, wave_first - window + 1) : 0;
+    // every key in [full_lo, full_hi] is seen by every live column of this wave
+    const int full_lo = window > 0 ? max(0, wave_last - window + 1) : 0, full_hi = wave_first;
+
+    // staging plan of this thread: chunk e is key row (tid + 256 e) / (HD/8) of the block
+    // for keys, and dim row (tid + 256 e) / (KB/8) for values; fixed over the blocks
+    int k_key[MAXC], k_dch[MAXC], k_lds[MAXC], v_lds[MAXC];
+    size_t v_dim_off[MAXC];
+    const int v_g8 = tid % (KB / 8);                  // this thread's group of 8 keys in every value row
+    const size_t head_k = (size_t)kv_head * page_size * HD, page_k = (size_t)kv_heads * page_size * HD;
+    const size_t head_v = (size_t)kv_head * HD * page_size, page_v = (size_t)kv_heads * HD * page_size;
+#pragma unroll
+    for (int e = 0; e < MAXC; ++e) {
+        const int idx = tid + e * 256;
+        k_key[e] = idx / (HD / 8);
+        k_dch[e] = (idx % (HD / 8)) * 8;
+        k_lds[e] = k_key[e] * K_PITCH + k_dch[e];
+        const int d = idx / (KB / 8);
+        v_lds[e] = d * V_PITCH + v_g8 * 8;
+        v_dim_off[e] = (size_t)d * page_size;
+    }
+    uint4 kreg[MAXC], vreg[MAXC];
+    auto page_of = [&](int key) {
+        const int pidx = key >> page_shift;
+        int page = pidx < table_width ? table[pidx] : 0;
+        return (page < 0 || page >= num_pages) ? 0 : page;
+    };
+    auto fetch = [&](int t0) {
+        const int vkey = t0 + v_g8 * 8;
+        const bf16_t* vbase = v_cache + (size_t)page_of(vkey) * page_v + head_v + (vkey & (page_size - 1));
+#pragma unroll
+        for (int e = 0; e < MAXC; ++e) {
+            if (K_CHUNKS % 256 == 0 || tid + e * 256 < K_CHUNKS) {
+                const int key = t0 + k_key[e];
+                kreg[e] = *reinterpret_cast<const uint4*>(
+                    k_cache + (size_t)page_of(key) * page_k + head_k + (size_t)(key & (page_size - 1)) * HD + k_dch[e]);
+                vreg[e] = *reinterpret_cast<const uint4*>(vbase + v_dim_off[e]);
+            }
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int e = 0; e < MAXC; ++e) {
+            if (K_CHUNKS % 256 == 0 || tid + e * 256 < K_CHUNKS) {
+                *reinterpret_cast<uint4*>(ks + k_lds[e]) = kreg[e];
+                *reinterpret_cast<uint4*>(vs + v_lds[e]) = vreg[e];
+            }
+        }
+    };
+    static_assert(K_CHUNKS == V_CHUNKS, "keys and values of a block have as many chunks");
+
+    // LDS offsets of this lane's fragments inside a 32-key step
+    int ka_off[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) ka_off[u] = (8 * (r / 4) + 4 * u + (r % 4)) * K_PITCH + c * 8 * NJ;
+    const int vt_off = r * V_PITCH + 8 * c;
+
+    int t0 = (wg_lo / KB) * KB;
+    fetch(t0);
+    for (; t0 <= wg_last; t0 += KB) {
+        __syncthreads();                 // everyone has finished reading the previous block
+        stage();
+        __syncthreads();
+        if (t0 + KB <= wg_last) fetch(t0 + KB);
+#pragma unroll
+        for (int sub = 0; sub < KB / 32; ++sub) {
+            const int s0 = t0 + sub * 32;
+            if (wave_rows <= 0 || s0 > wave_last || s0 + 31 < wave_lo) continue;   // nothing this wave sees
+            Frag ka[2][NJ], vt[ND];
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    if (c * 8 * NJ + j * 8 < HD)
+                        ka[u][j].u = *reinterpret_cast<const uint4*>(ks + sub * 32 * K_PITCH + ka_off[u] + j * 8);
+                    else
+                        ka[u][j].u = make_uint4(0, 0, 0, 0);
+                }
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt)
+                vt[dt].u = *reinterpret_cast<const uint4*>(vs + dt * 16 * V_PITCH + vt_off + sub * 32);
+            if (s0 >= full_lo && s0 + 31 <= full_hi) {
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) tile_consume<NJ, ND, false>(t[ct], ka, vt, s0 + 8 * c, 4, scale_log2);
+            } else {
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) tile_consume<NJ, ND, true>(t[ct], ka, vt, s0 + 8 * c, 4, scale_log2);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        if (!live[ct]) continue;
+        const float inv = t[ct].l > 0.f ? 1.0f / t[ct].l : 0.f;
+        bf16_t* o = out + ((size_t)row[ct] * heads + head) * HD;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) {
+            uint2 packed;
+            packed.x = pack_bf16x2(t[ct].acc[dt][0] * inv, t[ct].acc[dt][1] * inv);
+            packed.y = pack_bf16x2(t[ct].acc[dt][2] * inv, t[ct].acc[dt][3] * inv);
+            *reinterpret_cast<uint2*>(o + dt * 16 + 4 * c) = packed;
+        }
+    }
+}
+
+// grid (row blocks, kv_heads * head_tiles), or with `pair` (ceil(row blocks / 2), ...):
+// row blocks late in a sequence walk more keys than early ones, so when there are
+// workgroups to spare each takes block (last - b) and then block b, and all do about
+// the same work.
+template <int NJ, int ND, int CT, int KB>
+__global__ void __launch_bounds__(256)
+attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
+                             const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+                             const int* __restrict__ row_start, const int* __restrict__ seq_start,
+                             int num_seqs, const int* __restrict__ tables, int table_width, int page_size,
+                             int page_shift, int num_pages, int heads, int kv_heads,
+                             float scale_log2, int window, int rq, int pair) {
+    const int rows_per_block = 4 * CT * rq;
+    int total = 0;
+    for (int seq = 0; seq < num_seqs; ++seq)
+        total += (row_start[seq + 1] - row_start[seq] + rows_per_block - 1) / rows_per_block;
+    const int first = blockIdx.x, second = pair ? total - 1 - first : first;
+    if (first >= total || first > second) return;
+    prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+                                      table_width, page_size, page_shift, num_pages, heads, kv_heads,
+                                      scale_log2, window, rq, second);
+    if (second != first) {
+        __syncthreads();
+        prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+                                          table_width, page_size, page_shift, num_pages, heads, kv_heads,
+                                          scale_log2, window, rq, first);
     }
 }
 
 // ------------------------------------------------------------------------ host --
+static const float LOG2E = 1.4426950408889634f;     // scores are kept in units of log2
+
 static int log2_exact(int v) {
     int s = 0;
     while ((1 << s) < v) ++s;
@@ -397,7 +653,7 @@ extern "C" int tli_attention_decode_bf16(
     attention_decode_kernel<NJ, ND><<<grid, 256, 3 * 64 * (ND * 4 + 2) * sizeof(float), s>>>(           \
         (const bf16_t*)q, (bf16_t*)out, partial, (const bf16_t*)k_cache, (const bf16_t*)v_cache,        \
         positions, seq_of_row, tables, table_width, page_size, shift, num_pages, heads, kv_heads,       \
-        head_dim, scale, window, splits, keys_per_split)
+        head_dim, scale * LOG2E, window, splits, keys_per_split)
     DISPATCH_HEAD_DIM(CALL)
 #undef CALL
     if (tli_check_launch("attention_decode")) return 1;
@@ -409,26 +665,55 @@ extern "C" int tli_attention_decode_bf16(
 }
 
 // Rows of a sequence are contiguous and ascend in position; row_start has num_seqs+1 entries.
+// direct = 1: every wave reads its keys and values straight from the cache (no LDS staging);
+// 0: through LDS, tiles per wave by shape; 2, 3: through LDS with one, two tiles per wave.
 extern "C" int tli_attention_prefill_bf16(
     const void* q, void* out, const void* k_cache, const void* v_cache, const int* row_start,
     const int* seq_start, int num_seqs, int rows, const int* tables, int table_width, int page_size,
-    int num_pages, int heads, int kv_heads, int head_dim, float scale, int window, void* stream) {
+    int num_pages, int heads, int kv_heads, int head_dim, float scale, int window, int direct,
+    void* stream) {
     if (rows <= 0 || num_seqs <= 0) return 0;
     if (check_common("attention_prefill", heads, kv_heads, head_dim, page_size, table_width, num_pages)) return 1;
     hipStream_t s = (hipStream_t)stream;
     const int group = heads / kv_heads, head_tiles = (group + 15) / 16;
     const int rq = group >= 16 ? 1 : 16 / group;
-    const int rows_per_block = 4 * rq;
-    const long blocks = (rows + rows_per_block - 1) / rows_per_block + num_seqs;   // upper bound
-    if (blocks > 2147483647L) return tli_fail("attention_prefill: too many rows");
-    dim3 grid((unsigned)blocks, kv_heads * head_tiles);
     const int shift = log2_exact(page_size);
-#define CALL(NJ, ND)                                                                                  \
-    attention_prefill_kernel<NJ, ND><<<grid, 256, 0, s>>>(                                            \
-        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, row_start,    \
-        seq_start, num_seqs, tables, table_width, page_size, shift, num_pages, heads, kv_heads,       \
-        head_dim, scale, window, rq)
-    DISPATCH_HEAD_DIM(CALL)
+    if (page_size >= 8 && direct != 1) {
+        // through LDS: two column tiles a wave for head sizes up to 128 when the portions are
+        // long enough to fill the chip that way; blocks of 64 keys (32 for large heads)
+        bool two = head_dim <= 128 && (long)rows * kv_heads * head_tiles >= (long)8 * rq * 512;
+        if (direct == 2) two = false;
+        if (direct == 3) two = head_dim <= 128;
+        const int rows_per_block = 4 * rq * (two ? 2 : 1);
+        const long blocks = (rows + rows_per_block - 1) / rows_per_block + num_seqs;   // upper bound
+        if (blocks > 2147483647L) return tli_fail("attention_prefill: too many rows");
+        const int pair = blocks * kv_heads * head_tiles >= 1024 ? 1 : 0;
+        dim3 grid((unsigned)(pair ? (blocks + 1) / 2 : blocks), kv_heads * head_tiles);
+        const int kb = head_dim <= 128 ? 64 : 32;
+        const size_t lds = ((size_t)kb * (head_dim + 8) + (size_t)head_dim * (kb + 8)) * sizeof(bf16_t);
+#define ARGS (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, row_start, \
+             seq_start, num_seqs, tables, table_width, page_size, shift, num_pages, heads, kv_heads
+#define TAIL scale * LOG2E, window, rq
+#define TAIL_LDS scale * LOG2E, window, rq, pair
+#define CALL(NJ, ND)                                                                                    \
+    if (ND <= 8 && two) attention_prefill_lds_kernel<NJ, (ND <= 8 ? ND : 1), 2, 64><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS); \
+    else if (ND <= 8) attention_prefill_lds_kernel<NJ, (ND <= 8 ? ND : 1), 1, 64><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS);   \
+    else attention_prefill_lds_kernel<NJ, ND, 1, 32><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS)
+        DISPATCH_HEAD_DIM(CALL)
 #undef CALL
+        return tli_check_launch("attention_prefill_lds");
+    }
+    {
+        const int rows_per_block = 4 * rq;
+        const long blocks = (rows + rows_per_block - 1) / rows_per_block + num_seqs;   // upper bound
+        if (blocks > 2147483647L) return tli_fail("attention_prefill: too many rows");
+        dim3 grid((unsigned)blocks, kv_heads * head_tiles);
+#define CALL(NJ, ND) attention_prefill_kernel<NJ, ND, 1><<<grid, 256, 0, s>>>(ARGS, head_dim, TAIL)
+        DISPATCH_HEAD_DIM(CALL)
+#undef CALL
+#undef ARGS
+#undef TAIL
+#undef TAIL_LDS
+    }
     return tli_check_launch("attention_prefill");
 }

@@ -20,12 +20,18 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
     return __uint_as_float(((uint32_t)v) << 16);
 }
 
-// round to nearest, ties to even; NaN stays NaN
+// round to nearest, ties to even (v_cvt_pk_bf16_f32 on gfx950)
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
+    const __bf16 b = (__bf16)f;
+    return *reinterpret_cast<const bf16_t*>(&b);
+}
+
+// two at once: low half = a, high half = b
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+    const bf16x2_t r = __builtin_convertvector((f32x2_t){a, b}, bf16x2_t);
+    return *reinterpret_cast<const uint32_t*>(&r);
 }
 
 __device__ __forceinline__ float to_f32(float v) { return v; }

@@ -172,6 +172,28 @@ extern "C" int tli_add_rmsnorm(float* resid, const void* delta, const float* wei
     return tli_check_launch("add_rmsnorm");
 }
 
+// 8 outputs a thread, 16-byte loads: inter % 8 == 0
+__global__ void swiglu_vec_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int inter,
+                                  size_t groups) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= groups) return;
+    const int per_row = inter / 8;
+    const size_t row = idx / per_row;
+    const int col = (int)(idx - row * per_row) * 8;
+    const uint4 g4 = *reinterpret_cast<const uint4*>(gu + row * 2 * inter + col);
+    const uint4 u4 = *reinterpret_cast<const uint4*>(gu + row * 2 * inter + inter + col);
+    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float g0 = bf16_to_f32((bf16_t)(gw[i] & 0xffffu)), g1 = bf16_to_f32((bf16_t)(gw[i] >> 16));
+        const float u0 = bf16_to_f32((bf16_t)(uw[i] & 0xffffu)), u1 = bf16_to_f32((bf16_t)(uw[i] >> 16));
+        const float a0 = g0 / (1.0f + expf(-g0)) * u0, a1 = g1 / (1.0f + expf(-g1)) * u1;
+        ow[i] = (uint32_t)f32_to_bf16(a0) | ((uint32_t)f32_to_bf16(a1) << 16);
+    }
+    *reinterpret_cast<uint4*>(out + row * inter + col) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 extern "C" int tli_swiglu(const void* gu, void* out, int rows, int inter, int dtype, void* stream) {
     if (rows <= 0) return 0;
     if (inter <= 0) return tli_fail("swiglu: bad size %d", inter);
@@ -180,7 +202,10 @@ extern "C" int tli_swiglu(const void* gu, void* out, int rows, int inter, int dt
     const unsigned blocks = (unsigned)((total + 255) / 256);
     if (dtype == TLI_F32)
         swiglu_kernel<float><<<blocks, 256, 0, s>>>((const float*)gu, (float*)out, inter, total);
-    else if (dtype == TLI_BF16)
+    else if (dtype == TLI_BF16 && inter % 8 == 0) {
+        const size_t groups = total / 8;
+        swiglu_vec_kernel<<<(unsigned)((groups + 255) / 256), 256, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, inter, groups);
+    } else if (dtype == TLI_BF16)
         swiglu_kernel<bf16_t><<<blocks, 256, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, inter, total);
     else
         return tli_fail("swiglu: unknown dtype %d", dtype);

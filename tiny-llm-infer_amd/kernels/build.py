@@ -24,6 +24,10 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={ARCH}",
          # packed float32 instructions are switched off for all device code
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         # MFMA accumulators stay in ordinary vector registers: the softmax rescales them
+         # with vector instructions, and copies to and from the accumulation registers
+         # cost more than the registers they save
+         "-mllvm", "-amdgpu-mfma-vgpr-form=1",
          "-Wno-unused-command-line-argument"]
 
 

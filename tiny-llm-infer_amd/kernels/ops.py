@@ -55,7 +55,7 @@ def load_library():
         "tli_gemm_plain": [P, P, P, I, I, I, I, I, I, P],
         "tli_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, I, P],
         "tli_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
-        "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, P],
+        "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P],
     }
     for name, args in sigs.items():
@@ -86,6 +86,7 @@ class HipOps:
             raise KernelError("no GPU is visible to torch; this engine has no CPU path")
         self.lib = load_library()
         self.force_plain = False     # tests: run the plain attention kernel for bfloat16 too
+        self.prefill_direct = 0      # tests: 1 = the prefill attention kernel without LDS staging; 2, 3 = with, 1 or 2 tiles a wave
         self.skinny_cfg = 0          # measurements: force a launch shape of the weight-streaming kernel
 
     # ---- helpers ----------------------------------------------------------
@@ -293,7 +294,8 @@ class HipOps:
             self._call(self.lib.tli_attention_prefill_bf16, q.data_ptr(), out.data_ptr(), kc.data_ptr(),
                        vc.data_ptr(), step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs,
                        T, g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], heads, kv_heads,
-                       head_dim, float(scale), int(window or 0), self._stream())
+                       head_dim, float(scale), int(window or 0), int(self.prefill_direct),
+                       self._stream())
             return out
         self._call(self.lib.tli_attention_plain, q.data_ptr(), out.data_ptr(), kc.data_ptr(),
                    vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
@@ -307,7 +309,8 @@ class HipOps:
         T = step.num_rows
         reach = step.reach if not window else min(step.reach, (window + 31) // 32 * 32 + 32)
         groups = T * kv_heads * ((heads // kv_heads + 15) // 16)
-        splits = max(1, min((self.DECODE_WORKGROUPS + groups - 1) // groups, (reach + 127) // 128, 64))
+        # a split costs a merge pass: only worth it when a workgroup would walk many keys
+        splits = max(1, min((self.DECODE_WORKGROUPS + groups - 1) // groups, reach // 512, 64))
         per_split = ((reach + splits - 1) // splits + 127) // 128 * 128
         splits = (reach + per_split - 1) // per_split
         partial = None
