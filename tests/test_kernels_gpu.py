@@ -118,12 +118,26 @@ def test_skinny_linear_against_plain_kernel_and_reference(ops, mnk, out):
     xd, wd = x.to(DEV), w.to(DEV)
     got = ops.linear(xd, wd, out_dtype=out)
     plain = ops.linear_plain(xd, wd, out_dtype=out)
+    want = x.double() @ w.double().t()
+    scale = float(want.abs().max())
+    # float32 out: only the order of the float32 additions differs
+    bound = 2e-5 * scale * (K ** 0.5) / 8 + 1e-6 if out == torch.float32 else 1.2e-2 * scale
 
     class Both:                      # the matrix with its decode layout, as the parts hold it
         w = wd
         tiled = ops.tile_matrix(wd)
     streamed = ops.linear(xd, Both, out_dtype=out)
-    assert torch.equal(streamed, got)          # same additions in the same order, other addresses
+    if M < ops.MID_ROWS_FROM:
+        assert torch.equal(streamed, got)      # same additions in the same order, other addresses
+    else:                                      # 17..64 rows: the kernel that shares x through LDS
+        assert float((streamed.double().cpu() - want).abs().max()) <= bound
+        for splits, cfg in ((1, 24), (2, 28), (4, 44), (3, 48)):
+            ops.mid_splits, ops.mid_cfg = splits, cfg
+            try:
+                again = ops.linear(xd, Both, out_dtype=out)
+            finally:
+                ops.mid_splits = ops.mid_cfg = 0
+            assert float((again.double().cpu() - want).abs().max()) <= bound, (splits, cfg)
     want = x.double() @ w.double().t()
     scale = float(want.abs().max())
     # float32 out: only the order of the float32 additions differs

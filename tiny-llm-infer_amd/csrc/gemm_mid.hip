@@ -1,0 +1,253 @@
+// Matrix product for 17..64 rows (a large decode batch): y[M,N] = x[M,K] . W^T with W in
+// the decode layout (see gemm_skinny.hip).  Still bound by streaming W once, but with
+// four 16-row tiles of x every W fragment meets four x fragments, and taking those
+// from L2 for every wave (as the kernel for <= 16 rows does) would cost four times
+// the traffic of W itself.  Here the waves of a workgroup own different output
+// columns and walk k together: each 128-wide slice of x (64 rows, 16 KiB) is staged
+// once in LDS and shared by all of them.
+//
+// A workgroup owns 16*RT*WAVES output columns and one of `splits` contiguous ranges
+// of k.  With splits > 1 it writes float32 partial sums [split][M][N] and a second
+// small kernel adds them in split order (and applies the SwiGLU epilogue for a gated
+// matrix), so the result does not depend on timing.
+#include "common.h"
+#include <type_traits>
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+union Pack16m {
+    uint4 u;
+    bf16x8 v;
+};
+
+#define MID_ROWS 64
+#define MID_XPITCH (128 + 8)        // elements per staged x row: 272 bytes
+
+template <int RT, int WAVES, typename TO, bool GATED>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* __restrict__ y,
+                float* __restrict__ part, int M, int N, int K, int splits, int steps_per_split) {
+    __shared__ __attribute__((aligned(16))) bf16_t xs[2][MID_ROWS][MID_XPITCH];
+    constexpr int THREADS = WAVES * 64;
+    constexpr int CHUNKS = MID_ROWS * 16 / THREADS;          // 16-byte chunks of a slice a thread stages
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
+    const int k_steps = (K + 127) / 128;
+    const int tile0 = (blockIdx.x * WAVES + wave) * RT;       // this wave's first 16-column tile
+    const int n_tiles = (N + 15) / 16;
+    const int step_begin = blockIdx.y * steps_per_split;
+    const int step_end = min(k_steps, step_begin + steps_per_split);
+
+    f32x4 acc[RT][4];
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[t][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    // W fragments straight from the decode layout: block (tile, step) is 2048 elements,
+    // fragment j of this lane at j*512 + lane*8
+    const bf16_t* w_tile[RT];
+    bool w_ok[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        w_ok[t] = tile0 + t < n_tiles;
+        w_tile[t] = w + (size_t)(w_ok[t] ? tile0 + t : 0) * k_steps * 2048 + lane * 8;
+    }
+    // Three register stages for the fetched W fragments and x chunks (two fetches are in
+    // flight while a slice is multiplied), two LDS buffers for the staged x slices.
+    // x staging plan: chunk e of this thread is row (tid + e*THREADS) / 16, 16-byte column (..) % 16
+    Pack16m a[3][RT][4];
+    uint4 xreg[3][CHUNKS];
+    auto fetch = [&](int step, auto STAGE) {
+        constexpr int S = decltype(STAGE)::value;
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                a[S][t][j].u = w_ok[t] ? *reinterpret_cast<const uint4*>(w_tile[t] + (size_t)step * 2048 + j * 512)
+                                       : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int e = 0; e < CHUNKS; ++e) {
+            const int idx = tid + e * THREADS;
+            const int row = idx / 16, k = step * 128 + (idx % 16) * 8;
+            xreg[S][e] = (row < M && k < K) ? *reinterpret_cast<const uint4*>(x + (size_t)row * K + k)
+                                            : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto stage = [&](int buf, auto STAGE) {
+        constexpr int S = decltype(STAGE)::value;
+#pragma unroll
+        for (int e = 0; e < CHUNKS; ++e) {
+            const int idx = tid + e * THREADS;
+            *reinterpret_cast<uint4*>(&xs[buf][idx / 16][(idx % 16) * 8]) = xreg[S][e];
+        }
+    };
+    // one slice: `step` is multiplied from register stage S and LDS buffer `buf`
+    auto slice = [&](int step, int buf, auto STAGE) {
+        constexpr int S = decltype(STAGE)::value;
+        __syncthreads();                                   // slice `buf` is staged; the other is free
+        if (step + 2 < step_end) fetch(step + 2, std::integral_constant<int, (S + 2) % 3>{});
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            Pack16m b[4];
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+                b[m].u = *reinterpret_cast<const uint4*>(&xs[buf][m * 16 + r][c * 32 + j * 8]);
+#pragma unroll
+            for (int t = 0; t < RT; ++t)
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+                    acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[S][t][j].v, b[m].v, acc[t][m], 0, 0, 0);
+        }
+        // nobody reads the other buffer before the next barrier
+        if (step + 1 < step_end) stage(buf ^ 1, std::integral_constant<int, (S + 1) % 3>{});
+    };
+
+    if (step_begin < step_end) {
+        fetch(step_begin, std::integral_constant<int, 0>{});
+        if (step_begin + 1 < step_end) fetch(step_begin + 1, std::integral_constant<int, 1>{});
+        stage(0, std::integral_constant<int, 0>{});
+    }
+    for (int step = step_begin; step < step_end; step += 3) {
+        const int b0 = (step - step_begin) & 1;
+        slice(step, b0, std::integral_constant<int, 0>{});
+        if (step + 1 < step_end) slice(step + 1, b0 ^ 1, std::integral_constant<int, 1>{});
+        if (step + 2 < step_end) slice(step + 2, b0, std::integral_constant<int, 2>{});
+    }
+
+    // lane holds y[m*16 + r][tile*16 + 4c + i]
+    if (splits > 1) {
+        float* dst = part + (size_t)blockIdx.y * M * N;
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            const int n0 = (tile0 + t) * 16 + 4 * c;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const int row = m * 16 + r;
+                if (row >= M) continue;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n0 + i < N) dst[(size_t)row * N + n0 + i] = acc[t][m][i];
+            }
+        }
+        return;
+    }
+    if (GATED) {
+        const int n_out = N / 2;
+#pragma unroll
+        for (int t = 0; t + 1 < RT; t += 2) {
+            const int n0 = ((tile0 + t) / 2) * 16 + 4 * c;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const int row = m * 16 + r;
+                if (row >= M) continue;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n0 + i < n_out) {
+                        const float g = acc[t][m][i], u = acc[t + 1][m][i];
+                        from_f32(y + (size_t)row * n_out + n0 + i, g / (1.0f + expf(-g)) * u);
+                    }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        const int n0 = (tile0 + t) * 16 + 4 * c;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            const int row = m * 16 + r;
+            if (row >= M) continue;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (n0 + i < N) from_f32(y + (size_t)row * N + n0 + i, acc[t][m][i]);
+        }
+    }
+}
+
+// Sum of the partial products in split order.  gated: output column j of [M, N/2] takes
+// gate column (j/16)*32 + j%16 and up column 16 further.
+template <typename TO>
+__global__ void gemm_mid_reduce_kernel(const float* __restrict__ part, TO* __restrict__ y, int M, int N,
+                                       int splits, int gated) {
+    const int n_out = gated ? N / 2 : N;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)M * n_out) return;
+    const int row = (int)(idx / n_out), j = (int)(idx % n_out);
+    const size_t plane = (size_t)M * N;
+    if (gated) {
+        const size_t gcol = (size_t)(j / 16) * 32 + j % 16;
+        float g = 0.f, u = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            g += part[s * plane + (size_t)row * N + gcol];
+            u += part[s * plane + (size_t)row * N + gcol + 16];
+        }
+        from_f32(y + idx, g / (1.0f + expf(-g)) * u);
+    } else {
+        float v = 0.f;
+        for (int s = 0; s < splits; ++s) v += part[s * plane + (size_t)row * N + j];
+        from_f32(y + idx, v);
+    }
+}
+
+template <int RT, int WAVES>
+static int launch_mid(const bf16_t* x, const bf16_t* w, void* y, float* part, int M, int N, int K,
+                      int y_dtype, int gated, int splits, hipStream_t s) {
+    const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
+    const int steps_per_split = (k_steps + splits - 1) / splits;
+    dim3 grid((n_tiles + RT * WAVES - 1) / (RT * WAVES), splits);
+    if (gated)
+        gemm_mid_kernel<RT, WAVES, bf16_t, true><<<grid, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, part, M, N, K, splits, steps_per_split);
+    else if (y_dtype == TLI_BF16)
+        gemm_mid_kernel<RT, WAVES, bf16_t, false><<<grid, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, part, M, N, K, splits, steps_per_split);
+    else
+        gemm_mid_kernel<RT, WAVES, float, false><<<grid, WAVES * 64, 0, s>>>(x, w, (float*)y, part, M, N, K, splits, steps_per_split);
+    if (tli_check_launch("gemm_mid")) return 1;
+    if (splits > 1) {
+        const size_t total = (size_t)M * (gated ? N / 2 : N);
+        const unsigned blocks = (unsigned)((total + 255) / 256);
+        if (y_dtype == TLI_BF16)
+            gemm_mid_reduce_kernel<bf16_t><<<blocks, 256, 0, s>>>(part, (bf16_t*)y, M, N, splits, gated);
+        else
+            gemm_mid_reduce_kernel<float><<<blocks, 256, 0, s>>>(part, (float*)y, M, N, splits, gated);
+        return tli_check_launch("gemm_mid_reduce");
+    }
+    return 0;
+}
+
+// How many ranges of k a product of this shape is cut into (the caller sizes `part` by it).
+extern "C" int tli_gemm_mid_splits(int N, int K) {
+    const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
+    const int groups = (n_tiles + 7) / 8;                 // workgroups with RT = 2, WAVES = 4
+    int splits = 1;
+    while (groups * splits < 192 && splits * 2 <= k_steps && splits < 16) splits *= 2;
+    return splits;
+}
+
+// y[M,N] = x[M,K] . W^T for 1 <= M <= 64, W in the decode layout (`gated` as tiled = 2 of
+// tli_gemm_skinny_bf16: y is [M, N/2] bfloat16).  `part`: splits*M*N floats when
+// splits > 1 (splits as returned by tli_gemm_mid_splits, or forced by the caller);
+// cfg 0 picks the launch shape, else RT*10 + WAVES.
+extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* part, int M, int N, int K,
+                                 int y_dtype, int gated, int splits, int cfg, void* stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > MID_ROWS) return tli_fail("gemm_mid: %d rows, at most %d", M, MID_ROWS);
+    if (K <= 0 || K % 8) return tli_fail("gemm_mid: K = %d must be a positive multiple of 8", K);
+    if (y_dtype != TLI_BF16 && y_dtype != TLI_F32) return tli_fail("gemm_mid: bad output dtype %d", y_dtype);
+    if (gated && (N % 32 || y_dtype != TLI_BF16))
+        return tli_fail("gemm_mid: a gated product needs N %% 32 == 0 and bfloat16 output");
+    if (splits < 1 || splits > 64) return tli_fail("gemm_mid: %d splits", splits);
+    if (splits > 1 && !part) return tli_fail("gemm_mid: splits need a buffer for partial sums");
+    if (((uintptr_t)x | (uintptr_t)w) & 15) return tli_fail("gemm_mid: operands must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    const bf16_t* xp = (const bf16_t*)x;
+    const bf16_t* wp = (const bf16_t*)w;
+    if (cfg == 0) cfg = 24;
+    switch (cfg) {
+        case 24: return launch_mid<2, 4>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
+        case 28: return launch_mid<2, 8>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
+        case 44: return launch_mid<4, 4>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
+        case 48: return launch_mid<4, 8>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
+        default: return tli_fail("gemm_mid: unknown configuration %d", cfg);
+    }
+}

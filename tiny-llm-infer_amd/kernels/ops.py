@@ -54,6 +54,8 @@ def load_library():
         "tli_attention_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
         "tli_gemm_plain": [P, P, P, I, I, I, I, I, I, P],
         "tli_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, I, P],
+        "tli_gemm_mid_bf16": [P, P, P, P, I, I, I, I, I, I, I, P],
+        "tli_gemm_mid_splits": [I, I],
         "tli_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
         "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P],
@@ -76,6 +78,7 @@ class HipOps:
     name = "hip-gfx950"
     MAX_HEAD_DIM = 512
     SKINNY_ROWS = 64
+    MID_ROWS_FROM = 17           # from this many rows the x-sharing kernel multiplies
     DECODE_WORKGROUPS = 512      # aim of the decode attention's key splitting
 
     def __init__(self, device):
@@ -87,6 +90,8 @@ class HipOps:
         self.lib = load_library()
         self.force_plain = False     # tests: run the plain attention kernel for bfloat16 too
         self.prefill_direct = 0      # tests: 1 = the prefill attention kernel without LDS staging; 2, 3 = with, 1 or 2 tiles a wave
+        self.mid_cfg = 0             # measurements: launch shape and k ranges of the 17..64-row kernel
+        self.mid_splits = 0
         self.skinny_cfg = 0          # measurements: force a launch shape of the weight-streaming kernel
 
     # ---- helpers ----------------------------------------------------------
@@ -187,6 +192,8 @@ class HipOps:
             if M <= self.SKINNY_ROWS or out_dtype == torch.float32:
                 # few rows (decode), or float32 logits: the weight-streaming MFMA kernel,
                 # 64 rows at a time
+                if tiled is not None and self.MID_ROWS_FROM <= M <= self.SKINNY_ROWS:
+                    return self._linear_mid(x, tiled, y, M, N, K, 0)
                 wp = w if tiled is None else tiled
                 for m0 in range(0, M, self.SKINNY_ROWS):
                     m1 = min(M, m0 + self.SKINNY_ROWS)
@@ -200,6 +207,17 @@ class HipOps:
             return y
         self._call(self.lib.tli_gemm_plain, x.data_ptr(), w.data_ptr(), y.data_ptr(), M, N, K,
                    _dtype_code(x.dtype), _dtype_code(w.dtype), _dtype_code(out_dtype), self._stream())
+        return y
+
+    def _linear_mid(self, x, tiled, y, M, N, K, gated):
+        """17..64 rows: the kernel that shares x through LDS, k cut into ranges when the
+        output alone gives too few workgroups."""
+        splits = self.mid_splits or self.lib.tli_gemm_mid_splits(N, K)
+        part = None
+        if splits > 1:
+            part = torch.empty((splits * M * N,), dtype=torch.float32, device=self.device)
+        self._call(self.lib.tli_gemm_mid_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), _ptr(part),
+                   M, N, K, _dtype_code(y.dtype), gated, splits, self.mid_cfg, self._stream())
         return y
 
     def linear_plain(self, x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
@@ -223,6 +241,8 @@ class HipOps:
         if gated is not None and 0 < M <= self.SKINNY_ROWS and x.dtype == torch.bfloat16:
             self._want(x, "linear input", torch.bfloat16, (M, m.w.shape[1]))
             y = torch.empty((M, m.inter), dtype=x.dtype, device=self.device)
+            if M >= self.MID_ROWS_FROM:
+                return self._linear_mid(x, gated, y, M, 2 * m.inter, K, 1)
             self._call(self.lib.tli_gemm_skinny_bf16, x.data_ptr(), gated.data_ptr(), y.data_ptr(), M,
                        2 * m.inter, K, BF16, 2, self.skinny_cfg if self.skinny_cfg >= 20 else 0, self._stream())
             return y
