@@ -245,3 +245,55 @@ def test_a_prompt_larger_than_the_pool_is_an_error_and_a_stuck_queue_too():
     s.add(_seq(1, 5))
     with pytest.raises(SchedulerError, match="could not make progress"):
         s.schedule()
+
+
+# ------------------------------------------------------------ prefix caching --
+def test_page_hash_is_chained_fnv1a():
+    from tiny_llm_infer_amd.cache.manager import page_hash
+    # FNV-1a, 64 bit, over 8 bytes of the previous hash then 4 bytes per token, little-endian
+    h = 1469598103934665603
+    for byte in [0] * 8 + [7, 0, 0, 0, 1, 1, 0, 0]:
+        h = ((h ^ byte) * 1099511628211) % (1 << 64)
+    assert page_hash([7, 257], 0) == h
+    assert page_hash([7, 257], 1) != h and page_hash([257, 7], 0) != h
+
+
+def test_prefix_pages_are_shared_revived_and_forgotten():
+    m = CacheManager([FULL, FULL], page_size=4, num_pages=8, max_requests=3, prefix_caching=True)
+    a = list(range(100, 111))                     # 11 tokens: 2 full pages + 3
+    m.admit("a")
+    assert m.adopt_prefix("a", a) == 0
+    m.reserve("a", 11)
+    m.advance("a", 11)
+    m.register_pages("a", a)
+    # b shares a's first two pages while a is live; its third page is its own
+    b = a[:8] + [1, 2, 3]
+    m.admit("b")
+    assert m.adopt_prefix("b", b) == 8
+    assert m.get("b").tables[0] == m.get("a").tables[0][:2]
+    assert m.groups[0].pool.ref_count(m.get("a").tables[0][0]) == 2
+    m.reserve("b", 11)
+    assert m.get("b").tables[0][2] != m.get("a").tables[0][2]
+    m.advance("b", 11)
+    m.check()
+    # never the last page: a prompt of exactly 8 tokens still computes its second page
+    m.admit("c")
+    assert m.adopt_prefix("c", a[:8]) == 4
+    m.release("c")
+    m.release("a")
+    m.release("b")
+    assert m.free_pages() == [8]
+    # free pages are revived by id ...
+    m.admit("d")
+    assert m.adopt_prefix("d", a) == 8 and m.prefix_hits == 2 + 1 + 2
+    m.release("d")
+    # ... until the pool hands them out for something else
+    m.admit("e")
+    m.reserve("e", 32)
+    m.release("e")
+    m.admit("f")
+    assert m.adopt_prefix("f", a) == 0
+    m.release("f")
+    m.check()
+    with pytest.raises(ValueError):
+        CacheManager([FULL, WIN], page_size=4, num_pages=8, max_requests=1, prefix_caching=True)

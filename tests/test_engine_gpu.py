@@ -178,3 +178,21 @@ def test_recorded_decode_steps_equal_eager_ones(model_folders):
                 slow.release(k)
                 del live[k]
     assert compared > 30 and fast.graph_replays == compared and len(fast.graphs) >= 3
+
+
+def test_prefix_caching_on_the_gpu(model_folders):
+    """Requests that share a prompt prefix take its pages over instead of computing
+    them; the tokens are those of an engine without the cache."""
+    from tiny_llm_infer_amd.sampling.params import SamplingParams
+    folder = model_folders["A"]
+    shared = random_prompt(256, 40, 9)
+    prompts = [shared + random_prompt(256, n, 20 + n) for n in (3, 9, 1)] + [shared[:33]]
+    params = SamplingParams(max_tokens=6, ignore_eos=True)
+    for dtype in ("float32", "bfloat16"):
+        plain = _engine(folder, "A", dtype).generate(prompts, params)
+        eng = _engine(folder, "A", dtype, enable_prefix_caching=True, max_num_seqs=1)
+        got = eng.generate(prompts, params)
+        if dtype == "float32":
+            assert [r.token_ids for r in got] == [r.token_ids for r in plain]
+        assert eng.runner.cache.prefix_hits == 14
+        eng.runner.cache.check()

@@ -82,3 +82,22 @@ def test_temperature_tokens_do_not_depend_on_the_batch(model_folders):
     assert [r.token_ids for r in together] == [r.token_ids for r in alone]
     greedy = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
     assert [r.token_ids for r in greedy] != [r.token_ids for r in together]
+
+
+def test_prefix_caching_gives_the_same_tokens_and_skips_work(model_folders):
+    folder = model_folders["A"]
+    shared = random_prompt(256, 40, 9)
+    prompts = [shared + random_prompt(256, n, 20 + n) for n in (3, 9, 1)] + [shared[:33]]
+    params = SamplingParams(max_tokens=6, ignore_eos=True)
+    plain = _engine(folder, "A").generate(prompts, params)
+    eng = _engine(folder, "A", enable_prefix_caching=True, max_num_seqs=1)    # one after the other
+    got = eng.generate(prompts, params)
+    assert [r.token_ids for r in got] == [r.token_ids for r in plain]
+    assert eng.runner.cache.prefix_hits == 2 * 5 + 4      # 40 shared tokens = 5 pages of 8; the first request finds none
+    eng.runner.cache.check()
+    # and together, under preemption
+    small = _engine(folder, "A", enable_prefix_caching=True, num_kv_blocks=14)
+    got = small.generate(prompts, params)
+    assert [r.token_ids for r in got] == [r.token_ids for r in plain]
+    small.runner.cache.check()
+    assert small.runner.cache.free_pages() == [14]

@@ -10,6 +10,18 @@ window of all tokens still to come; every group gives all of a request's pages
 back when the request ends.  (The reference has one group and no window:
 model/src/qwen3_kv_cache.cpp:14-44, engine/src/block_manager.cpp.)
 
+Prefix caching (off unless asked for; the reference's block manager does the same,
+engine/src/block_manager.cpp:24-64, 184-224): every full page gets a hash chained
+over the hashes of the pages before it and its own token ids (FNV-1a, 64 bit).  A
+new request whose leading full pages (all but its last page, so that at least one
+token is always computed) are known takes those pages instead of computing them:
+a page that is still held is shared (its reference count goes up), a page that is
+free but not yet handed out again is revived.  A page leaves the cache when the
+pool hands it out for something else.  Shared pages are never written: the tokens
+of a shared prefix are not run again.  It is available only when every group keeps
+all keys and no mixer keeps state, because a passed window page or a state cannot
+be taken over.
+
 Page layout on the device: keys ``[cache layer in group, page, kv head, slot,
 head_dim]``, values ``[cache layer in group, page, kv head, head_dim, slot]``, so
 that one head's part of a page is contiguous and each matrix-core operand is
@@ -60,6 +72,8 @@ class RequestCache:
     key: Hashable
     slot: int
     num_tokens: int = 0                               # tokens whose keys are in the cache
+    hashed_blocks: int = 0                            # leading pages already in the prefix cache
+    prefix_hash: int = 0                              # chained hash of those pages
     tables: List[List[int]] = field(default_factory=list)   # per group: block -> page or -1
     reserved_tokens: int = 0                          # positions [0, reserved) are covered
 
@@ -68,9 +82,27 @@ def _blocks(tokens: int, page: int) -> int:
     return (tokens + page - 1) // page
 
 
+_FNV_OFFSET = 1469598103934665603
+_FNV_PRIME = 1099511628211
+_MASK64 = (1 << 64) - 1
+
+
+def page_hash(tokens: Sequence[int], prefix_hash: int) -> int:
+    """FNV-1a over the 8 bytes of the previous page's hash, then the 4 bytes of
+    each token id, little-endian (engine/src/block_manager.cpp:24-43)."""
+    h = _FNV_OFFSET
+    for shift in range(0, 64, 8):
+        h = ((h ^ ((prefix_hash >> shift) & 0xFF)) * _FNV_PRIME) & _MASK64
+    for t in tokens:
+        v = int(t) & 0xFFFFFFFF
+        for shift in range(0, 32, 8):
+            h = ((h ^ ((v >> shift) & 0xFF)) * _FNV_PRIME) & _MASK64
+    return h
+
+
 class CacheManager:
     def __init__(self, needs: Sequence[Optional[CacheNeed]], page_size: int, num_pages: int,
-                 max_requests: int):
+                 max_requests: int, prefix_caching: bool = False):
         """``needs[i]`` is the need of cache layer i (None: that layer keeps nothing).
         Every group gets ``num_pages`` pages of ``page_size`` slots."""
         if page_size <= 0 or num_pages <= 0 or max_requests <= 0:
@@ -95,6 +127,13 @@ class CacheManager:
         self._live: Dict[Hashable, RequestCache] = {}
         self.pages_taken_total = 0
         self.pages_returned_total = 0
+        if prefix_caching and any(g.need.window is not None for g in self.groups):
+            raise ValueError("prefix caching needs every layer to keep all keys (no window)")
+        self.prefix_caching = prefix_caching
+        # per group: hash -> page, and per page its (hash, token ids) while it is in the cache
+        self._page_of_hash: List[Dict[int, int]] = [dict() for _ in self.groups]
+        self._known: List[Dict[int, Tuple[int, Tuple[int, ...]]]] = [dict() for _ in self.groups]
+        self.prefix_hits = 0                # pages taken over instead of computed
 
     # ---- requests -------------------------------------------------------
     def live(self) -> List[Hashable]:
@@ -119,6 +158,88 @@ class CacheManager:
         rc = RequestCache(key=key, slot=slot, tables=[[] for _ in self.groups])
         self._live[key] = rc
         return rc
+
+    # ---- prefix cache ---------------------------------------------------
+    def _take(self, gi: int) -> int:
+        """A fresh page of group gi; what the prefix cache knew of it is forgotten."""
+        page = self.groups[gi].pool.take()
+        known = self._known[gi].pop(page, None)
+        if known is not None and self._page_of_hash[gi].get(known[0]) == page:
+            del self._page_of_hash[gi][known[0]]
+        self.pages_taken_total += 1
+        return page
+
+    def match_prefix(self, tokens: Sequence[int]) -> List[List[int]]:
+        """Pages (per group) that hold the leading full pages of ``tokens``: as many
+        as every group knows, never the last page of the sequence."""
+        if not self.prefix_caching or not self.groups:
+            return [[] for _ in self.groups]
+        out: List[List[int]] = [[] for _ in self.groups]
+        prefix = 0
+        nb = _blocks(len(tokens), self.page_size)
+        for b in range(nb - 1):
+            chunk = tuple(int(t) for t in tokens[b * self.page_size:(b + 1) * self.page_size])
+            if len(chunk) != self.page_size:
+                break
+            prefix = page_hash(chunk, prefix)
+            found = []
+            for gi in range(len(self.groups)):
+                page = self._page_of_hash[gi].get(prefix)
+                known = None if page is None else self._known[gi].get(page)
+                if known is None or known[0] != prefix or known[1] != chunk:   # collision check
+                    found = None
+                    break
+                found.append(page)
+            if found is None:
+                break
+            for gi, page in enumerate(found):
+                out[gi].append(page)
+        return out
+
+    def adopt_prefix(self, key: Hashable, tokens: Sequence[int]) -> int:
+        """Give a just admitted request the cached pages of its prefix; returns how
+        many tokens need not be computed."""
+        rc = self._live[key]
+        if rc.num_tokens or any(rc.tables):
+            raise ValueError("a prefix can only be adopted by a request that holds nothing")
+        matched = self.match_prefix(tokens)
+        n = len(matched[0]) if matched else 0
+        for gi, pages in enumerate(matched):
+            pool = self.groups[gi].pool
+            for page in pages:
+                if pool.is_free(page):
+                    pool.revive(page)
+                    self.pages_taken_total += 1
+                else:
+                    pool.share(page)
+                rc.tables[gi].append(page)
+        rc.num_tokens = n * self.page_size
+        rc.reserved_tokens = rc.num_tokens
+        rc.hashed_blocks = n
+        rc.prefix_hash = 0
+        for b in range(n):
+            rc.prefix_hash = page_hash(tokens[b * self.page_size:(b + 1) * self.page_size], rc.prefix_hash)
+        self.prefix_hits += n
+        return rc.num_tokens
+
+    def register_pages(self, key: Hashable, tokens: Sequence[int]) -> None:
+        """After a step: the request's newly completed full pages enter the cache
+        (engine/src/block_manager.cpp:184-224).  ``tokens`` are all its tokens."""
+        if not self.prefix_caching:
+            return
+        rc = self._live[key]
+        full = min(rc.num_tokens, len(tokens)) // self.page_size
+        for b in range(rc.hashed_blocks, full):
+            chunk = tuple(int(t) for t in tokens[b * self.page_size:(b + 1) * self.page_size])
+            rc.prefix_hash = page_hash(chunk, rc.prefix_hash)
+            for gi in range(len(self.groups)):
+                page = rc.tables[gi][b]
+                old = self._known[gi].pop(page, None)
+                if old is not None and self._page_of_hash[gi].get(old[0]) == page:
+                    del self._page_of_hash[gi][old[0]]
+                self._known[gi][page] = (rc.prefix_hash, chunk)
+                self._page_of_hash[gi][rc.prefix_hash] = page
+        rc.hashed_blocks = max(rc.hashed_blocks, full)
 
     # ---- pages ----------------------------------------------------------
     def _first_needed_block(self, g: GroupLayout, first_query_pos: int) -> int:
@@ -163,8 +284,7 @@ class CacheManager:
             first = self._first_needed_block(g, rc.num_tokens)
             for b in range(first, nb):
                 if table[b] < 0:
-                    table[b] = g.pool.take()
-                    self.pages_taken_total += 1
+                    table[b] = self._take(gi)
         rc.reserved_tokens = max(rc.reserved_tokens, new_total)
 
     def advance(self, key: Hashable, new_total: int) -> None:

@@ -30,6 +30,8 @@ def _common(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--max-num-batched-tokens", type=int, default=None)
     ap.add_argument("--max-num-seqs", type=int, default=None)
+    ap.add_argument("--enable-prefix-caching", action="store_true",
+                    help="take over cached full pages of a known prompt prefix instead of computing them")
     ap.add_argument("--random-weights", action="store_true",
                     help="with --config: draw seeded random weights instead of reading a checkpoint")
     ap.add_argument("--config", help="a config.json, for --random-weights")
@@ -109,7 +111,7 @@ def run_inference(argv: List[str]) -> int:
         num_kv_blocks=args.num_kv_blocks,
         max_num_seqs=args.max_num_seqs or min(16, len(prompts)),
         max_num_batched_tokens=args.max_num_batched_tokens or min(max_seq_len, 256),
-        gpu_memory_utilization=util)
+        gpu_memory_utilization=util, enable_prefix_caching=args.enable_prefix_caching)
     if args.eos_id is not None:
         engine.eos_token_ids = set(args.eos_id)
     print(f"Preallocating {engine.runner.cache.num_pages} KV blocks "
@@ -173,7 +175,7 @@ def run_benchmark(argv: List[str]) -> int:
         model, max_model_len=max_seq_len, page_size=page, num_kv_blocks=blocks,
         max_num_seqs=args.max_num_seqs or args.num_seqs,
         max_num_batched_tokens=args.max_num_batched_tokens or min(max_seq_len, 256),
-        gpu_memory_utilization=util)
+        gpu_memory_utilization=util, enable_prefix_caching=args.enable_prefix_caching)
     vocab = model.spec.vocab_size
     import torch
     rates, total_tokens, total_time = [], 0, 0.0

@@ -47,18 +47,19 @@ class LLMEngine:
     def from_folder(cls, model_dir: str, dtype="bfloat16", device="cuda:0", max_model_len: int = 2048,
                     page_size: int = 16, num_kv_blocks: int = 0, max_num_seqs: int = 16,
                     max_num_batched_tokens: int = 256, gpu_memory_utilization: float = 0.9,
-                    ops=None) -> "LLMEngine":
+                    enable_prefix_caching: bool = False, ops=None) -> "LLMEngine":
         from .loading import load_model
         model, cfg = load_model(model_dir, dtype, device, max_model_len, ops)
         return cls.from_model(model, max_model_len=max_model_len, page_size=page_size,
                               num_kv_blocks=num_kv_blocks, max_num_seqs=max_num_seqs,
                               max_num_batched_tokens=max_num_batched_tokens,
-                              gpu_memory_utilization=gpu_memory_utilization)
+                              gpu_memory_utilization=gpu_memory_utilization,
+                              enable_prefix_caching=enable_prefix_caching)
 
     @classmethod
     def from_model(cls, model, max_model_len: int = 2048, page_size: int = 16, num_kv_blocks: int = 0,
                    max_num_seqs: int = 16, max_num_batched_tokens: int = 256,
-                   gpu_memory_utilization: float = 0.9) -> "LLMEngine":
+                   gpu_memory_utilization: float = 0.9, enable_prefix_caching: bool = False) -> "LLMEngine":
         from .sizing import estimate_num_pages
         max_model_len = min(max_model_len, model.spec.max_positions)
         page_size = min(page_size, max_model_len)
@@ -66,7 +67,8 @@ class LLMEngine:
             num_kv_blocks = estimate_num_pages(model, page_size, max_num_batched_tokens,
                                                max_num_seqs, max_model_len, gpu_memory_utilization)
         runner = ModelRunner(model, model.env, page_size=page_size, num_pages=num_kv_blocks,
-                             max_requests=max_num_seqs, max_batch_tokens=max_num_batched_tokens)
+                             max_requests=max_num_seqs, max_batch_tokens=max_num_batched_tokens,
+                             prefix_caching=enable_prefix_caching)
         return cls(runner, max_model_len, max_num_seqs, max_num_batched_tokens,
                    model.spec.eos_token_ids)
 

@@ -95,7 +95,7 @@ class StepInputs:
 
 class ModelRunner:
     def __init__(self, model: Model, env: BuildEnv, page_size: int, num_pages: int,
-                 max_requests: int, max_batch_tokens: int):
+                 max_requests: int, max_batch_tokens: int, prefix_caching: bool = False):
         self.model = model
         self.env = env
         self.page_size = page_size
@@ -103,7 +103,9 @@ class ModelRunner:
         self.max_requests = max_requests
         self.max_model_len = min(env.max_model_len, model.spec.max_positions)
         env.ops.check_page_size(page_size)
-        self.cache = CacheManager(model.cache_needs(), page_size, num_pages, max_requests)
+        if prefix_caching and any(n is not None for n in model.state_needs()):
+            raise ValueError("prefix caching cannot take over per-request state of a mixer")
+        self.cache = CacheManager(model.cache_needs(), page_size, num_pages, max_requests, prefix_caching)
         self.group_tensors = []
         for g in self.cache.groups:
             n, heads, hd = len(g.cache_layers), g.need.num_kv_heads, g.need.head_dim

@@ -10,7 +10,8 @@ The policy is the reference's (engine/src/scheduler.cpp:40-121):
 2. Then prompts.  Waiting requests, in order, each get at most one portion per
    step, cut to the budget that is left.  A request is admitted only when the
    pages for all its current tokens are free (and a state slot); otherwise it
-   goes to the back of the queue.  A prompt that needs more pages than the pool
+   goes to the back of the queue.  With prefix caching, leading full pages that
+   the cache knows are taken over and not computed again.  A prompt that needs more pages than the pool
    owns is an error.
 3. If nothing could be scheduled while work remains, that is an error.
 
@@ -96,12 +97,14 @@ class Scheduler:
         if self.cache.free_slots() == 0:
             return False
         self.cache.admit(seq.request_id)
+        # with prefix caching the leading full pages that are known are taken over
+        cached = self.cache.adopt_prefix(seq.request_id, seq.token_ids) if self.cache.prefix_caching else 0
         if not self.cache.can_reserve(seq.request_id, seq.size):
             self.cache.release(seq.request_id)
             return False
         self.cache.reserve(seq.request_id, seq.size)
         seq.admitted = True
-        seq.num_cached_tokens = 0
+        seq.num_cached_tokens = cached
         return True
 
     # ---- one step's plan -----------------------------------------------------
@@ -160,6 +163,7 @@ class Scheduler:
             seq = item.sequence
             seq.num_cached_tokens += seq.num_scheduled_tokens
             seq.num_scheduled_tokens = 0
+            self.cache.register_pages(seq.request_id, seq.token_ids)     # full pages enter the prefix cache
             if item.is_prefill and seq.num_cached_tokens < seq.size:
                 continue
             if token is None or token < 0:
