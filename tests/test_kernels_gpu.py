@@ -443,6 +443,39 @@ def test_temperature_sampling_is_gumbel_max_over_a_hash(ops):
     assert alone[0] == out[3]
 
 
+def test_sampling_a_large_vocabulary_in_pieces(ops):
+    """Large vocabularies are scanned in pieces; the winner and the tie rule are the same."""
+    from tiny_llm_infer_amd.kernels.ops import sample_uniform
+    rows, vocab = 3, 151936
+    logits = rnd((rows, vocab), torch.float32, 5, 2.0)
+    logits[0, 150000] = logits[0, 9] = logits[0, 77777] = 50.0           # a tie across pieces
+    assert ops.sample(logits.to(DEV)).cpu().tolist() == [9, int(logits[1].argmax()), int(logits[2].argmax())]
+    temps = torch.tensor([0.9, 0.0, 1.3])
+    seeds = torch.tensor([5, 6, 2 ** 50 + 3], dtype=torch.int64)
+    got = ops.sample(logits.to(DEV), temps.to(DEV), seeds.to(DEV)).cpu().tolist()
+    def uniforms(seed, n):
+        """The kernel's hash of (seed, token), vectorised: three rounds of the murmur3 finaliser."""
+        def mix(h):
+            h = h.copy()
+            h ^= h >> np.uint32(16); h *= np.uint32(0x85EBCA6B); h ^= h >> np.uint32(13)
+            h *= np.uint32(0xC2B2AE35); h ^= h >> np.uint32(16)
+            return h
+        lo, hi = np.uint32(seed & 0xFFFFFFFF), np.uint32(seed >> 32)
+        with np.errstate(over="ignore"):
+            h = mix(np.arange(n, dtype=np.uint32) ^ np.uint32(0x9E3779B9))
+            h = mix(h ^ lo)
+            h = mix(h + hi * np.uint32(0x85EBCA6B) + np.uint32(0x27D4EB2F))
+        return ((h >> np.uint32(8)).astype(np.float64) + 0.5) / 16777216.0
+
+    assert abs(uniforms(12345, 10)[7] - sample_uniform(12345, 7)) < 1e-9
+    for r in (0, 2):
+        u = uniforms(int(seeds[r]), vocab)
+        score = logits[r].double().numpy() + float(temps[r]) * -np.log(-np.log(u))
+        order = np.argsort(-score)
+        assert got[r] == int(order[0]) or score[order[0]] - score[got[r]] < 1e-5     # float32 noise on a near-tie
+    assert got[1] == int(logits[1].argmax())
+
+
 def test_temperature_sampling_follows_softmax(ops):
     vocab, n = 6, 4000
     base = torch.tensor([2.0, 1.0, 0.0, -1.0, 0.5, 1.5])

@@ -19,6 +19,7 @@
 // turn and their partial sums are added through LDS in wave order, so the
 // result does not depend on the launch.
 #include "common.h"
+#include <type_traits>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -32,7 +33,7 @@ __device__ __forceinline__ uint4 load16_or_zero(const bf16_t* p, bool ok) {
     return ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
 }
 
-template <int RT, int MT, int WAVES, typename TO, bool TILED = false, bool GATED = false>
+template <int RT, int MT, int WAVES, typename TO, bool TILED = false, bool GATED = false, int DEPTH = 2>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* __restrict__ y,
                    int M, int N, int K) {
@@ -67,42 +68,58 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
         x_row[m] = x + (size_t)(x_ok[m] ? row : 0) * K;
     }
 
-    // two-stage pipeline: the loads of the next 128-wide step are issued before the
-    // MFMAs of the current one, so a wave keeps 4*(RT+MT) 16-byte loads in flight
-    Pack16 a[2][RT][4], b[2][MT][4];
-    auto load_step = [&](int buf, int kb) {
+    // DEPTH-stage pipeline: the loads of the next DEPTH-1 128-wide steps are in flight
+    // while the MFMAs of the current one run, so a wave keeps up to
+    // 4*(RT+MT)*(DEPTH-1) 16-byte loads in flight
+    Pack16 a[DEPTH][RT][4], b[DEPTH][MT][4];
+    auto load_step = [&](auto STAGE, int kb) {
+        constexpr int S = decltype(STAGE)::value;
         const int k = kb + c * 32;
 #pragma unroll
         for (int t = 0; t < RT; ++t)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                a[buf][t][j].u = TILED ? *reinterpret_cast<const uint4*>(w_row[t] + (size_t)(kb / 128) * 2048 + j * 512)
-                                       : load16_or_zero(w_row[t] + k + j * 8, w_ok[t] && (k + j * 8 < K));
+                a[S][t][j].u = TILED ? *reinterpret_cast<const uint4*>(w_row[t] + (size_t)(kb / 128) * 2048 + j * 512)
+                                     : load16_or_zero(w_row[t] + k + j * 8, w_ok[t] && (k + j * 8 < K));
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                b[buf][m][j].u = load16_or_zero(x_row[m] + k + j * 8, x_ok[m] && (k + j * 8 < K));
+                b[S][m][j].u = load16_or_zero(x_row[m] + k + j * 8, x_ok[m] && (k + j * 8 < K));
     };
-    auto mma_step = [&](int buf) {
+    auto mma_step = [&](auto STAGE) {
+        constexpr int S = decltype(STAGE)::value;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int t = 0; t < RT; ++t)
 #pragma unroll
                 for (int m = 0; m < MT; ++m)
-                    acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[buf][t][j].v, b[buf][m][j].v,
+                    acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[S][t][j].v, b[S][m][j].v,
                                                                         acc[t][m], 0, 0, 0);
     };
-    int kb = wave * 128;
-    if (kb < K) load_step(0, kb);
-    for (; kb < K; kb += 2 * WAVES * 128) {
-        const int k1 = kb + WAVES * 128;
-        if (k1 < K) load_step(1, k1);
-        mma_step(0);
-        if (k1 < K) {
-            if (k1 + WAVES * 128 < K) load_step(0, k1 + WAVES * 128);
-            mma_step(1);
+    constexpr int STRIDE = WAVES * 128;
+    const int kb0 = wave * 128;
+    // prologue: stages 0 .. DEPTH-2
+    if (kb0 < K) load_step(std::integral_constant<int, 0>{}, kb0);
+    if (DEPTH > 2 && kb0 + STRIDE < K) load_step(std::integral_constant<int, 1 % DEPTH>{}, kb0 + STRIDE);
+    if (DEPTH > 3 && kb0 + 2 * STRIDE < K) load_step(std::integral_constant<int, 2 % DEPTH>{}, kb0 + 2 * STRIDE);
+    for (int kb = kb0; kb < K; kb += DEPTH * STRIDE) {
+        // step s of this round multiplies stage s and refills stage (s + DEPTH - 1) % DEPTH
+        if (kb + (DEPTH - 1) * STRIDE < K)
+            load_step(std::integral_constant<int, (DEPTH - 1) % DEPTH>{}, kb + (DEPTH - 1) * STRIDE);
+        mma_step(std::integral_constant<int, 0>{});
+        if (kb + STRIDE < K) {
+            if (kb + DEPTH * STRIDE < K) load_step(std::integral_constant<int, 0>{}, kb + DEPTH * STRIDE);
+            mma_step(std::integral_constant<int, 1 % DEPTH>{});
+        }
+        if (DEPTH > 2 && kb + 2 * STRIDE < K) {
+            if (kb + (DEPTH + 1) * STRIDE < K) load_step(std::integral_constant<int, 1 % DEPTH>{}, kb + (DEPTH + 1) * STRIDE);
+            mma_step(std::integral_constant<int, 2 % DEPTH>{});
+        }
+        if (DEPTH > 3 && kb + 3 * STRIDE < K) {
+            if (kb + (DEPTH + 2) * STRIDE < K) load_step(std::integral_constant<int, 2 % DEPTH>{}, kb + (DEPTH + 2) * STRIDE);
+            mma_step(std::integral_constant<int, 3 % DEPTH>{});
         }
     }
 
@@ -154,17 +171,22 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
     }
 }
 
+#ifndef PIPE_DEPTH
+#define PIPE_DEPTH 2
+#endif
+
 template <int RT, int MT, int WAVES>
 static int launch_skinny(const bf16_t* x, const bf16_t* w, void* y, int M, int N, int K, int y_dtype,
                          int tiled, hipStream_t s) {
     const int blocks = (N + 16 * RT - 1) / (16 * RT);
+    constexpr int D = (MT == 1 && RT <= 2) ? PIPE_DEPTH : 2;    // deep prefetch where the registers allow
     if (tiled == 2) {       // gated: pairs of row tiles, silu(gate)*up written as bfloat16
-        gemm_skinny_kernel<RT, MT, WAVES, bf16_t, true, true><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
+        gemm_skinny_kernel<RT, MT, WAVES, bf16_t, true, true, D><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
     } else if (tiled) {
         if (y_dtype == TLI_BF16)
-            gemm_skinny_kernel<RT, MT, WAVES, bf16_t, true><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
+            gemm_skinny_kernel<RT, MT, WAVES, bf16_t, true, false, D><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
         else
-            gemm_skinny_kernel<RT, MT, WAVES, float, true><<<blocks, WAVES * 64, 0, s>>>(x, w, (float*)y, M, N, K);
+            gemm_skinny_kernel<RT, MT, WAVES, float, true, false, D><<<blocks, WAVES * 64, 0, s>>>(x, w, (float*)y, M, N, K);
     } else {
         if (y_dtype == TLI_BF16)
             gemm_skinny_kernel<RT, MT, WAVES, bf16_t, false><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);

@@ -88,19 +88,85 @@ __global__ void sample_kernel(const float* __restrict__ logits, int vocab,
     }
 }
 
+// Without top-p a row is cut into SAMPLE_CHUNKS pieces that one workgroup each scans
+// (a single workgroup on 150 thousand logits is bound by latency); a second pass picks
+// the best of the pieces.  The winner is the same: the highest score, lowest id on ties.
+#define SAMPLE_CHUNKS 32
+
+__global__ void sample_chunks_kernel(const float* __restrict__ logits, int vocab,
+                                     const float* __restrict__ temperatures,
+                                     const uint32_t* __restrict__ seeds, float* __restrict__ best_value,
+                                     int* __restrict__ best_index) {
+    __shared__ float bvs[256 / TLI_WAVE];
+    __shared__ int bis[256 / TLI_WAVE];
+    const int row = blockIdx.y, chunk = blockIdx.x;
+    const float* l = logits + (size_t)row * vocab;
+    const float temp = temperatures ? temperatures[row] : 0.f;
+    const bool draw = temp > 1.0e-6f;
+    const uint32_t lo = seeds ? seeds[2 * row] : 0u, hi = seeds ? seeds[2 * row + 1] : 0u;
+    const int per = (vocab + SAMPLE_CHUNKS - 1) / SAMPLE_CHUNKS;
+    const int begin = chunk * per, end = min(vocab, begin + per);
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int t = begin + threadIdx.x; t < end; t += blockDim.x) {
+        float s = l[t];
+        if (draw) s += temp * -logf(-logf(tli_uniform(lo, hi, (uint32_t)t)));
+        if (s > bv || (s == bv && t < bi)) { bv = s; bi = t; }
+    }
+    for (int off = TLI_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, TLI_WAVE);
+        const int oi = __shfl_xor(bi, off, TLI_WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE;
+    if (lane == 0) { bvs[wave] = bv; bis[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x / TLI_WAVE); ++w)
+            if (bvs[w] > bv || (bvs[w] == bv && bis[w] < bi)) { bv = bvs[w]; bi = bis[w]; }
+        best_value[row * SAMPLE_CHUNKS + chunk] = bv;
+        best_index[row * SAMPLE_CHUNKS + chunk] = bi;
+    }
+}
+
+__global__ void sample_pick_kernel(const float* __restrict__ best_value, const int* __restrict__ best_index,
+                                   int* __restrict__ out) {
+    const int row = blockIdx.x, lane = threadIdx.x;          // one wave
+    float bv = lane < SAMPLE_CHUNKS ? best_value[row * SAMPLE_CHUNKS + lane] : -INFINITY;
+    int bi = lane < SAMPLE_CHUNKS ? best_index[row * SAMPLE_CHUNKS + lane] : 0x7fffffff;
+    for (int off = TLI_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, TLI_WAVE);
+        const int oi = __shfl_xor(bi, off, TLI_WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if (lane == 0) out[row] = (bi == 0x7fffffff) ? 0 : bi;
+}
+
 // temperatures: float [rows] or null (greedy); seeds: uint32 [rows][2] (low, high word) or null;
 // top_p: float [rows] or null (1 everywhere)
+// scratch: rows * SAMPLE_CHUNKS * 8 bytes, used when top_p is null and the vocabulary is large
 extern "C" int tli_sample(const float* logits, int rows, int vocab, const float* temperatures,
-                          const uint32_t* seeds, const float* top_p, int* out, void* stream) {
+                          const uint32_t* seeds, const float* top_p, int* out, void* scratch, void* stream) {
     if (rows <= 0) return 0;
     if (vocab <= 0) return tli_fail("sample: bad vocabulary size %d", vocab);
     if (temperatures && !seeds) return tli_fail("sample: temperatures need seeds");
+    if (!top_p && scratch && vocab >= 8192 && rows <= 65535) {
+        float* bv = (float*)scratch;
+        int* bi = (int*)(bv + (size_t)rows * SAMPLE_CHUNKS);
+        sample_chunks_kernel<<<dim3(SAMPLE_CHUNKS, rows), 256, 0, (hipStream_t)stream>>>(logits, vocab, temperatures,
+                                                                                      seeds, bv, bi);
+        if (tli_check_launch("sample_chunks")) return 1;
+        sample_pick_kernel<<<rows, TLI_WAVE, 0, (hipStream_t)stream>>>(bv, bi, out);
+        return tli_check_launch("sample_pick");
+    }
     sample_kernel<<<rows, SAMPLE_THREADS, 0, (hipStream_t)stream>>>(logits, vocab, temperatures, seeds,
                                                                      top_p, out);
     return tli_check_launch("sample");
 }
 
 // the same draw on the host, for tests and for callers that hold logits there
+extern "C" int tli_sample_scratch_bytes(int rows) { return rows * SAMPLE_CHUNKS * 8; }
+
 extern "C" float tli_sample_uniform(uint32_t seed_lo, uint32_t seed_hi, uint32_t token) {
     return tli_uniform(seed_lo, seed_hi, token);
 }

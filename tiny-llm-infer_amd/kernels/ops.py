@@ -58,7 +58,8 @@ def load_library():
         "tli_gemm_mid_splits": [I, I],
         "tli_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
         "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, I, P],
-        "tli_sample": [P, I, I, P, P, P, P, P],
+        "tli_sample": [P, I, I, P, P, P, P, P, P],
+        "tli_sample_scratch_bytes": [I],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -357,9 +358,11 @@ class HipOps:
         if top_p is not None:
             self._want(top_p, "top_p", torch.float32, (rows,))
         out = torch.empty((rows,), dtype=torch.int32, device=self.device)
+        scratch = torch.empty((self.lib.tli_sample_scratch_bytes(rows),), dtype=torch.uint8, device=self.device)
         self._call(self.lib.tli_sample, logits.data_ptr(), rows, vocab, _ptr(temperatures),
                    _ptr(seeds) if temperatures is not None else None,
-                   _ptr(top_p) if temperatures is not None else None, out.data_ptr(), self._stream())
+                   _ptr(top_p) if temperatures is not None else None, out.data_ptr(), scratch.data_ptr(),
+                   self._stream())
         return out
 
 
