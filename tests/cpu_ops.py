@@ -17,6 +17,10 @@ class CpuOps:
     def check_page_size(self, page_size):
         pass
 
+    def feed_tokens(self, token_ids, token_from, src, rows):
+        take = token_from[:rows] >= 0
+        token_ids[:rows][take] = src[token_from[:rows][take].long()]
+
     def embed(self, table, token_ids, num_rows):
         return table[token_ids.long()].to(torch.float32)
 

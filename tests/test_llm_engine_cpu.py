@@ -101,3 +101,25 @@ def test_prefix_caching_gives_the_same_tokens_and_skips_work(model_folders):
     assert [r.token_ids for r in got] == [r.token_ids for r in plain]
     small.runner.cache.check()
     assert small.runner.cache.free_pages() == [14]
+
+
+def test_steps_put_on_the_device_ahead_change_nothing(model_folders):
+    """The next decode step is launched before this step's tokens are read; requests
+    that stop on an end-of-sequence token or at max_tokens meanwhile, and sampling
+    with a temperature, give exactly what the step-by-step engine gives."""
+    folder = model_folders["B"]
+    prompts = [random_prompt(384, n, 50 + n) for n in (4, 30, 17, 9)]
+    params = [SamplingParams(max_tokens=m, temperature=t, seed=7 + i)
+              for i, (m, t) in enumerate([(9, 0.0), (14, 0.8), (3, 0.0), (11, 0.5)])]
+    outs = []
+    for ahead in (False, True):
+        eng = _engine(folder, "B", max_num_batched_tokens=64)
+        eng.lookahead = ahead
+        free = _engine(folder, "B", max_num_batched_tokens=64).generate([prompts[0]], [SamplingParams(max_tokens=9)])
+        eng.eos_token_ids = {free[0].token_ids[4]}            # request 0 stops early on this token
+        outs.append(eng.generate(prompts, params))
+        assert (eng.num_steps_ahead > 5) == ahead
+        eng.runner.cache.check()
+        assert eng.runner.cache.free_pages() == [64, 64] and eng.is_finished()
+    assert [r.token_ids for r in outs[0]] == [r.token_ids for r in outs[1]]
+    assert len(outs[1][0].token_ids) <= 5 and len(outs[1][2].token_ids) <= 3

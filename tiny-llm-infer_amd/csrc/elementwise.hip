@@ -141,6 +141,23 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
     from_f32(out + idx, g / (1.0f + expf(-g)) * u);
 }
 
+// token_ids[r] = src[from[r]] where from[r] >= 0: the tokens a step sampled become the
+// next step's inputs without leaving the device
+__global__ void feed_tokens_kernel(int* __restrict__ token_ids, const int* __restrict__ from,
+                                   const int* __restrict__ src, int rows, int src_count) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= rows) return;
+    const int f = from[r];
+    if (f >= 0 && f < src_count) token_ids[r] = src[f];
+}
+
+extern "C" int tli_feed_tokens(int* token_ids, const int* from, const int* src, int rows, int src_count,
+                               void* stream) {
+    if (rows <= 0) return 0;
+    feed_tokens_kernel<<<(rows + 255) / 256, 256, 0, (hipStream_t)stream>>>(token_ids, from, src, rows, src_count);
+    return tli_check_launch("feed_tokens");
+}
+
 extern "C" int tli_embed(const void* table, const int* ids, float* out, int rows, int hidden,
                          int vocab, int dtype, void* stream) {
     if (rows <= 0) return 0;

@@ -16,7 +16,17 @@ from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .runner import ModelRunner, StepEntry
 from .scheduler import BatchPlan, Scheduler, SchedulerConfig
-from .sequence import Sequence
+from .sequence import Sequence, Status
+
+
+@dataclass
+class _Inflight:
+    """A step that is on the device: its plan, which items sample, the sampled token
+    ids (int32 tensor on the device, not yet read) and each request's row in them."""
+    plan: BatchPlan
+    sampled_items: List[int]
+    tokens: Optional[torch.Tensor]
+    row_of: dict
 
 
 @dataclass
@@ -41,6 +51,9 @@ class LLMEngine:
         self._next_request_id = 1
         self.total_generated_tokens = 0
         self.num_steps = 0
+        self.num_steps_ahead = 0
+        self.lookahead = True                # put the next decode step on the device before reading this one
+        self._inflight: Optional[_Inflight] = None
 
     # ---- construction ---------------------------------------------------------
     @classmethod
@@ -101,37 +114,68 @@ class LLMEngine:
 
     def is_finished(self) -> bool:
         with self._lock:
-            return self.scheduler.is_finished()
+            return self.scheduler.is_finished() and self._inflight is None
 
     def is_eos(self, token: int) -> bool:
         return token in self.eos_token_ids
 
     # ---- one step -------------------------------------------------------------------
-    def step(self) -> List[GenerationResult]:
-        """engine/src/llm_engine.cpp:148-248."""
-        with self._lock:
-            plan = self.scheduler.schedule()
-        if not plan.sequences:
-            return []
+    def _launch(self, plan: BatchPlan, ahead_of: Optional["_Inflight"] = None) -> "_Inflight":
+        """Put one planned step on the device: the batch, then the sampling.  Nothing
+        is waited for.  With ``ahead_of``, every item's token is the one that step
+        sampled for the same request and is taken on the device."""
         entries, sampled_items = [], []
         for i, item in enumerate(plan.sequences):
             seq = item.sequence
-            toks = seq.token_ids[item.token_start:item.token_start + item.token_count]
             want = [item.token_count - 1] if item.samples else []
-            entries.append(StepEntry(seq.request_id, toks, want))
+            if ahead_of is None:
+                toks = seq.token_ids[item.token_start:item.token_start + item.token_count]
+                entries.append(StepEntry(seq.request_id, toks, want))
+            else:
+                entries.append(StepEntry(seq.request_id, [0], want, token_from=ahead_of.row_of[seq.request_id]))
             if item.samples:
                 sampled_items.append(i)
-        logits = self.runner.step(entries)
-        sampled: List[Optional[int]] = [None] * len(plan.sequences)
+        logits = self.runner.step(entries, feed=None if ahead_of is None else ahead_of.tokens)
+        tokens = None
+        row_of = {}
         if sampled_items:
             seqs = [plan.sequences[i].sequence for i in sampled_items]
-            tokens = self.sampler.sample(logits, [s.sampling for s in seqs],
-                                         [s.rng_seed for s in seqs], [s.num_sampled for s in seqs])
-            for i, tok in zip(sampled_items, tokens):
+            # a request whose previous draw is still on the device has one more sample behind it
+            extra = 0 if ahead_of is None else 1
+            tokens = self.sampler.launch(logits, [s.sampling for s in seqs], [s.rng_seed for s in seqs],
+                                         [s.num_sampled + extra for s in seqs])
+            row_of = {s.request_id: j for j, s in enumerate(seqs)}
+        return _Inflight(plan, sampled_items, tokens, row_of)
+
+    def step(self) -> List[GenerationResult]:
+        """One step of the engine (engine/src/llm_engine.cpp:148-248): schedule, run the
+        batch, sample, post-process.  When the step after this one is already known
+        (decode only, see Scheduler.plan_ahead) it is put on the device before this
+        step's tokens are read back, fed on the device with the tokens sampled here,
+        so the device does not wait for the host between steps."""
+        cur = self._inflight
+        if cur is None:
+            with self._lock:
+                plan = self.scheduler.schedule()
+            if not plan.sequences:
+                return []
+            cur = self._launch(plan)
+        nxt = None
+        if self.lookahead and cur.tokens is not None:
+            with self._lock:
+                ahead = self.scheduler.plan_ahead(cur.plan)
+            if ahead is not None:
+                nxt = self._launch(ahead, ahead_of=cur)
+                self.num_steps_ahead += 1
+        sampled: List[Optional[int]] = [None] * len(cur.plan.sequences)
+        if cur.sampled_items:
+            for i, tok in zip(cur.sampled_items, cur.tokens.tolist()):      # waits for this step only
                 sampled[i] = int(tok)
+        live = sum(1 for i in cur.sampled_items if cur.plan.sequences[i].sequence.status != Status.FINISHED)
         with self._lock:
-            finished = self.scheduler.postprocess(plan, sampled, self.is_eos)
-        self.total_generated_tokens += len(sampled_items)
+            finished = self.scheduler.postprocess(cur.plan, sampled, self.is_eos)
+        self._inflight = nxt
+        self.total_generated_tokens += live
         self.num_steps += 1
         return [GenerationResult(s.request_id, s.completion_tokens, s.token_ids[:s.prompt_size],
                                  s.preemptions) for s in finished]

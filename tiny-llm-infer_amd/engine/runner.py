@@ -28,6 +28,8 @@ class StepEntry:
     key: Hashable                 # the request
     tokens: Sequence[int]         # its next tokens
     want: Sequence[int] = ()      # places among ``tokens`` whose logits are wanted
+    token_from: Optional[int] = None   # a single token that is not known on the host yet: its value is
+                                       # element ``token_from`` of the tensor given to step(feed=...)
 
 
 class StepError(ValueError):
@@ -52,7 +54,7 @@ class StepInputs:
 
     def __init__(self, device, max_rows: int, max_seqs: int, num_groups: int, max_width: int):
         self.device = torch.device(device)
-        cap = (3 * _pad4(max_rows) + _pad4(max_rows) + _pad4(max_seqs + 1) + 3 * _pad4(max_seqs)
+        cap = (4 * _pad4(max_rows) + _pad4(max_rows) + _pad4(max_seqs + 1) + 3 * _pad4(max_seqs)
                + num_groups * max_seqs * max_width + 64)
         pin = self.device.type == "cuda"
         self.host = [torch.zeros(cap, dtype=torch.int32, pin_memory=pin) for _ in range(2)]
@@ -65,7 +67,7 @@ class StepInputs:
     def layout(self, rows: int, seqs: int, wanted: int, width: int) -> Dict[str, slice]:
         off = 0
         out = {}
-        for name, n in (("token_ids", rows), ("positions", rows), ("seq_of_row", rows),
+        for name, n in (("token_ids", rows), ("token_from", rows), ("positions", rows), ("seq_of_row", rows),
                         ("row_start", seqs + 1), ("seq_start", seqs), ("seq_len", seqs),
                         ("slots", seqs), ("sample_rows", wanted)):
             out[name] = slice(off, off + n)
@@ -169,6 +171,8 @@ class ModelRunner:
                 if not 0 <= int(t) < vocab:
                     raise StepError(f"token id {t} of request {e.key!r} is outside the "
                                     f"vocabulary of {vocab}")
+            if e.token_from is not None and n != 1:
+                raise StepError(f"request {e.key!r}: only a single token can come from the device")
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"wanted place {w} of request {e.key!r} is outside its "
@@ -176,7 +180,7 @@ class ModelRunner:
         if rows > self.max_batch_tokens:
             raise StepError(f"{rows} tokens in one step, at most {self.max_batch_tokens}")
 
-    def _pack(self, entries: Sequence[StepEntry]) -> StepView:
+    def _pack(self, entries: Sequence[StepEntry], feed: Optional[torch.Tensor] = None) -> StepView:
         page = self.page_size
         rcs = [self.cache.get(e.key) for e in entries]
         starts = [rc.num_tokens for rc in rcs]
@@ -187,18 +191,22 @@ class ModelRunner:
         width = _pow2_at_least(max(max((len(tab) for tab in rc.tables), default=1) for rc in rcs))
         lay = self.inputs.layout(rows, seqs, wanted, width)
         buf = self.inputs.begin()
-        row_start = [0]
+        # every field is put together as one list and written with one assignment
+        tok, pos, sor, sample, row_start, src = [], [], [], [], [0], []
         r = 0
-        sample = []
         for i, e in enumerate(entries):
             n = counts[i]
-            buf[lay["token_ids"].start + r: lay["token_ids"].start + r + n] = np.asarray(e.tokens, dtype=np.int32)
-            buf[lay["positions"].start + r: lay["positions"].start + r + n] = np.arange(
-                starts[i], starts[i] + n, dtype=np.int32)
-            buf[lay["seq_of_row"].start + r: lay["seq_of_row"].start + r + n] = i
+            tok.extend(e.tokens)
+            src.extend([-1] * n if e.token_from is None else [int(e.token_from)])
+            pos.extend(range(starts[i], starts[i] + n))
+            sor.extend([i] * n)
             sample.extend(r + int(w) for w in e.want)
             r += n
             row_start.append(r)
+        buf[lay["token_ids"]] = tok
+        buf[lay["token_from"]] = src
+        buf[lay["positions"]] = pos
+        buf[lay["seq_of_row"]] = sor
         buf[lay["row_start"]] = row_start
         buf[lay["seq_start"]] = starts
         buf[lay["seq_len"]] = totals
@@ -206,13 +214,16 @@ class ModelRunner:
         if wanted:
             buf[lay["sample_rows"]] = sample
         for g in range(len(self.cache.groups)):
-            t = buf[lay[f"tables{g}"]].reshape(seqs, width)
-            t[:] = -1
-            for i, rc in enumerate(rcs):
+            flat = []
+            for rc in rcs:
                 tab = rc.tables[g]
-                t[i, :len(tab)] = tab
+                flat.extend(tab)
+                flat.extend([-1] * (width - len(tab)))
+            buf[lay[f"tables{g}"]] = flat
         self.inputs.upload(lay["_end"].stop)
         dev = self.inputs.dev
+        if feed is not None:
+            self.env.ops.feed_tokens(dev[lay["token_ids"]], dev[lay["token_from"]], feed, rows)
         groups = []
         for g, gl in enumerate(self.cache.groups):
             k, v = self.group_tensors[g]
@@ -270,9 +281,11 @@ class ModelRunner:
         self.graph_replays += 1
         return entry[1]
 
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], feed: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run one batch.  Pages are reserved for every entry first; if the pool
-        cannot hold the batch, CacheFull is raised and no token has been run."""
+        cannot hold the batch, CacheFull is raised and no token has been run.
+        ``feed``: int32 tensor on the device that entries with ``token_from`` take
+        their token from (the tokens the previous step sampled)."""
         self._check(entries)
         # all or nothing over the whole batch: groups are independent, requests compete
         need = [0] * len(self.cache.groups)
@@ -286,7 +299,9 @@ class ModelRunner:
                                 f"{self.cache.groups[g].pool.free_count} are free")
         for e in entries:
             self.cache.reserve(e.key, self.cache.get(e.key).num_tokens + len(e.tokens))
-        view = self._pack(entries)
+        if feed is None and any(e.token_from is not None for e in entries):
+            raise StepError("an entry takes its token from the device but no tensor was given")
+        view = self._pack(entries, feed)
         wanted = sum(len(e.want) for e in entries)
         if self.use_graphs and view.max_rows_per_seq == 1 and wanted == len(entries):
             logits = self._replay(view, wanted)

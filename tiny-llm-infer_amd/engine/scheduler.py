@@ -77,6 +77,34 @@ class Scheduler:
     def is_finished(self) -> bool:
         return not self.waiting and not self.running
 
+    def plan_ahead(self, plan: BatchPlan) -> Optional[BatchPlan]:
+        """The plan of the step after ``plan``, made while ``plan`` is still running on
+        the device, or None if it cannot be known yet.  It can when the next step is
+        decode only: nothing waits, ``plan`` covers every running request and every item
+        of it samples (so each request needs exactly its next token), and the pages for
+        those tokens are free.  A request that reaches ``max_tokens`` with the running
+        step is left out; one that will stop on an end-of-sequence token cannot be known
+        and is skipped when its result comes in."""
+        if self.waiting or len(plan.sequences) != len(self.running) or not plan.sequences:
+            return None
+        if any(not item.samples or item.sequence.status == Status.FINISHED for item in plan.sequences):
+            return None
+        ahead = BatchPlan()
+        for item in plan.sequences:
+            seq = item.sequence
+            if seq.completion_size + 1 >= seq.sampling.max_tokens:
+                continue                      # the running step's token is its last
+            # seq.size does not count the running step's token yet: that token goes to position seq.size
+            if not self.cache.can_reserve(seq.request_id, seq.size + 1):
+                return None                   # pages run out: the ordinary path decides whom to preempt
+            ahead.sequences.append(ScheduledSequence(seq, seq.size, 1, False))
+        if not ahead.sequences or len(ahead.sequences) > self.config.max_num_seqs:
+            return None
+        for item in ahead.sequences:
+            self.cache.reserve(item.sequence.request_id, item.token_start + 1)
+        ahead.num_tokens = len(ahead.sequences)
+        return ahead
+
     # ---- pages ------------------------------------------------------------
     def _preempt(self, seq: Sequence) -> None:
         if seq.admitted:
@@ -161,7 +189,9 @@ class Scheduler:
         finished = []
         for item, token in zip(plan.sequences, sampled):
             seq = item.sequence
-            seq.num_cached_tokens += seq.num_scheduled_tokens
+            if seq.status == Status.FINISHED:
+                continue            # it ended in the step before, while this one was already running
+            seq.num_cached_tokens += item.token_count
             seq.num_scheduled_tokens = 0
             self.cache.register_pages(seq.request_id, seq.token_ids)     # full pages enter the prefix cache
             if item.is_prefill and seq.num_cached_tokens < seq.size:

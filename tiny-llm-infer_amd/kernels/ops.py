@@ -48,6 +48,7 @@ def load_library():
     sigs = {
         "tli_abi_version": [],
         "tli_embed": [P, P, P, I, I, I, I, P],
+        "tli_feed_tokens": [P, P, P, I, I, P],
         "tli_add_rmsnorm": [P, P, P, P, P, I, I, I, F, I, P],
         "tli_swiglu": [P, P, I, I, I, P],
         "tli_qkv_to_cache": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I, I, I, I, P],
@@ -126,6 +127,15 @@ class HipOps:
             raise KernelError(f"page size {page_size} is not supported: powers of two up to 256")
 
     # ---- ops ------------------------------------------------------------------
+    def feed_tokens(self, token_ids: torch.Tensor, token_from: torch.Tensor, src: torch.Tensor, rows: int):
+        """token_ids[r] = src[token_from[r]] where token_from[r] >= 0 (all int32, on the device)."""
+        for t, what in ((token_ids, "token ids"), (token_from, "token sources"), (src, "sampled tokens")):
+            self._want(t, what, torch.int32)
+        if token_ids.numel() < rows or token_from.numel() < rows:
+            raise KernelError("fewer token ids than rows")
+        self._call(self.lib.tli_feed_tokens, token_ids.data_ptr(), token_from.data_ptr(), src.data_ptr(),
+                   rows, src.numel(), self._stream())
+
     def embed(self, table: torch.Tensor, token_ids: torch.Tensor, num_rows: int) -> torch.Tensor:
         vocab, hidden = table.shape
         self._want(table, "embedding table")

@@ -44,10 +44,15 @@ class Sampler:
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams],
                request_seeds: Sequence[int], sample_indices: Sequence[int]) -> List[int]:
         """One token id per row of ``logits`` [rows, vocab] (float32, on the device)."""
+        return self.launch(logits, params, request_seeds, sample_indices).tolist()
+
+    def launch(self, logits: torch.Tensor, params: Sequence[SamplingParams],
+               request_seeds: Sequence[int], sample_indices: Sequence[int]) -> torch.Tensor:
+        """The same without waiting: the token ids as an int32 tensor on the device."""
         rows = logits.shape[0]
         assert rows == len(params) == len(request_seeds) == len(sample_indices)
         if all(p.greedy for p in params):
-            return self.ops.sample(logits).tolist()
+            return self.ops.sample(logits)
         temps = torch.tensor([0.0 if p.greedy else p.temperature for p in params],
                              dtype=torch.float32)
         seeds = [draw_seed(s, i) for s, i in zip(request_seeds, sample_indices)]
@@ -56,5 +61,4 @@ class Sampler:
         top_p = None
         if any(p.top_p < 1.0 and not p.greedy for p in params):
             top_p = torch.tensor([p.top_p for p in params], dtype=torch.float32).to(self.device)
-        return self.ops.sample(logits, temps.to(self.device), seeds_t.to(self.device),
-                               top_p=top_p).tolist()
+        return self.ops.sample(logits, temps.to(self.device), seeds_t.to(self.device), top_p=top_p)
