@@ -346,6 +346,9 @@ QKV_CASES = [
     (8, 2, 128, 128, True, 16),
     (3, 3, 64, 32, False, 16),      # partial rotation, no norms
     (2, 1, 80, 0, True, 16),        # no rotation at all
+    (4, 4, 64, 64, True, 8),        # head sizes 64 and 256: the kernel without LDS, 1 and 4 elements a lane
+    (3, 1, 256, 256, True, 16),
+    (2, 2, 128, 0, False, 16),
 ]
 
 

@@ -100,6 +100,91 @@ __global__ void qkv_to_cache_kernel(
     }
 }
 
+// The same for head sizes that are multiples of 64 (EPL = head_dim / 64 elements a
+// lane), without LDS: a lane holds EPL consecutive elements, so the first half of
+// the head lies in lanes 0..31 and the rotation partner of lane l is lane l ^ 32.
+// Needs rotary_dim == head_dim (or no rotation).  bfloat16 only.
+template <int EPL>
+__global__ void __launch_bounds__(QKV_WAVES * TLI_WAVE)
+qkv_to_cache_wide_kernel(
+    const bf16_t* __restrict__ qkv, bf16_t* __restrict__ q_out, bf16_t* __restrict__ k_cache,
+    bf16_t* __restrict__ v_cache, const int* __restrict__ positions, const int* __restrict__ seq_of_row,
+    const int* __restrict__ tables, int table_width, int page_size, int num_pages,
+    int heads, int kv_heads,
+    const float* __restrict__ q_norm_w, float q_eps, const float* __restrict__ k_norm_w, float k_eps,
+    const float* __restrict__ cos_table, const float* __restrict__ sin_table, int table_positions,
+    int write_cache) {
+    constexpr int HD = 64 * EPL;
+    const int row = blockIdx.x;
+    const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE;
+    const int h = blockIdx.y * QKV_WAVES + wave;
+    if (h >= heads + 2 * kv_heads) return;
+    const int q_dim = heads * HD, kv_dim = kv_heads * HD;
+    const int pos = positions[row];
+    const bf16_t* src = qkv + (size_t)row * (q_dim + 2 * kv_dim) + (size_t)h * HD + lane * EPL;
+    const bool is_q = h < heads, is_v = h >= heads + kv_heads;
+
+    int page = -1;
+    if (write_cache && !is_q) {
+        page = tables[(size_t)seq_of_row[row] * table_width + pos / page_size];
+        if (page < 0 || page >= num_pages) return;
+    } else if (!is_q) {
+        return;                                       // keys and values of a read-only cache layer
+    }
+    // EPL consecutive elements of this lane
+    float x[EPL];
+    if (EPL == 1) {
+        x[0] = bf16_to_f32(src[0]);
+    } else if (EPL == 2) {
+        const uint32_t u = *reinterpret_cast<const uint32_t*>(src);
+        x[0] = bf16_to_f32((bf16_t)(u & 0xffffu));
+        x[1 % EPL] = bf16_to_f32((bf16_t)(u >> 16));
+    } else {
+        const uint2 u = *reinterpret_cast<const uint2*>(src);
+        x[0] = bf16_to_f32((bf16_t)(u.x & 0xffffu));
+        x[1 % EPL] = bf16_to_f32((bf16_t)(u.x >> 16));
+        x[2 % EPL] = bf16_to_f32((bf16_t)(u.y & 0xffffu));
+        x[3 % EPL] = bf16_to_f32((bf16_t)(u.y >> 16));
+    }
+    if (is_v) {
+        const int g = h - heads - kv_heads;
+        bf16_t* dst = v_cache + ((size_t)page * kv_heads + g) * HD * page_size + (pos % page_size);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) dst[(size_t)(lane * EPL + e) * page_size] = src[e];
+        return;
+    }
+    const float* nw = is_q ? q_norm_w : k_norm_w;
+    if (nw) {
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) ss += x[e] * x[e];
+        ss = wave_sum(ss);
+        const float scale = 1.0f / sqrtf(ss / (float)HD + (is_q ? q_eps : k_eps));
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) x[e] = nw[lane * EPL + e] * x[e] * scale;
+    }
+    if (cos_table && pos >= 0 && pos < table_positions) {
+        const float* cr = cos_table + (size_t)pos * (HD / 2) + (lane % 32) * EPL;
+        const float* sr = sin_table + (size_t)pos * (HD / 2) + (lane % 32) * EPL;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            const float partner = __shfl_xor(x[e], 32, TLI_WAVE);
+            // first half: x cos - partner sin; second half: partner sin + x cos
+            x[e] = lane < 32 ? x[e] * cr[e] - partner * sr[e] : partner * sr[e] + x[e] * cr[e];
+        }
+    }
+    bf16_t* dst = is_q ? q_out + (size_t)row * q_dim + (size_t)h * HD
+                       : k_cache + (((size_t)page * kv_heads + (h - heads)) * page_size + (pos % page_size)) * HD;
+    dst += lane * EPL;
+    if (EPL == 1) {
+        dst[0] = f32_to_bf16(x[0]);
+    } else if (EPL == 2) {
+        *reinterpret_cast<uint32_t*>(dst) = pack_bf16x2(x[0], x[1 % EPL]);
+    } else {
+        *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(x[0], x[1 % EPL]), pack_bf16x2(x[2 % EPL], x[3 % EPL]));
+    }
+}
+
 extern "C" int tli_qkv_to_cache(
     const void* qkv, void* q_out, void* k_cache, void* v_cache, const int* positions,
     const int* seq_of_row, const int* tables, int table_width, int page_size, int num_pages,
@@ -120,6 +205,19 @@ extern "C" int tli_qkv_to_cache(
     const int units = heads + 2 * kv_heads;
     if ((units + QKV_WAVES - 1) / QKV_WAVES > 65535) return tli_fail("qkv_to_cache: too many heads");
     dim3 grid(rows, (units + QKV_WAVES - 1) / QKV_WAVES);
+    if (dtype == TLI_BF16 && head_dim % 64 == 0 && head_dim <= 256 && head_dim != 192 &&
+        (!cos_table || rotary_dim == head_dim)) {
+#define WIDE(EPL)                                                                                        \
+    qkv_to_cache_wide_kernel<EPL><<<grid, threads, 0, s>>>(                                              \
+        (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, positions, seq_of_row,   \
+        tables, table_width, page_size, num_pages, heads, kv_heads, q_norm_w, q_eps, k_norm_w, k_eps,    \
+        cos_table, sin_table, table_positions, write_cache)
+        if (head_dim == 64) WIDE(1);
+        else if (head_dim == 128) WIDE(2);
+        else WIDE(4);
+#undef WIDE
+        return tli_check_launch("qkv_to_cache_wide");
+    }
     if (dtype == TLI_F32)
         qkv_to_cache_kernel<float><<<grid, threads, 0, s>>>(
             (const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache, positions, seq_of_row,

@@ -167,10 +167,10 @@ class ModelRunner:
             if total > self.max_model_len:
                 raise StepError(f"request {e.key!r} would reach {total} tokens, "
                                 f"the limit is {self.max_model_len}")
-            for t in e.tokens:
-                if not 0 <= int(t) < vocab:
-                    raise StepError(f"token id {t} of request {e.key!r} is outside the "
-                                    f"vocabulary of {vocab}")
+            lo, hi = (min(e.tokens), max(e.tokens))
+            if lo < 0 or hi >= vocab:
+                raise StepError(f"token id {lo if lo < 0 else hi} of request {e.key!r} is outside the "
+                                f"vocabulary of {vocab}")
             if e.token_from is not None and n != 1:
                 raise StepError(f"request {e.key!r}: only a single token can come from the device")
             for w in e.want:
