@@ -27,6 +27,14 @@ class _Inflight:
     sampled_items: List[int]
     tokens: Optional[torch.Tensor]
     row_of: dict
+    host_copy: Optional[tuple] = None        # (pinned tensor the ids are being copied to, event after the copy)
+
+    def token_list(self) -> List[int]:
+        if self.host_copy is None:
+            return self.tokens.tolist()
+        host, done = self.host_copy
+        done.synchronize()
+        return host.tolist()
 
 
 @dataclass
@@ -145,7 +153,18 @@ class LLMEngine:
             tokens = self.sampler.launch(logits, [s.sampling for s in seqs], [s.rng_seed for s in seqs],
                                          [s.num_sampled + extra for s in seqs])
             row_of = {s.request_id: j for j, s in enumerate(seqs)}
-        return _Inflight(plan, sampled_items, tokens, row_of)
+        return _Inflight(plan, sampled_items, tokens, row_of, self._read_back(tokens))
+
+    def _read_back(self, tokens: Optional[torch.Tensor]):
+        """Start copying sampled token ids to the host now, so that reading them later
+        waits for this step only and not for whatever is put on the device after it."""
+        if tokens is None or tokens.device.type != "cuda":
+            return None
+        host = torch.empty(tokens.shape, dtype=tokens.dtype, pin_memory=True)
+        host.copy_(tokens, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        return host, done
 
     def step(self) -> List[GenerationResult]:
         """One step of the engine (engine/src/llm_engine.cpp:148-248): schedule, run the
@@ -169,7 +188,7 @@ class LLMEngine:
                 self.num_steps_ahead += 1
         sampled: List[Optional[int]] = [None] * len(cur.plan.sequences)
         if cur.sampled_items:
-            for i, tok in zip(cur.sampled_items, cur.tokens.tolist()):      # waits for this step only
+            for i, tok in zip(cur.sampled_items, cur.token_list()):         # waits for this step only
                 sampled[i] = int(tok)
         live = sum(1 for i in cur.sampled_items if cur.plan.sequences[i].sequence.status != Status.FINISHED)
         with self._lock:
