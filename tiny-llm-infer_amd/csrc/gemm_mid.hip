@@ -9,7 +9,11 @@
 // A workgroup owns 16*RT*WAVES output columns and one of `splits` contiguous ranges
 // of k.  With splits > 1 it writes float32 partial sums [split][M][N] and a second
 // small kernel adds them in split order (and applies the SwiGLU epilogue for a gated
-// matrix), so the result does not depend on timing.
+// matrix), so the result does not depend on timing.  (Letting the workgroup that
+// finishes last do the sum inside the same kernel was measured and is much slower: the
+// eight L2 caches of the chip are not coherent with each other, so publishing partial
+// sums between workgroups costs a write-back and an invalidation in every workgroup;
+// the kernel boundary does both once.)
 #include "common.h"
 #include <type_traits>
 
@@ -216,11 +220,13 @@ static int launch_mid(const bf16_t* x, const bf16_t* w, void* y, float* part, in
 }
 
 // How many ranges of k a product of this shape is cut into (the caller sizes `part` by it).
-extern "C" int tli_gemm_mid_splits(int N, int K) {
+extern "C" int tli_gemm_mid_splits(int N, int K, int gated) {
     const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
-    const int groups = (n_tiles + 7) / 8;                 // workgroups with RT = 2, WAVES = 4
+    const int per_group = gated ? 8 : 4;                  // tiles a workgroup of the default shape owns
+    const int groups = (n_tiles + per_group - 1) / per_group;
+    const int target = gated ? 192 : (K >= 8192 ? 512 : 256);
     int splits = 1;
-    while (groups * splits < 192 && splits * 2 <= k_steps && splits < 16) splits *= 2;
+    while (groups * splits < target && splits * 2 <= k_steps && splits < 16) splits *= 2;
     return splits;
 }
 
@@ -242,8 +248,10 @@ extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* p
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xp = (const bf16_t*)x;
     const bf16_t* wp = (const bf16_t*)w;
-    if (cfg == 0) cfg = 24;
+    if (cfg == 0) cfg = gated ? 24 : 14;
     switch (cfg) {
+        case 14: if (!gated) return launch_mid<1, 4>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
+                 return tli_fail("gemm_mid: a gated product needs pairs of row tiles");
         case 24: return launch_mid<2, 4>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
         case 28: return launch_mid<2, 8>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
         case 44: return launch_mid<4, 4>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);

@@ -56,7 +56,7 @@ def load_library():
         "tli_gemm_plain": [P, P, P, I, I, I, I, I, I, P],
         "tli_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, I, P],
         "tli_gemm_mid_bf16": [P, P, P, P, I, I, I, I, I, I, I, P],
-        "tli_gemm_mid_splits": [I, I],
+        "tli_gemm_mid_splits": [I, I, I],
         "tli_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
         "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
@@ -223,7 +223,7 @@ class HipOps:
     def _linear_mid(self, x, tiled, y, M, N, K, gated):
         """17..64 rows: the kernel that shares x through LDS, k cut into ranges when the
         output alone gives too few workgroups."""
-        splits = self.mid_splits or self.lib.tli_gemm_mid_splits(N, K)
+        splits = self.mid_splits or self.lib.tli_gemm_mid_splits(N, K, gated)
         part = None
         if splits > 1:
             part = torch.empty((splits * M * N,), dtype=torch.float32, device=self.device)
