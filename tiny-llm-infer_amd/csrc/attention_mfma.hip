@@ -114,8 +114,7 @@ __device__ __forceinline__ void tile_consume(Tile<NJ, ND>& t, const Frag (&ka)[2
             p[u][i] = v;
             mx = fmaxf(mx, v);
         }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = quad_rows_max(mx);
     const float m_new = fmaxf(t.m, mx);
     const float base = (m_new == -INFINITY) ? 0.f : m_new;      // nothing seen yet: all p become 0
     const float corr = __builtin_amdgcn_exp2f(t.m - base);      // exp2(-inf) = 0 on the first block
@@ -130,8 +129,7 @@ __device__ __forceinline__ void tile_consume(Tile<NJ, ND>& t, const Frag (&ka)[2
     Frag pb;
     pb.u = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
                       pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
-    sum += __shfl_xor(sum, 16, 64);
-    sum += __shfl_xor(sum, 32, 64);
+    sum = quad_rows_sum(sum);
     t.l = t.l * corr + sum;
     t.m = m_new;
     // ---- output ----------------------------------------------------------------
@@ -145,6 +143,80 @@ __device__ __forceinline__ void tile_consume(Tile<NJ, ND>& t, const Frag (&ka)[2
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt)
         t.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt].v, pb.v, t.acc[dt], 0, 0, 0);
+}
+
+// The same for CT tiles that share the fragments, in phases (all score MFMAs, then all
+// softmax updates, then all output MFMAs), so that one tile's vector arithmetic can
+// run beside another tile's matrix instructions.
+template <int NJ, int ND, int CT, bool MASK>
+__device__ __forceinline__ void tiles_consume(Tile<NJ, ND> (&tiles)[CT], const Frag (&ka)[2][NJ],
+                                              const Frag (&vt)[ND], int key_c0, int u_stride,
+                                              float scale_log2) {
+    f32x4 s[CT][2];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            s[ct][u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                s[ct][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[u][j].v, tiles[ct].q[j].v, s[ct][u], 0, 0, 0);
+        }
+    Frag pb[CT];
+    float corr[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        Tile<NJ, ND>& t = tiles[ct];
+        float p[2][4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float v = s[ct][u][i] * scale_log2;
+                if (MASK) {
+                    const int key = key_c0 + u * u_stride + i;
+                    v = (key >= t.lo && key <= t.pos) ? v : -INFINITY;
+                } else if (t.pos < 0) {
+                    v = -INFINITY;
+                }
+                p[u][i] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = quad_rows_max(mx);
+        const float m_new = fmaxf(t.m, mx);
+        const float base = (m_new == -INFINITY) ? 0.f : m_new;
+        corr[ct] = __builtin_amdgcn_exp2f(t.m - base);
+        float sum = 0.f;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                p[u][i] = __builtin_amdgcn_exp2f(p[u][i] - base);
+                sum += p[u][i];
+            }
+        pb[ct].u = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
+                              pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
+        sum = quad_rows_sum(sum);
+        t.l = t.l * corr[ct] + sum;
+        t.m = m_new;
+    }
+    bool moved = false;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) moved = moved || corr[ct] != 1.0f;
+    if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) tiles[ct].acc[dt][i] *= corr[ct];
+    }
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+            tiles[ct].acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt].v, pb[ct].v, tiles[ct].acc[dt], 0, 0, 0);
 }
 
 // Process the 32 keys t0 .. t0+31 (t0 a multiple of 32) for CT column tiles that
@@ -404,7 +476,7 @@ __device__ __forceinline__ void prefill_lds_block(
     const bf16_t* __restrict__ v_cache, const int* __restrict__ row_start,
     const int* __restrict__ seq_start, int num_seqs, const int* __restrict__ tables, int table_width,
     int page_size, int page_shift, int num_pages, int heads, int kv_heads, float scale_log2, int window,
-    int rq, int block) {
+    int rq, int block, int head_index) {
     constexpr int HD = ND * 16;
     constexpr int K_PITCH = HD + 8;                   // elements per key row in LDS
     constexpr int V_PITCH = KB + 8;                   // elements per value (dim) row in LDS
@@ -416,7 +488,7 @@ __device__ __forceinline__ void prefill_lds_block(
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
     const int group = heads / kv_heads;
     const int head_tiles = (group + 15) / 16;
-    const int kv_head = blockIdx.y / head_tiles, head_tile = blockIdx.y % head_tiles;
+    const int kv_head = head_index / head_tiles, head_tile = head_index % head_tiles;
     const int heads_here = min(16, group - head_tile * 16);
     const int rows_per_wave = CT * rq, rows_per_block = 4 * rows_per_wave;
     int seq = 0, first_row = 0, n_rows = 0;
@@ -536,13 +608,10 @@ __device__ __forceinline__ void prefill_lds_block(
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt)
                 vt[dt].u = *reinterpret_cast<const uint4*>(vs + dt * 16 * V_PITCH + vt_off + sub * 32);
-            if (s0 >= full_lo && s0 + 31 <= full_hi) {
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct) tile_consume<NJ, ND, false>(t[ct], ka, vt, s0 + 8 * c, 4, scale_log2);
-            } else {
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct) tile_consume<NJ, ND, true>(t[ct], ka, vt, s0 + 8 * c, 4, scale_log2);
-            }
+            if (s0 >= full_lo && s0 + 31 <= full_hi)
+                tiles_consume<NJ, ND, CT, false>(t, ka, vt, s0 + 8 * c, 4, scale_log2);
+            else
+                tiles_consume<NJ, ND, CT, true>(t, ka, vt, s0 + 8 * c, 4, scale_log2);
         }
     }
 
@@ -577,16 +646,42 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
     int total = 0;
     for (int seq = 0; seq < num_seqs; ++seq)
         total += (row_start[seq + 1] - row_start[seq] + rows_per_block - 1) / rows_per_block;
+    const int head_count = gridDim.y;
+    if (pair == 2) {
+        // All workgroups are resident at once, two a compute unit, and late row blocks walk
+        // more keys than early ones.  Workgroups are handed to the compute units in order
+        // of their linear index, so index L and index L + total/2 tend to share a unit: the
+        // second half of the indices gets the row blocks in reverse order (and the other
+        // half of the heads), which puts a long block beside a short one.
+        const int all = total * head_count, half = all / 2;
+        const int linear = blockIdx.y * gridDim.x + blockIdx.x;
+        if (blockIdx.x >= total) return;                       // the grid's slack
+        const int lin = blockIdx.y * total + blockIdx.x;       // index among the real workgroups
+        int rb, hd_i;
+        if (head_count % 2 == 0) {
+            const int round = lin / half, p = lin % half;
+            rb = round == 0 ? p % total : total - 1 - p % total;
+            hd_i = p / total + round * (head_count / 2);
+        } else {
+            rb = blockIdx.x;
+            hd_i = blockIdx.y;
+        }
+        (void)linear;
+        prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+                                          table_width, page_size, page_shift, num_pages, heads, kv_heads,
+                                          scale_log2, window, rq, rb, hd_i);
+        return;
+    }
     const int first = blockIdx.x, second = pair ? total - 1 - first : first;
     if (first >= total || first > second) return;
     prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                       table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                      scale_log2, window, rq, second);
+                                      scale_log2, window, rq, second, blockIdx.y);
     if (second != first) {
         __syncthreads();
         prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                           table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                          scale_log2, window, rq, first);
+                                          scale_log2, window, rq, first, blockIdx.y);
     }
 }
 
@@ -683,12 +778,13 @@ extern "C" int tli_attention_prefill_bf16(
         // long enough to fill the chip that way; blocks of 64 keys (32 for large heads)
         bool two = head_dim <= 128 && (long)rows * kv_heads * head_tiles >= (long)8 * rq * 512;
         if (direct == 2) two = false;
-        if (direct == 3) two = head_dim <= 128;
+        if (direct == 3 || direct >= 4) two = head_dim <= 128;
         const int rows_per_block = 4 * rq * (two ? 2 : 1);
         const long blocks = (rows + rows_per_block - 1) / rows_per_block + num_seqs;   // upper bound
         if (blocks > 2147483647L) return tli_fail("attention_prefill: too many rows");
-        const int pair = blocks * kv_heads * head_tiles >= 1024 ? 1 : 0;
-        dim3 grid((unsigned)(pair ? (blocks + 1) / 2 : blocks), kv_heads * head_tiles);
+        int pair = blocks * kv_heads * head_tiles >= 1024 ? 1 : 2;
+        if (direct >= 4) pair = direct - 4;               // measurements: 4, 5, 6 force the pairing mode
+        dim3 grid((unsigned)(pair == 1 ? (blocks + 1) / 2 : blocks), kv_heads * head_tiles);
         const int kb = head_dim <= 128 ? 64 : 32;
         const size_t lds = ((size_t)kb * (head_dim + 8) + (size_t)head_dim * (kb + 8)) * sizeof(bf16_t);
 #define ARGS (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, row_start, \

@@ -46,6 +46,30 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Maximum / sum over the four lanes l, l^16, l^32, l^48 (the lane groups of an MFMA
+// tile), every lane gets the result.  v_permlane16_swap / v_permlane32_swap exchange
+// rows of 16 (halves of 32) lanes between two registers without going through LDS:
+// with both operands holding x, one result has the even rows (lower half) twice and the
+// other the odd rows (upper half) twice, so combining the two is the exchange with l^16
+// (l^32) done for every lane at once.
+__device__ __forceinline__ float quad_rows_max(float x) {
+    const uint32_t u = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const float m = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const uint32_t v = __float_as_uint(m);
+    const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+__device__ __forceinline__ float quad_rows_sum(float x) {
+    const uint32_t u = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const float m = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const uint32_t v = __float_as_uint(m);
+    const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = TLI_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, TLI_WAVE);
