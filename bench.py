@@ -1,5 +1,5 @@
 """Serving benchmark on one MI355X: decode tokens a second of a Qwen3-8B-shaped
-model with random bfloat16 weights (BASELINE.json configs[2]), plus the prefill
+model with random bfloat16 weights (the layer sizes of Qwen3-8B), plus the prefill
 of one 2,048-token prompt and decode at batch 1 and 64.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]

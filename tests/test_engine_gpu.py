@@ -1,5 +1,5 @@
 """Generation through the entry points on the GPU: the Python engine and the
-command line, greedy against the plain implementation, the BASELINE workloads
+command line, greedy against the plain implementation, the small serving workloads
 of the two tiny configurations, and top-p sampling against a plain version."""
 import os
 import subprocess

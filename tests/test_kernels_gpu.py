@@ -131,7 +131,7 @@ def test_skinny_linear_against_plain_kernel_and_reference(ops, mnk, out):
         assert torch.equal(streamed, got)      # same additions in the same order, other addresses
     else:                                      # 17..64 rows: the kernel that shares x through LDS
         assert float((streamed.double().cpu() - want).abs().max()) <= bound
-        for splits, cfg in ((1, 24), (2, 28), (4, 44), (3, 48)):
+        for splits, cfg in ((1, 224), (2, 228), (4, 314), (3, 418), (5, 424), (7, 218)):
             ops.mid_splits, ops.mid_cfg = splits, cfg
             try:
                 again = ops.linear(xd, Both, out_dtype=out)

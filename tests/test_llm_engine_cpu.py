@@ -19,7 +19,7 @@ def _engine(folder, name, **kw):
 
 
 def test_greedy_generation_matches_plain(model_folders):
-    """BASELINE workload of configuration A: prompts of 5/17/33 tokens, 16
+    """Small serving workload of configuration A: prompts of 5/17/33 tokens, 16
     greedy tokens each, page 8, budget 24."""
     folder = model_folders["A"]
     cfg, w = plain_qwen3.read_model(folder)

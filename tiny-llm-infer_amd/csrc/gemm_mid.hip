@@ -28,19 +28,26 @@ union Pack16m {
 #define MID_ROWS 64
 #define MID_XPITCH (128 + 8)        // elements per staged x row: 272 bytes
 
-template <int RT, int WAVES, typename TO, bool GATED>
+template <int RT, int WAVES, int DEPTH, typename TO, bool GATED>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* __restrict__ y,
                 float* __restrict__ part, int M, int N, int K, int splits, int steps_per_split) {
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][MID_ROWS][MID_XPITCH];
     constexpr int THREADS = WAVES * 64;
     constexpr int CHUNKS = MID_ROWS * 16 / THREADS;          // 16-byte chunks of a slice a thread stages
+    constexpr int STAGES = DEPTH + 1;                        // register stages: DEPTH fetches in flight, one in use
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
     const int k_steps = (K + 127) / 128;
     const int tile0 = (blockIdx.x * WAVES + wave) * RT;       // this wave's first 16-column tile
     const int n_tiles = (N + 15) / 16;
     const int step_begin = blockIdx.y * steps_per_split;
     const int step_end = min(k_steps, step_begin + steps_per_split);
+    // Workgroups walk their k range from different starting slices, wrapping round: a
+    // slice of x is 64 rows a power of two apart, which all lie in one channel of the L2
+    // cache, and workgroups in step would all wait for that one channel.  (Workgroups go
+    // round the eight dies in turn, so neighbours on a die are blockIdx.x / 8 apart.)
+    const int rot = step_begin < step_end ? (blockIdx.x / 8) % (step_end - step_begin) : 0;
+    auto at = [&](int step) { return step + rot < step_end ? step + rot : step + rot - (step_end - step_begin); };
 
     f32x4 acc[RT][4];
 #pragma unroll
@@ -50,47 +57,66 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
 
     // W fragments straight from the decode layout: block (tile, step) is 2048 elements,
     // fragment j of this lane at j*512 + lane*8
+    // (a tile past the last one reads tile 0 instead: its columns are never stored.  No
+    // load below is predicated: a branch around a load makes the compiler wait for every
+    // load in flight at the next use, which would undo the prefetching)
     const bf16_t* w_tile[RT];
-    bool w_ok[RT];
 #pragma unroll
-    for (int t = 0; t < RT; ++t) {
-        w_ok[t] = tile0 + t < n_tiles;
-        w_tile[t] = w + (size_t)(w_ok[t] ? tile0 + t : 0) * k_steps * 2048 + lane * 8;
-    }
-    // Three register stages for the fetched W fragments and x chunks (two fetches are in
-    // flight while a slice is multiplied), two LDS buffers for the staged x slices.
+    for (int t = 0; t < RT; ++t)
+        w_tile[t] = w + (size_t)(tile0 + t < n_tiles ? tile0 + t : 0) * k_steps * 2048 + lane * 8;
+    // W fragments and the slices of x (the first workgroup of a die to ask for a slice
+    // gets it from memory, not from L2) are fetched DEPTH slices ahead into a ring of
+    // register stages; a slice of x is written to the LDS buffer that is free one slice
+    // before its use.  Loads complete in the order of issue, so the x fetch of a slice is
+    // issued before its W fetch: the wait for an x chunk never waits for W fragments
+    // that were asked for later.
     // x staging plan: chunk e of this thread is row (tid + e*THREADS) / 16, 16-byte column (..) % 16
-    Pack16m a[3][RT][4];
-    uint4 xreg[3][CHUNKS];
-    auto fetch = [&](int step, auto STAGE) {
+    Pack16m a[STAGES][RT][4];
+    uint4 xreg[STAGES][CHUNKS];
+    auto fetch_w = [&](int logical, auto STAGE) {
         constexpr int S = decltype(STAGE)::value;
+        const int step = at(logical);
 #pragma unroll
         for (int t = 0; t < RT; ++t)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                a[S][t][j].u = w_ok[t] ? *reinterpret_cast<const uint4*>(w_tile[t] + (size_t)step * 2048 + j * 512)
-                                       : make_uint4(0, 0, 0, 0);
+                a[S][t][j].u = *reinterpret_cast<const uint4*>(w_tile[t] + (size_t)step * 2048 + j * 512);
+    };
+    auto fetch_x = [&](int logical, auto STAGE) {
+        constexpr int S = decltype(STAGE)::value;
+        const int step = at(logical);
+#pragma unroll
+        for (int e = 0; e < CHUNKS; ++e) {
+            // rows past M repeat the last row (never stored); columns past K read column 0 and are zeroed when staged
+            const int idx = tid + e * THREADS;
+            const int row = min(idx / 16, M - 1), k = step * 128 + (idx % 16) * 8;
+            xreg[S][e] = *reinterpret_cast<const uint4*>(x + (size_t)row * K + (k < K ? k : 0));
+        }
+    };
+    auto stage = [&](int logical, int buf, auto STAGE) {
+        constexpr int S = decltype(STAGE)::value;
+        const int step = at(logical);
 #pragma unroll
         for (int e = 0; e < CHUNKS; ++e) {
             const int idx = tid + e * THREADS;
-            const int row = idx / 16, k = step * 128 + (idx % 16) * 8;
-            xreg[S][e] = (row < M && k < K) ? *reinterpret_cast<const uint4*>(x + (size_t)row * K + k)
-                                            : make_uint4(0, 0, 0, 0);
+            unsigned keep = step * 128 + (idx % 16) * 8 < K ? 0xffffffffu : 0u;
+            asm volatile("" : "+v"(keep));       // opaque, or the load is moved under a branch on it
+            const uint4 v = xreg[S][e];
+            *reinterpret_cast<uint4*>(&xs[buf][idx / 16][(idx % 16) * 8]) =
+                make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
         }
     };
-    auto stage = [&](int buf, auto STAGE) {
+    // one slice: `step` is multiplied from register stage S and LDS buffer `buf`.  FULL: every
+    // fetch of this slice exists, so none is under a branch (after a branch that may have
+    // issued loads the compiler waits as if it had not, that is for all of them)
+    auto slice = [&](int step, int buf, auto STAGE, auto FULL_T) {
         constexpr int S = decltype(STAGE)::value;
-#pragma unroll
-        for (int e = 0; e < CHUNKS; ++e) {
-            const int idx = tid + e * THREADS;
-            *reinterpret_cast<uint4*>(&xs[buf][idx / 16][(idx % 16) * 8]) = xreg[S][e];
-        }
-    };
-    // one slice: `step` is multiplied from register stage S and LDS buffer `buf`
-    auto slice = [&](int step, int buf, auto STAGE) {
-        constexpr int S = decltype(STAGE)::value;
+        constexpr bool FULL = decltype(FULL_T)::value;
         __syncthreads();                                   // slice `buf` is staged; the other is free
-        if (step + 2 < step_end) fetch(step + 2, std::integral_constant<int, (S + 2) % 3>{});
+        if (FULL || step + DEPTH < step_end) {
+            fetch_x(step + DEPTH, std::integral_constant<int, (S + DEPTH) % STAGES>{});
+            fetch_w(step + DEPTH, std::integral_constant<int, (S + DEPTH) % STAGES>{});
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             Pack16m b[4];
@@ -104,20 +130,37 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
                     acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[S][t][j].v, b[m].v, acc[t][m], 0, 0, 0);
         }
         // nobody reads the other buffer before the next barrier
-        if (step + 1 < step_end) stage(buf ^ 1, std::integral_constant<int, (S + 1) % 3>{});
+        if (FULL || step + 1 < step_end) stage(step + 1, buf ^ 1, std::integral_constant<int, (S + 1) % STAGES>{});
+    };
+    auto slices = [&](auto self, int step, int b0, auto INDEX, auto FULL_T) -> void {
+        constexpr int I = decltype(INDEX)::value;
+        if constexpr (I < STAGES) {
+            if (decltype(FULL_T)::value || step + I < step_end) {
+                slice(step + I, b0 ^ (I & 1), std::integral_constant<int, I>{}, FULL_T);
+                self(self, step, b0, std::integral_constant<int, I + 1>{}, FULL_T);
+            }
+        }
+    };
+    auto prologue = [&](auto self, auto INDEX) -> void {
+        constexpr int I = decltype(INDEX)::value;
+        if constexpr (I < DEPTH) {
+            if (step_begin + I < step_end) {
+                fetch_x(step_begin + I, std::integral_constant<int, I>{});
+                fetch_w(step_begin + I, std::integral_constant<int, I>{});
+            }
+            self(self, std::integral_constant<int, I + 1>{});
+        }
     };
 
     if (step_begin < step_end) {
-        fetch(step_begin, std::integral_constant<int, 0>{});
-        if (step_begin + 1 < step_end) fetch(step_begin + 1, std::integral_constant<int, 1>{});
-        stage(0, std::integral_constant<int, 0>{});
+        prologue(prologue, std::integral_constant<int, 0>{});
+        stage(step_begin, 0, std::integral_constant<int, 0>{});
     }
-    for (int step = step_begin; step < step_end; step += 3) {
-        const int b0 = (step - step_begin) & 1;
-        slice(step, b0, std::integral_constant<int, 0>{});
-        if (step + 1 < step_end) slice(step + 1, b0 ^ 1, std::integral_constant<int, 1>{});
-        if (step + 2 < step_end) slice(step + 2, b0, std::integral_constant<int, 2>{});
-    }
+    int step = step_begin;
+    for (; step + STAGES - 1 + DEPTH < step_end; step += STAGES)
+        slices(slices, step, (step - step_begin) & 1, std::integral_constant<int, 0>{}, std::true_type{});
+    for (; step < step_end; step += STAGES)
+        slices(slices, step, (step - step_begin) & 1, std::integral_constant<int, 0>{}, std::false_type{});
 
     // lane holds y[m*16 + r][tile*16 + 4c + i]
     if (splits > 1) {
@@ -194,18 +237,18 @@ __global__ void gemm_mid_reduce_kernel(const float* __restrict__ part, TO* __res
     }
 }
 
-template <int RT, int WAVES>
+template <int RT, int WAVES, int DEPTH>
 static int launch_mid(const bf16_t* x, const bf16_t* w, void* y, float* part, int M, int N, int K,
                       int y_dtype, int gated, int splits, hipStream_t s) {
     const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
     const int steps_per_split = (k_steps + splits - 1) / splits;
     dim3 grid((n_tiles + RT * WAVES - 1) / (RT * WAVES), splits);
     if (gated)
-        gemm_mid_kernel<RT, WAVES, bf16_t, true><<<grid, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, part, M, N, K, splits, steps_per_split);
+        gemm_mid_kernel<RT, WAVES, DEPTH, bf16_t, true><<<grid, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, part, M, N, K, splits, steps_per_split);
     else if (y_dtype == TLI_BF16)
-        gemm_mid_kernel<RT, WAVES, bf16_t, false><<<grid, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, part, M, N, K, splits, steps_per_split);
+        gemm_mid_kernel<RT, WAVES, DEPTH, bf16_t, false><<<grid, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, part, M, N, K, splits, steps_per_split);
     else
-        gemm_mid_kernel<RT, WAVES, float, false><<<grid, WAVES * 64, 0, s>>>(x, w, (float*)y, part, M, N, K, splits, steps_per_split);
+        gemm_mid_kernel<RT, WAVES, DEPTH, float, false><<<grid, WAVES * 64, 0, s>>>(x, w, (float*)y, part, M, N, K, splits, steps_per_split);
     if (tli_check_launch("gemm_mid")) return 1;
     if (splits > 1) {
         const size_t total = (size_t)M * (gated ? N / 2 : N);
@@ -219,21 +262,25 @@ static int launch_mid(const bf16_t* x, const bf16_t* w, void* y, float* part, in
     return 0;
 }
 
+// Launch shape by measurement on MI355X (4096..151936 columns, k of 4096 and 12288): two
+// column tiles a wave once that still leaves about 192 workgroups, else one; k is cut into
+// ranges until there are about 192 workgroups.
+static int mid_tiles_per_wave(int N, int gated) { return gated || (N + 15) / 16 >= 8 * 192 ? 2 : 1; }
+
 // How many ranges of k a product of this shape is cut into (the caller sizes `part` by it).
 extern "C" int tli_gemm_mid_splits(int N, int K, int gated) {
     const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
-    const int per_group = gated ? 8 : 4;                  // tiles a workgroup of the default shape owns
+    const int per_group = 4 * mid_tiles_per_wave(N, gated);
     const int groups = (n_tiles + per_group - 1) / per_group;
-    const int target = gated ? 192 : (K >= 8192 ? 512 : 256);
     int splits = 1;
-    while (groups * splits < target && splits * 2 <= k_steps && splits < 16) splits *= 2;
+    while (groups * splits < 192 && splits * 2 <= k_steps && splits < 16) splits *= 2;
     return splits;
 }
 
 // y[M,N] = x[M,K] . W^T for 1 <= M <= 64, W in the decode layout (`gated` as tiled = 2 of
 // tli_gemm_skinny_bf16: y is [M, N/2] bfloat16).  `part`: splits*M*N floats when
 // splits > 1 (splits as returned by tli_gemm_mid_splits, or forced by the caller);
-// cfg 0 picks the launch shape, else RT*10 + WAVES.
+// cfg 0 picks the launch shape, else DEPTH*100 + RT*10 + WAVES.
 extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* part, int M, int N, int K,
                                  int y_dtype, int gated, int splits, int cfg, void* stream) {
     if (M <= 0 || N <= 0) return 0;
@@ -248,14 +295,12 @@ extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* p
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xp = (const bf16_t*)x;
     const bf16_t* wp = (const bf16_t*)w;
-    if (cfg == 0) cfg = gated ? 24 : 14;
+    if (cfg == 0) cfg = 204 + 10 * mid_tiles_per_wave(N, gated);
+    if (gated && (cfg / 10) % 10 < 2) return tli_fail("gemm_mid: a gated product needs pairs of row tiles");
+#define MID_CASE(D, R, W) case D * 100 + R * 10 + W: return launch_mid<R, W, D>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
     switch (cfg) {
-        case 14: if (!gated) return launch_mid<1, 4>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
-                 return tli_fail("gemm_mid: a gated product needs pairs of row tiles");
-        case 24: return launch_mid<2, 4>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
-        case 28: return launch_mid<2, 8>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
-        case 44: return launch_mid<4, 4>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
-        case 48: return launch_mid<4, 8>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
+        MID_CASE(2, 1, 4) MID_CASE(3, 1, 4) MID_CASE(2, 1, 8) MID_CASE(4, 1, 8)
+        MID_CASE(2, 2, 4) MID_CASE(4, 2, 4) MID_CASE(2, 2, 8)
         default: return tli_fail("gemm_mid: unknown configuration %d", cfg);
     }
 }

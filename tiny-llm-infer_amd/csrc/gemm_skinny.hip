@@ -48,6 +48,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
 #pragma unroll
         for (int m = 0; m < MT; ++m) acc[t][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
+    // Rows past the end read a valid row instead (w: row 0, x: the last row) and are
+    // never stored, so that no load of the main loop is predicated.
     const bf16_t* w_row[RT];
     bool w_ok[RT];
 #pragma unroll
@@ -60,32 +62,30 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
             w_row[t] = w + ((size_t)(blockIdx.x * RT + t) * ((K + 127) / 128)) * 2048 + lane * 8;
     }
     const bf16_t* x_row[MT];
-    bool x_ok[MT];
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
-        const int row = m * 16 + r;
-        x_ok[m] = row < M;
-        x_row[m] = x + (size_t)(x_ok[m] ? row : 0) * K;
-    }
+    for (int m = 0; m < MT; ++m) x_row[m] = x + (size_t)min(m * 16 + r, M - 1) * K;
 
-    // DEPTH-stage pipeline: the loads of the next DEPTH-1 128-wide steps are in flight
-    // while the MFMAs of the current one run, so a wave keeps up to
-    // 4*(RT+MT)*(DEPTH-1) 16-byte loads in flight
+    // Ring of DEPTH register stages: the loads of the next DEPTH-1 128-wide steps are in
+    // flight while the MFMAs of the current one run, so a wave keeps up to
+    // 4*(RT+MT)*(DEPTH-1) 16-byte loads in flight.  The main loop takes whole steps only
+    // and none of its loads is under a branch: after a branch that may have issued loads
+    // the compiler waits for all loads in flight, which would undo the prefetching.
     Pack16 a[DEPTH][RT][4], b[DEPTH][MT][4];
     auto load_step = [&](auto STAGE, int kb) {
         constexpr int S = decltype(STAGE)::value;
         const int k = kb + c * 32;
-#pragma unroll
-        for (int t = 0; t < RT; ++t)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                a[S][t][j].u = TILED ? *reinterpret_cast<const uint4*>(w_row[t] + (size_t)(kb / 128) * 2048 + j * 512)
-                                     : load16_or_zero(w_row[t] + k + j * 8, w_ok[t] && (k + j * 8 < K));
+        // x first: it comes from L2 and loads complete in the order of issue
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                b[S][m][j].u = load16_or_zero(x_row[m] + k + j * 8, x_ok[m] && (k + j * 8 < K));
+                b[S][m][j].u = *reinterpret_cast<const uint4*>(x_row[m] + k + j * 8);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int t = 0; t < RT; ++t)
+                a[S][t][j].u = TILED ? *reinterpret_cast<const uint4*>(w_row[t] + (size_t)(kb / 128) * 2048 + j * 512)
+                                     : *reinterpret_cast<const uint4*>(w_row[t] + k + j * 8);
     };
     auto mma_step = [&](auto STAGE) {
         constexpr int S = decltype(STAGE)::value;
@@ -97,30 +97,57 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
                 for (int m = 0; m < MT; ++m)
                     acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[S][t][j].v, b[S][m][j].v,
                                                                         acc[t][m], 0, 0, 0);
+        // keeps the scheduler from moving the loads of the next step (issued after this
+        // in program order) ahead of these products, where they would have to be waited
+        // for together with the operands used here
+        __builtin_amdgcn_sched_barrier(0);
     };
-    constexpr int STRIDE = WAVES * 128;
-    const int kb0 = wave * 128;
-    // prologue: stages 0 .. DEPTH-2
-    if (kb0 < K) load_step(std::integral_constant<int, 0>{}, kb0);
-    if (DEPTH > 2 && kb0 + STRIDE < K) load_step(std::integral_constant<int, 1 % DEPTH>{}, kb0 + STRIDE);
-    if (DEPTH > 3 && kb0 + 2 * STRIDE < K) load_step(std::integral_constant<int, 2 % DEPTH>{}, kb0 + 2 * STRIDE);
-    for (int kb = kb0; kb < K; kb += DEPTH * STRIDE) {
-        // step s of this round multiplies stage s and refills stage (s + DEPTH - 1) % DEPTH
-        if (kb + (DEPTH - 1) * STRIDE < K)
-            load_step(std::integral_constant<int, (DEPTH - 1) % DEPTH>{}, kb + (DEPTH - 1) * STRIDE);
+    // this wave's whole steps: number i is at k = (wave + i*WAVES) * 128
+    const int whole = K / 128;
+    const int mine = wave < whole ? (whole - wave + WAVES - 1) / WAVES : 0;
+    auto k_of = [&](int i) { return (wave + i * WAVES) * 128; };
+    auto prologue = [&](auto self, auto INDEX) -> void {
+        constexpr int I = decltype(INDEX)::value;
+        if constexpr (I < DEPTH - 1) {
+            if (I < mine) load_step(std::integral_constant<int, I>{}, k_of(I));
+            self(self, std::integral_constant<int, I + 1>{});
+        }
+    };
+    // a round: step i + I multiplies stage I after the load of step i + I + DEPTH - 1 went out
+    auto round = [&](auto self, int i, auto INDEX, auto FULL_T) -> void {
+        constexpr int I = decltype(INDEX)::value;
+        constexpr bool FULL = decltype(FULL_T)::value;
+        if constexpr (I < DEPTH) {
+            if (FULL || i + I < mine) {
+                if (FULL || i + I + DEPTH - 1 < mine)
+                    load_step(std::integral_constant<int, (I + DEPTH - 1) % DEPTH>{}, k_of(i + I + DEPTH - 1));
+                __builtin_amdgcn_sched_barrier(0);
+                mma_step(std::integral_constant<int, I>{});
+                self(self, i, std::integral_constant<int, I + 1>{}, FULL_T);
+            }
+        }
+    };
+    prologue(prologue, std::integral_constant<int, 0>{});
+    int i = 0;
+    for (; i + 2 * (DEPTH - 1) < mine; i += DEPTH)
+        round(round, i, std::integral_constant<int, 0>{}, std::true_type{});
+    for (; i < mine; i += DEPTH)
+        round(round, i, std::integral_constant<int, 0>{}, std::false_type{});
+    // the last, partial step of k belongs to the wave whose turn it is; it comes after
+    // that wave's whole steps, as it would in one loop over all steps
+    if (K % 128 && wave == whole % WAVES) {
+        const int k = whole * 128 + c * 32;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool in = k + j * 8 < K;
+#pragma unroll
+            for (int t = 0; t < RT; ++t)
+                a[0][t][j].u = TILED ? *reinterpret_cast<const uint4*>(w_row[t] + (size_t)whole * 2048 + j * 512)
+                                     : load16_or_zero(w_row[t] + k + j * 8, in);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) b[0][m][j].u = load16_or_zero(x_row[m] + k + j * 8, in);
+        }
         mma_step(std::integral_constant<int, 0>{});
-        if (kb + STRIDE < K) {
-            if (kb + DEPTH * STRIDE < K) load_step(std::integral_constant<int, 0>{}, kb + DEPTH * STRIDE);
-            mma_step(std::integral_constant<int, 1 % DEPTH>{});
-        }
-        if (DEPTH > 2 && kb + 2 * STRIDE < K) {
-            if (kb + (DEPTH + 1) * STRIDE < K) load_step(std::integral_constant<int, 1 % DEPTH>{}, kb + (DEPTH + 1) * STRIDE);
-            mma_step(std::integral_constant<int, 2 % DEPTH>{});
-        }
-        if (DEPTH > 3 && kb + 3 * STRIDE < K) {
-            if (kb + (DEPTH + 2) * STRIDE < K) load_step(std::integral_constant<int, 2 % DEPTH>{}, kb + (DEPTH + 2) * STRIDE);
-            mma_step(std::integral_constant<int, 3 % DEPTH>{});
-        }
     }
 
 #pragma unroll
