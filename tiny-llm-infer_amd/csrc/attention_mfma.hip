@@ -3,7 +3,8 @@
 //
 //   decode:  every sequence brings one row.  A workgroup owns one (sequence, kv
 //            head, key split); its four waves take the 32-key blocks of the
-//            split in turn and are merged through LDS; splits are merged by a
+//            split in turn, each asking for its next block before it multiplies
+//            the current one, and are merged through LDS; splits are merged by a
 //            second small kernel.
 //   prefill: sequences bring portions of prompts (and single rows beside them).
 //            A workgroup owns up to 4*RQ consecutive rows of one sequence and
@@ -269,6 +270,53 @@ __device__ __forceinline__ void tile_step(Tile<NJ, ND>& t, const CacheView& cv, 
 }
 
 // --------------------------------------------------------------------- decode --
+// The fragments of one block of 32 keys, as tile_consume takes them.
+template <int NJ, int ND>
+struct KeyBlock {
+    Frag ka[2][NJ];
+    Frag vt[ND];
+};
+
+// Ask for the 32 keys t0 .. t0+31 (same lane-to-key plan as tiles_step).  `seg` holds the
+// block table entries seg_first .. seg_first+seg_len-1 in LDS.  No load is predicated, so
+// that the fragments of the next block can be in flight while this one is multiplied
+// (after a branch that may have issued loads the compiler waits for all loads in flight):
+// a key without a page reads page 0 instead.  Such keys lie outside lo..pos, their
+// scores are masked, and their values meet a weight of exactly 0; the cache is allocated
+// zeroed, so they are finite.
+template <int NJ, int ND>
+__device__ __forceinline__ void decode_fetch(KeyBlock<NJ, ND>& b, const CacheView& cv, const int* seg,
+                                             int seg_first, int seg_len, int t0) {
+    const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
+    auto page_at = [&](int key) {
+        const int rel = (key >> cv.page_shift) - seg_first;          // >= 0: t0 is not before the split
+        const int page = seg[min(rel, seg_len - 1)];
+        return (unsigned)page < (unsigned)cv.num_pages ? page : 0;
+    };
+    const int in_page = cv.page_size - 1;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const int key = t0 + u * 16 + r;
+        const bf16_t* kp = cv.k + (((size_t)page_at(key) * cv.kv_heads + cv.kv_head) * cv.page_size +
+                                   (key & in_page)) * cv.head_dim;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int d = c * 8 * NJ + j * 8;                        // past head_dim the query is zero
+            b.ka[u][j].u = *reinterpret_cast<const uint4*>(kp + (d < cv.head_dim ? d : 0));
+        }
+    }
+    const int key_a = t0 + 4 * c, key_b = t0 + 16 + 4 * c;
+    const size_t head_stride = (size_t)cv.head_dim * cv.page_size;
+    const bf16_t* va = cv.v + ((size_t)page_at(key_a) * cv.kv_heads + cv.kv_head) * head_stride + (key_a & in_page);
+    const bf16_t* vb = cv.v + ((size_t)page_at(key_b) * cv.kv_heads + cv.kv_head) * head_stride + (key_b & in_page);
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) {
+        const size_t off = (size_t)(dt * 16 + r) * cv.page_size;
+        b.vt[dt].h[0] = *reinterpret_cast<const uint2*>(va + off);
+        b.vt[dt].h[1] = *reinterpret_cast<const uint2*>(vb + off);
+    }
+}
+
 // grid (splits, kv_heads * head_tiles, rows); 256 threads
 template <int NJ, int ND>
 __global__ void __launch_bounds__(256)
@@ -278,7 +326,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
                         const int* __restrict__ tables, int table_width, int page_size, int page_shift,
                         int num_pages, int heads, int kv_heads, int head_dim, float scale, int window,
                         int splits, int keys_per_split) {
-    extern __shared__ float lds[];       // 3 waves x 64 lanes x (ND*4 + 2)
+    extern __shared__ float lds[];       // 3 waves x 64 lanes x (ND*4 + 2), then this split's table entries
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, c = lane / 16;
     const int split = blockIdx.x, row = blockIdx.z;
     const int group = heads / kv_heads;
@@ -289,9 +337,10 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     const int head = kv_head * group + col_head;
     const int pos = positions[row];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int* table = tables + (size_t)seq_of_row[row] * table_width;
 
-    CacheView cv{k_cache, v_cache, tables + (size_t)seq_of_row[row] * table_width, table_width, page_size,
-                 page_shift, num_pages, kv_heads, head_dim, kv_head};
+    CacheView cv{k_cache, v_cache, table, table_width, page_size, page_shift, num_pages, kv_heads, head_dim,
+                 kv_head};
     Tile<NJ, ND> t;
     tile_init(t);
     t.pos = live ? pos : -1;
@@ -302,7 +351,37 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     const int first_block = lo / 32;
     const int begin = first_block * 32 + split * keys_per_split;
     const int end = min(pos + 1, begin + keys_per_split);
-    for (int t0 = begin + wave * 32; t0 < end; t0 += 4 * 32) tile_step(t, cv, t0, scale);
+    // its part of the block table goes to LDS once, so that a block's addresses do not
+    // wait for a table entry from memory first
+    int* seg = reinterpret_cast<int*>(lds + 3 * 64 * (ND * 4 + 2));
+    const int seg_first = begin >> page_shift;
+    const int seg_len = begin < end ? ((end - 1) >> page_shift) - seg_first + 1 : 0;
+    for (int i = threadIdx.x; i < seg_len; i += 256)
+        seg[i] = seg_first + i < table_width ? table[seg_first + i] : -1;
+    __syncthreads();
+
+    // a wave's blocks are 128 keys apart; the next block is asked for before this one is
+    // multiplied (the last block is asked for once more instead of branching round the loads)
+    int t0 = begin + wave * 32;
+    if (t0 < end) {
+        const int last = t0 + (end - 1 - t0) / 128 * 128;
+        KeyBlock<NJ, ND> b0, b1;
+        decode_fetch(b0, cv, seg, seg_first, seg_len, t0);
+        while (true) {
+            decode_fetch(b1, cv, seg, seg_first, seg_len, min(t0 + 128, last));
+            __builtin_amdgcn_sched_barrier(0);
+            tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 4 * c, 16, scale);
+            __builtin_amdgcn_sched_barrier(0);
+            if (t0 + 128 > last) break;
+            t0 += 128;
+            decode_fetch(b0, cv, seg, seg_first, seg_len, min(t0 + 128, last));
+            __builtin_amdgcn_sched_barrier(0);
+            tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, t0 + 4 * c, 16, scale);
+            __builtin_amdgcn_sched_barrier(0);
+            if (t0 + 128 > last) break;
+            t0 += 128;
+        }
+    }
 
     // merge the four waves: waves 1..3 hand over (m, l, acc), wave 0 combines in wave order
     const int stride = ND * 4 + 2;
@@ -744,8 +823,13 @@ extern "C" int tli_attention_decode_bf16(
     const int group = heads / kv_heads, head_tiles = (group + 15) / 16;
     dim3 grid(splits, kv_heads * head_tiles, rows);
     const int shift = log2_exact(page_size);
+    // the table entries of one split are kept in LDS
+    const size_t seg_bytes = ((size_t)(keys_per_split >> shift) + 2) * sizeof(int);
+    if (seg_bytes > 8192)
+        return tli_fail("attention_decode: %d keys per split in pages of %d are more than 2046 pages; use more splits",
+                        keys_per_split, page_size);
 #define CALL(NJ, ND)                                                                                    \
-    attention_decode_kernel<NJ, ND><<<grid, 256, 3 * 64 * (ND * 4 + 2) * sizeof(float), s>>>(           \
+    attention_decode_kernel<NJ, ND><<<grid, 256, 3 * 64 * (ND * 4 + 2) * sizeof(float) + seg_bytes, s>>>( \
         (const bf16_t*)q, (bf16_t*)out, partial, (const bf16_t*)k_cache, (const bf16_t*)v_cache,        \
         positions, seq_of_row, tables, table_width, page_size, shift, num_pages, heads, kv_heads,       \
         head_dim, scale * LOG2E, window, splits, keys_per_split)

@@ -342,6 +342,8 @@ class HipOps:
         groups = T * kv_heads * ((heads // kv_heads + 15) // 16)
         # a split costs a merge pass: only worth it when a workgroup would walk many keys
         splits = max(1, min((self.DECODE_WORKGROUPS + groups - 1) // groups, reach // 512, 64))
+        # (a split's block table entries are kept in LDS: at most 2046 pages a split)
+        splits = max(splits, -(-reach // (2046 * g.page_size // 128 * 128)))
         per_split = ((reach + splits - 1) // splits + 127) // 128 * 128
         splits = (reach + per_split - 1) // per_split
         partial = None
