@@ -99,7 +99,9 @@ def main():
 
     def decode_run(batch, steps, warmup):
         """Prefill ``batch`` prompts, then time ``steps`` decode steps."""
-        params = SamplingParams(max_tokens=steps + warmup + 1, temperature=0.0, ignore_eos=True)
+        # (prompts that were prefilled first decode a few tokens while the others are
+        # prefilled; the margin keeps every request alive through the timed steps)
+        params = SamplingParams(max_tokens=steps + warmup + 17, temperature=0.0, ignore_eos=True)
         for _ in range(batch):
             engine.add_request([rng.randrange(vocab) for _ in range(args.prompt_len)], params)
         while engine.scheduler.waiting:
