@@ -85,6 +85,10 @@ class CpuOps:
             cache.v[pages, :, :, slots] = v.to(cache.v.dtype)        # values are kept transposed
         return q.reshape(T, qd).to(qkv.dtype)
 
+    def qkv_attention(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary, scale, window):
+        q = self.qkv_to_cache(qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary)
+        return self.paged_attention(q, step, cache, heads, kv_heads, head_dim, scale, window)
+
     def paged_attention(self, q, step, cache, heads, kv_heads, head_dim, scale, window):
         T = step.num_rows
         page = cache.group.page_size

@@ -398,6 +398,80 @@ def test_qkv_to_cache(ops, dtype, case):
     assert torch.equal(step.cache.k.cpu()[untouched], before_k.cpu()[untouched])
 
 
+RAW_DECODE_CASES = [
+    # heads, kv_heads, head_dim, norms, rotation, page, seq_lens, window, writes
+    (32, 8, 128, True, True, 16, [1500, 40, 129, 1, 640], None, True),     # keys split over workgroups
+    (8, 8, 64, True, True, 8, [130, 257, 16, 17], 19, True),
+    (5, 1, 256, False, True, 16, [90, 33], None, True),
+    (6, 2, 192, True, False, 4, [70, 5], 64, True),
+    (16, 1, 64, True, True, 16, [48, 1], None, False),                      # reads another layer's cache
+]
+
+
+@pytest.mark.parametrize("case", RAW_DECODE_CASES)
+def test_decode_attention_from_raw_projections(ops, case):
+    """The decode kernel that norms and rotates q and k itself and writes the row's
+    key and value: against float64 mathematics, and the cache it leaves against
+    the two-kernel path's."""
+    heads, kv_heads, hd, norms, rotation, page, seq_lens, window, writes = case
+    dtype = torch.bfloat16
+    B = len(seq_lens)
+    num_pages = sum((n + page - 1) // page for n in seq_lens) + 3
+    step, tables, pos, seq = make_step(seq_lens, [1] * B, page, num_pages, 7, kv_heads, hd, dtype, window)
+    ks, vs = fill_cache(step, tables, seq_lens, kv_heads, hd, dtype, 300)
+    step.cache.writes = writes
+    qd, kd = heads * hd, kv_heads * hd
+    qkv = rnd((B, qd + 2 * kd), dtype, 21)
+    qw, kw = 1 + rnd((hd,), torch.float32, 22, 0.2), 1 + rnd((hd,), torch.float32, 23, 0.2)
+    eps_q, eps_k = 1e-5, 3e-6
+    qn = (qw.to(DEV), eps_q) if norms else None
+    kn = (kw.to(DEV), eps_k) if norms else None
+    rotary = None
+    half = hd // 2
+    if rotation:
+        ang = torch.arange(2048, dtype=torch.float64)[:, None] * (10000.0 ** (-2.0 * torch.arange(half, dtype=torch.float64) / hd))[None, :]
+        cos, sin = torch.cos(ang).float(), torch.sin(ang).float()
+        rotary = (cos.to(DEV), sin.to(DEV), hd)
+    scale = 1.0 / math.sqrt(hd)
+    k0, v0 = step.cache.k.clone(), step.cache.v.clone()
+    out = ops.qkv_attention(qkv.to(DEV), step, step.cache, heads, kv_heads, hd, qn, kn, rotary, scale, window)
+    k1, v1 = step.cache.k.clone(), step.cache.v.clone()
+    # the same through qkv_to_cache and paged_attention
+    step.cache.k.copy_(k0)
+    step.cache.v.copy_(v0)
+    ops.unfused_decode = True
+    try:
+        out2 = ops.qkv_attention(qkv.to(DEV), step, step.cache, heads, kv_heads, hd, qn, kn, rotary, scale, window)
+    finally:
+        ops.unfused_decode = False
+    assert torch.equal(v1, step.cache.v)
+    close(k1, step.cache.k.double().cpu(), dtype, "keys in the cache", scale=float(k1.abs().max()) / 50)
+    if not writes:
+        assert torch.equal(k1, k0) and torch.equal(v1, v0)
+    # float64
+    x = qkv.double()
+    qq = x[:, :qd].reshape(B, heads, hd)
+    kk = x[:, qd:qd + kd].reshape(B, kv_heads, hd)
+    vv = x[:, qd + kd:].reshape(B, kv_heads, hd)
+    if norms:
+        qq = qw.double() * qq / torch.sqrt((qq * qq).mean(-1, keepdim=True) + eps_q)
+        kk = kw.double() * kk / torch.sqrt((kk * kk).mean(-1, keepdim=True) + eps_k)
+    if rotation:
+        c, sn = cos.double()[pos][:, None, :], sin.double()[pos][:, None, :]
+
+        def rot(t):
+            a, b = t[..., :half], t[..., half:]
+            return torch.cat([a * c - b * sn, a * sn + b * c], -1)
+        qq, kk = rot(qq), rot(kk)
+    if writes:                      # the row's own key and value replace what the cache held there
+        for i in range(B):
+            ks[i][-1] = kk[i].to(dtype)
+            vs[i][-1] = vv[i].to(dtype)
+    want = ref_attention(qq.reshape(B, qd).to(dtype), ks, vs, pos, seq, heads, kv_heads, scale, window)
+    close(out, want, dtype, "attention from raw projections")
+    close(out2, want, dtype, "attention through two kernels")
+
+
 def test_rotation_pairs_halves_not_neighbours(ops):
     """A head with only element i set: after the rotation at a position whose
     angle for pair i is 90 degrees, the value has moved to element i + d/2."""

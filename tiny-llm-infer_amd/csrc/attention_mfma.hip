@@ -317,15 +317,79 @@ __device__ __forceinline__ void decode_fetch(KeyBlock<NJ, ND>& b, const CacheVie
     }
 }
 
-// grid (splits, kv_heads * head_tiles, rows); 256 threads
-template <int NJ, int ND>
+// The step's raw projections [rows][(heads + 2 kv_heads) * head_dim] and what turns them
+// into queries and keys, for the decode kernel that does that work itself
+// (model/src/qwen3_paged_batch.cpp:180-236: per-head norm, rotation, cache write).
+struct RawQkv {
+    const bf16_t* qkv;
+    const float* q_norm_w;    // [head_dim] or null
+    const float* k_norm_w;
+    const float* cos;         // [positions][head_dim / 2] or null
+    const float* sin;
+    float q_eps, k_eps;
+    int write_cache;          // 0: the layer reads a cache that another layer writes
+};
+
+// One head of the raw projections as a B operand of the score MFMAs (this lane: dims
+// [c*8*NJ, +8*NJ) of the head at `src`), after the per-head RMS norm (if nw) and the
+// half-split rotation (if cos_row).  head_dim == 32*NJ, so the first half of the head
+// lies in lane groups 0 and 1 and the rotation partner of a lane is lane ^ 32.
+template <int NJ>
+__device__ __forceinline__ void head_from_raw(Frag (&out)[NJ], const bf16_t* src, const float* nw, float eps,
+                                              const float* cos_row, const float* sin_row) {
+    const int c = (threadIdx.x % 64) / 16;
+    const int d0 = c * 8 * NJ;
+    float x[NJ][8];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        Frag f;
+        f.u = *reinterpret_cast<const uint4*>(src + d0 + j * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[j][e] = bf16_to_f32(f.e[e]);
+    }
+    if (nw) {
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss += x[j][e] * x[j][e];
+        ss = quad_rows_sum(ss);
+        const float scale = 1.0f / sqrtf(ss / (float)(32 * NJ) + eps);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[j][e] = nw[d0 + j * 8 + e] * x[j][e] * scale;
+    }
+    if (cos_row) {
+        const int i0 = (c & 1) * 8 * NJ;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float partner = __shfl_xor(x[j][e], 32, 64);
+                const float cs = cos_row[i0 + j * 8 + e], sn = sin_row[i0 + j * 8 + e];
+                // first half: x cos - partner sin; second half: partner sin + x cos
+                x[j][e] = c < 2 ? x[j][e] * cs - partner * sn : partner * sn + x[j][e] * cs;
+            }
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+        out[j].u = make_uint4(pack_bf16x2(x[j][0], x[j][1]), pack_bf16x2(x[j][2], x[j][3]),
+                              pack_bf16x2(x[j][4], x[j][5]), pack_bf16x2(x[j][6], x[j][7]));
+}
+
+// grid (splits, kv_heads * head_tiles, rows); 256 threads.  FUSED: queries come from the
+// raw projections `raw` (q is not read), and the workgroup whose keys include the row's
+// own position writes that key and value into the cache first; needs head_dim == 32*NJ
+// and at most 16 heads a kv head (one workgroup per kv head and split).
+template <int NJ, int ND, bool FUSED>
 __global__ void __launch_bounds__(256)
 attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ partial,
-                        const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+                        bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
                         const int* __restrict__ positions, const int* __restrict__ seq_of_row,
                         const int* __restrict__ tables, int table_width, int page_size, int page_shift,
                         int num_pages, int heads, int kv_heads, int head_dim, float scale, int window,
-                        int splits, int keys_per_split) {
+                        int splits, int keys_per_split, RawQkv raw) {
     extern __shared__ float lds[];       // 3 waves x 64 lanes x (ND*4 + 2), then this split's table entries
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, c = lane / 16;
     const int split = blockIdx.x, row = blockIdx.z;
@@ -345,7 +409,19 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     tile_init(t);
     t.pos = live ? pos : -1;
     t.lo = live ? lo : 0;
-    tile_load_q(t, q + ((size_t)row * heads + (live ? head : 0)) * head_dim, head_dim, live);
+    const bf16_t* raw_row = nullptr;
+    const float *cos_row = nullptr, *sin_row = nullptr;
+    if (FUSED) {
+        raw_row = raw.qkv + (size_t)row * (heads + 2 * kv_heads) * head_dim;
+        if (raw.cos) {
+            cos_row = raw.cos + (size_t)pos * (head_dim / 2);
+            sin_row = raw.sin + (size_t)pos * (head_dim / 2);
+        }
+        // (an idle column computes on head 0; it is masked by its pos of -1)
+        head_from_raw<NJ>(t.q, raw_row + (size_t)(live ? head : 0) * head_dim, raw.q_norm_w, raw.q_eps, cos_row, sin_row);
+    } else {
+        tile_load_q(t, q + ((size_t)row * heads + (live ? head : 0)) * head_dim, head_dim, live);
+    }
 
     // this split's keys, in 32-key blocks that the waves take in turn
     const int first_block = lo / 32;
@@ -359,6 +435,30 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     for (int i = threadIdx.x; i < seg_len; i += 256)
         seg[i] = seg_first + i < table_width ? table[seg_first + i] : -1;
     __syncthreads();
+    if (FUSED && raw.write_cache) {
+        // the row's own key and value: written by the workgroup that reads them below
+        if (begin <= pos && pos < end) {
+            const int page = seg[(pos >> page_shift) - seg_first];
+            const int slot = pos & (page_size - 1);
+            if ((unsigned)page < (unsigned)num_pages) {
+                if (wave == 0) {
+                    Frag kf[NJ];
+                    head_from_raw<NJ>(kf, raw_row + (size_t)(heads + kv_head) * head_dim, raw.k_norm_w, raw.k_eps,
+                                      cos_row, sin_row);
+                    bf16_t* dst = k_cache + (((size_t)page * kv_heads + kv_head) * page_size + slot) * head_dim + c * 8 * NJ;
+                    if (r == 0) {
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j) *reinterpret_cast<uint4*>(dst + j * 8) = kf[j].u;
+                    }
+                } else if (wave == 1) {
+                    const bf16_t* src = raw_row + (size_t)(heads + kv_heads + kv_head) * head_dim;
+                    bf16_t* dst = v_cache + ((size_t)page * kv_heads + kv_head) * head_dim * page_size + slot;
+                    for (int d = lane; d < head_dim; d += 64) dst[(size_t)d * page_size] = src[d];
+                }
+            }
+        }
+        __syncthreads();
+    }
 
     // a wave's blocks are 128 keys apart; the next block is asked for before this one is
     // multiplied (the last block is asked for once more instead of branching round the loads)
@@ -807,11 +907,11 @@ static int check_common(const char* what, int heads, int kv_heads, int head_dim,
 
 // Every row is its sequence's only row in this step.  `partial` holds
 // rows*heads*splits*(head_dim+2) floats when splits > 1.
-extern "C" int tli_attention_decode_bf16(
-    const void* q, void* out, float* partial, const void* k_cache, const void* v_cache,
-    const int* positions, const int* seq_of_row, const int* tables, int table_width, int page_size,
-    int num_pages, int rows, int heads, int kv_heads, int head_dim, float scale, int window,
-    int splits, int keys_per_split, void* stream) {
+static int launch_decode(const void* q, void* out, float* partial, void* k_cache, void* v_cache,
+                         const int* positions, const int* seq_of_row, const int* tables, int table_width,
+                         int page_size, int num_pages, int rows, int heads, int kv_heads, int head_dim,
+                         float scale, int window, int splits, int keys_per_split, const RawQkv* raw,
+                         void* stream) {
     if (rows <= 0) return 0;
     if (check_common("attention_decode", heads, kv_heads, head_dim, page_size, table_width, num_pages)) return 1;
     if (splits < 1 || splits > 65535 || keys_per_split <= 0 || keys_per_split % 128)
@@ -821,6 +921,9 @@ extern "C" int tli_attention_decode_bf16(
     if (rows > 65535) return tli_fail("attention_decode: %d rows exceed the grid limit", rows);
     hipStream_t s = (hipStream_t)stream;
     const int group = heads / kv_heads, head_tiles = (group + 15) / 16;
+    if (raw && (head_dim % 64 || group > 16))
+        return tli_fail("attention_decode from raw projections: head_dim %d must be a multiple of 64 and "
+                        "heads per kv head (%d) at most 16", head_dim, group);
     dim3 grid(splits, kv_heads * head_tiles, rows);
     const int shift = log2_exact(page_size);
     // the table entries of one split are kept in LDS
@@ -828,19 +931,54 @@ extern "C" int tli_attention_decode_bf16(
     if (seg_bytes > 8192)
         return tli_fail("attention_decode: %d keys per split in pages of %d are more than 2046 pages; use more splits",
                         keys_per_split, page_size);
-#define CALL(NJ, ND)                                                                                    \
-    attention_decode_kernel<NJ, ND><<<grid, 256, 3 * 64 * (ND * 4 + 2) * sizeof(float) + seg_bytes, s>>>( \
-        (const bf16_t*)q, (bf16_t*)out, partial, (const bf16_t*)k_cache, (const bf16_t*)v_cache,        \
-        positions, seq_of_row, tables, table_width, page_size, shift, num_pages, heads, kv_heads,       \
-        head_dim, scale * LOG2E, window, splits, keys_per_split)
+    const RawQkv none{};
+#define ARGS (const bf16_t*)q, (bf16_t*)out, partial, (bf16_t*)k_cache, (bf16_t*)v_cache, positions, seq_of_row, \
+             tables, table_width, page_size, shift, num_pages, heads, kv_heads, head_dim, scale * LOG2E, window, \
+             splits, keys_per_split
+#define LDS_BYTES(ND) (3 * 64 * (ND * 4 + 2) * sizeof(float) + seg_bytes)
+#define CALL(NJ, ND)                                                                                        \
+    if (raw) attention_decode_kernel<NJ, ND, NJ * 2 == ND><<<grid, 256, LDS_BYTES(ND), s>>>(ARGS, *raw);   \
+    else attention_decode_kernel<NJ, ND, false><<<grid, 256, LDS_BYTES(ND), s>>>(ARGS, none)
     DISPATCH_HEAD_DIM(CALL)
 #undef CALL
+#undef LDS_BYTES
+#undef ARGS
     if (tli_check_launch("attention_decode")) return 1;
     if (splits > 1) {
         attention_merge_splits_kernel<<<dim3(heads, rows), 64, 0, s>>>(partial, (bf16_t*)out, heads, head_dim, splits);
         return tli_check_launch("attention_merge_splits");
     }
     return 0;
+}
+
+extern "C" int tli_attention_decode_bf16(
+    const void* q, void* out, float* partial, const void* k_cache, const void* v_cache,
+    const int* positions, const int* seq_of_row, const int* tables, int table_width, int page_size,
+    int num_pages, int rows, int heads, int kv_heads, int head_dim, float scale, int window,
+    int splits, int keys_per_split, void* stream) {
+    return launch_decode(q, out, partial, (void*)k_cache, (void*)v_cache, positions, seq_of_row, tables,
+                         table_width, page_size, num_pages, rows, heads, kv_heads, head_dim, scale, window,
+                         splits, keys_per_split, nullptr, stream);
+}
+
+// Decode attention straight from the raw projections qkv [rows][(heads + 2 kv_heads) * head_dim]:
+// per-head norm (weights may be null), rotation (cos/sin [table_positions][head_dim/2] or null:
+// the whole head is rotated), the row's key and value into the cache (write_cache), then
+// attention as tli_attention_decode_bf16.  One row per sequence.  head_dim a multiple of 64,
+// at most 16 heads a kv head.
+extern "C" int tli_qkv_attention_decode_bf16(
+    const void* qkv, void* out, float* partial, void* k_cache, void* v_cache,
+    const int* positions, const int* seq_of_row, const int* tables, int table_width, int page_size,
+    int num_pages, int rows, int heads, int kv_heads, int head_dim,
+    const float* q_norm_w, float q_eps, const float* k_norm_w, float k_eps,
+    const float* cos_table, const float* sin_table, int write_cache,
+    float scale, int window, int splits, int keys_per_split, void* stream) {
+    if (!qkv) return tli_fail("attention_decode from raw projections: no projections");
+    if ((cos_table == nullptr) != (sin_table == nullptr)) return tli_fail("attention_decode: cos without sin");
+    const RawQkv raw{(const bf16_t*)qkv, q_norm_w, k_norm_w, cos_table, sin_table, q_eps, k_eps, write_cache};
+    return launch_decode(nullptr, out, partial, k_cache, v_cache, positions, seq_of_row, tables, table_width,
+                         page_size, num_pages, rows, heads, kv_heads, head_dim, scale, window, splits,
+                         keys_per_split, &raw, stream);
 }
 
 // Rows of a sequence are contiguous and ascend in position; row_start has num_seqs+1 entries.

@@ -58,6 +58,8 @@ def load_library():
         "tli_gemm_mid_bf16": [P, P, P, P, I, I, I, I, I, I, I, P],
         "tli_gemm_mid_splits": [I, I, I],
         "tli_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
+        "tli_qkv_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I,
+                                          F, I, I, I, P],
         "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
         "tli_sample_scratch_bytes": [I],
@@ -91,6 +93,7 @@ class HipOps:
             raise KernelError("no GPU is visible to torch; this engine has no CPU path")
         self.lib = load_library()
         self.force_plain = False     # tests: run the plain attention kernel for bfloat16 too
+        self.unfused_decode = False  # tests: decode steps through qkv_to_cache and paged_attention too
         self.prefill_direct = 0      # tests: 1 = the prefill attention kernel without LDS staging; 2, 3 = with, 1 or 2 tiles a wave
         self.mid_cfg = 0             # measurements: launch shape and k ranges of the 17..64-row kernel
         self.mid_splits = 0
@@ -334,8 +337,47 @@ class HipOps:
                    head_dim, float(scale), int(window or 0), _dtype_code(q.dtype), self._stream())
         return out
 
-    def _attention_decode(self, q, out, step, kc, vc, g, heads, kv_heads, head_dim, scale, window):
-        """One row per sequence.  The keys are split over workgroups when the
+    def qkv_attention(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary, scale, window):
+        """From the raw projections to the attention output: norms and rotation of q
+        and k, k and v into the cache, attention over the cache.  A decode step (one
+        row a sequence) does all of it in the attention kernel where the sizes allow;
+        other steps run qkv_to_cache and paged_attention."""
+        fused = (qkv.dtype == torch.bfloat16 and step.max_rows_per_seq == 1 and cache is not None
+                 and head_dim % 64 == 0 and head_dim <= 256 and heads // kv_heads <= 16
+                 and cache.group.page_size >= 4 and not self.force_plain and not self.unfused_decode
+                 and (rotary is None or rotary[2] == head_dim))
+        if not fused:
+            q = self.qkv_to_cache(qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary)
+            return self.paged_attention(q, step, cache, heads, kv_heads, head_dim, scale, window)
+        T = step.num_rows
+        self._want(qkv, "qkv", None, (T, (heads + 2 * kv_heads) * head_dim))
+        kc, vc, g = cache.k, cache.v, cache.group
+        self._check_cache(kc, vc, g, kv_heads, head_dim, qkv.dtype, step)
+        qw, qe = q_norm if q_norm is not None else (None, 0.0)
+        kw, ke = k_norm if k_norm is not None else (None, 0.0)
+        for w in (qw, kw):
+            if w is not None:
+                self._want(w, "head norm weight", torch.float32, (head_dim,))
+        cos = sin = None
+        if rotary is not None:
+            cos, sin, rd = rotary
+            npos = cos.shape[0]
+            self._want(cos, "cos table", torch.float32, (npos, rd // 2))
+            self._want(sin, "sin table", torch.float32, (npos, rd // 2))
+            if step.max_seq_len > npos:
+                raise KernelError(f"a position reaches {step.max_seq_len}, the rotation table has {npos}")
+        out = torch.empty((T, heads * head_dim), dtype=qkv.dtype, device=self.device)
+        splits, per_split, partial = self._decode_splits(step, g, heads, kv_heads, head_dim, window)
+        self._call(self.lib.tli_qkv_attention_decode_bf16, qkv.data_ptr(), out.data_ptr(), _ptr(partial),
+                   kc.data_ptr(), vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
+                   g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], T, heads, kv_heads,
+                   head_dim, _ptr(qw), float(qe), _ptr(kw), float(ke), _ptr(cos), _ptr(sin),
+                   1 if cache.writes else 0, float(scale), int(window or 0), splits, per_split,
+                   self._stream())
+        return out
+
+    def _decode_splits(self, step, g, heads, kv_heads, head_dim, window):
+        """How the keys of a decode step are split over workgroups: they are when the
         batch alone would leave most of the 256 compute units idle."""
         T = step.num_rows
         reach = step.reach if not window else min(step.reach, (window + 31) // 32 * 32 + 32)
@@ -350,6 +392,12 @@ class HipOps:
         if splits > 1:
             partial = torch.empty((T * heads * splits * (head_dim + 2),), dtype=torch.float32,
                                   device=self.device)
+        return splits, per_split, partial
+
+    def _attention_decode(self, q, out, step, kc, vc, g, heads, kv_heads, head_dim, scale, window):
+        """One row per sequence."""
+        T = step.num_rows
+        splits, per_split, partial = self._decode_splits(step, g, heads, kv_heads, head_dim, window)
         self._call(self.lib.tli_attention_decode_bf16, q.data_ptr(), out.data_ptr(), _ptr(partial),
                    kc.data_ptr(), vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
                    g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], T, heads, kv_heads,

@@ -72,13 +72,11 @@ class PagedAttention(Mixer):
         ops = self.env.ops
         qkv = ops.linear(x, self.w_qkv)
         rot = self.position.rotary() if self.position is not None else None
-        q = ops.qkv_to_cache(
+        o = ops.qkv_attention(
             qkv, step, step.cache, self.heads, self.kv_heads, self.head_dim,
             None if self.q_norm is None else (self.q_norm.weight, self.q_norm.eps),
             None if self.k_norm is None else (self.k_norm.weight, self.k_norm.eps),
-            rot)
-        o = ops.paged_attention(q, step, step.cache, self.heads, self.kv_heads, self.head_dim,
-                                self.scale, self.window)
+            rot, self.scale, self.window)
         return ops.linear(o, self.w_o)
 
 
