@@ -489,6 +489,39 @@ def test_rotation_pairs_halves_not_neighbours(ops):
     assert torch.allclose(q[0].cpu(), want, atol=1e-7)
 
 
+def test_partial_sums_as_residual_delta(ops):
+    """A product of 17..64 rows whose k range is split may leave its partial sums to
+    the norm that follows: the residual and the normed rows are bit for bit what the
+    product's own reduction followed by the norm gives, also for a subset of rows."""
+    from tiny_llm_infer_amd.kernels.ops import DeferredSum
+    M, N, K = 37, 200, 1024
+    x, w = rnd((M, K), torch.bfloat16, 1).to(DEV), rnd((N, K), torch.bfloat16, 2, 0.05).to(DEV)
+
+    class Both:
+        pass
+    Both.w, Both.tiled = w, ops.tile_matrix(w)
+    weight = (1 + rnd((N,), torch.float32, 3, 0.1)).to(DEV)
+    resid = rnd((M, N), torch.float32, 4).to(DEV)
+    ops.mid_splits = 4
+    try:
+        y = ops.linear(x, Both)
+        d = ops.linear(x, Both, deferred=True)
+    finally:
+        ops.mid_splits = 0
+    assert isinstance(d, DeferredSum) and tuple(d.parts.shape) == (4, M, N)
+    assert torch.equal(ops.resolve(d), y)
+    r1, r2 = resid.clone(), resid.clone()
+    o1 = ops.add_rmsnorm(r1, y, weight, 1e-5, torch.bfloat16)
+    o2 = ops.add_rmsnorm(r2, d, weight, 1e-5, torch.bfloat16)
+    assert torch.equal(r1, r2) and torch.equal(o1, o2)
+    rows = torch.tensor([36, 0, 5], dtype=torch.int32, device=DEV)
+    r3 = resid.clone()
+    o3 = ops.add_rmsnorm(r3, d, weight, 1e-5, torch.bfloat16, rows=rows)
+    assert torch.equal(r3, resid)                                  # a subset of rows leaves the residual alone
+    assert torch.equal(o3, ops.add_rmsnorm(resid.clone(), y, weight, 1e-5, torch.bfloat16, rows=rows))
+    assert torch.equal(o3, o1[rows.long()])
+
+
 # ------------------------------------------------------------------ sampling --
 def test_greedy_takes_the_lowest_index_on_ties(ops):
     logits = torch.zeros(3, 5000)

@@ -65,7 +65,7 @@ def test_swiglu_part(envs, dtype):
     x = rnd((9, 80), dtype, 3)
     f = {k: v.cpu().double() for k, v in w.items()}
     want = P.linear(P.swiglu(P.linear(x.double(), f["g"]), P.linear(x.double(), f["u"])), f["d"])
-    close(part.forward(x.to(DEV), None), want, dtype, "swiglu part")
+    close(envs[dtype].ops.resolve(part.forward(x.to(DEV), None)), want, dtype, "swiglu part")
 
 
 def _attention_spec(heads, kv, hd, hidden, window, theta=1e4, eps=1e-6):
@@ -92,7 +92,7 @@ def test_attention_part_whole_sequence(envs, dtype, window):
     assert part.cache_need().window == window
     step, tables, pos, seq = make_step([T], [T], 16, 5, 0, kv, hd, dtype, window)
     x = rnd((T, hidden), dtype, 5)
-    out = part.forward(x.to(DEV), step)
+    out = envs[dtype].ops.resolve(part.forward(x.to(DEV), step))     # (it may come as unadded partial sums)
     f = {("self." + k + ("_proj.weight" if k in "qkvo" else "")): v.cpu().double() for k, v in w.items()}
     f["self.q_norm.weight"], f["self.k_norm.weight"] = f.pop("self.qn"), f.pop("self.kn")
     cfg = dict(num_attention_heads=heads, num_key_value_heads=kv, head_dim=hd, hidden_size=hidden,
@@ -128,7 +128,7 @@ def test_prenorm_block(envs, dtype):
     m = P.rmsnorm(r, f["n2"], 1e-6)
     d = P.linear(P.swiglu(P.linear(m, f["g"]), P.linear(m, f["u"])), f["d"])
     close(resid, r, dtype, "residual after the mixer")     # the second sum is still owed
-    close(pending, d, dtype, "what the block owes the residual")
+    close(envs[dtype].ops.resolve(pending), d, dtype, "what the block owes the residual")
 
 
 # ------------------------------------------------------------------ toy mixer --

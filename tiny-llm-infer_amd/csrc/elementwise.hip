@@ -3,7 +3,10 @@
 // embed:       resid[t, :] = float(table[id[t], :])                       (layers/src/embedding.cpp:37-44)
 // add_rmsnorm: v = resid[r] (+ delta[r]);  out = w * v * 1/sqrt(mean(v^2) + eps), in float32
 //              (kernels/src/rmsnorm_kernel_cpu.cpp:27-43; the sum h + a of
-//              model/src/qwen3_paged_batch.cpp:273-275 is done here, unrounded)
+//              model/src/qwen3_paged_batch.cpp:273-275 is done here, unrounded).
+//              delta may also come as float32 partial sums [parts][rows][n] of a matrix
+//              product whose k range was split: they are added in order and rounded to
+//              bfloat16 first, which is what the product's own reduction would have stored
 // swiglu:      out = g / (1 + exp(-g)) * u over a fused [rows, 2*inter] input
 //              (kernels/src/swiglu_kernel_cpu.cpp:20-24)
 #include "common.h"
@@ -19,8 +22,35 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32(src[i]);
 }
 
+// What a row owes the residual: a row of T, or float32 partial sums [parts][total_rows][n]
+// added in order and rounded to bfloat16.
 template <typename T>
-__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+struct RowDelta {
+    const T* d;
+    const float* p;
+    int parts;
+    size_t plane;
+    __device__ __forceinline__ bool any() const { return d != nullptr || parts > 0; }
+    __device__ __forceinline__ float at(int i) const {
+        if (parts > 0) {
+            float a = 0.f;
+            for (int s = 0; s < parts; ++s) a += p[s * plane + i];
+            return bf16_to_f32(f32_to_bf16(a));
+        }
+        return to_f32(d[i]);
+    }
+};
+
+template <typename T>
+__device__ __forceinline__ RowDelta<T> row_delta(const void* delta, int parts, int r, int n, int total_rows) {
+    RowDelta<T> rd{nullptr, nullptr, parts, (size_t)total_rows * n};
+    if (parts > 0) rd.p = (const float*)delta + (size_t)r * n;
+    else if (delta) rd.d = (const T*)delta + (size_t)r * n;
+    return rd;
+}
+
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const void* __restrict__ delta, int parts,
                                    const float* __restrict__ weight, T* __restrict__ out,
                                    const int* __restrict__ rows, int n, float eps, int total_rows) {
     __shared__ float scratch[16];
@@ -28,12 +58,12 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
     int r = rows ? rows[out_row] : out_row;
     if (r < 0 || r >= total_rows) r = 0;
     float* x = resid + (size_t)r * n;
-    const T* d = delta ? delta + (size_t)r * n : nullptr;
-    const bool update = (rows == nullptr) && (d != nullptr);
+    const RowDelta<T> d = row_delta<T>(delta, parts, r, n, total_rows);
+    const bool update = (rows == nullptr) && d.any();
     float ss = 0.f;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         float v = x[i];
-        if (d) v += to_f32(d[i]);
+        if (d.any()) v += d.at(i);
         if (update) x[i] = v;
         ss += v * v;
     }
@@ -42,7 +72,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
     T* o = out + (size_t)out_row * n;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         float v = x[i];
-        if (d && !update) v += to_f32(d[i]);
+        if (d.any() && !update) v += d.at(i);
         from_f32(o + i, weight[i] * v * scale);
     }
 }
@@ -69,7 +99,7 @@ __device__ __forceinline__ void store4(bf16_t* p, const float v[4]) {
 }
 
 template <typename T, int IT>
-__global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const void* __restrict__ delta, int parts,
                                        const float* __restrict__ weight, T* __restrict__ out,
                                        const int* __restrict__ rows, int n, float eps, int total_rows) {
     __shared__ float scratch[16];
@@ -77,8 +107,8 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __res
     int r = rows ? rows[out_row] : out_row;
     if (r < 0 || r >= total_rows) r = 0;
     float* x = resid + (size_t)r * n;
-    const T* d = delta ? delta + (size_t)r * n : nullptr;
-    const bool update = (rows == nullptr) && (d != nullptr);
+    const RowDelta<T> d = row_delta<T>(delta, parts, r, n, total_rows);
+    const bool update = (rows == nullptr) && d.any();
     float v[IT][4];
     float ss = 0.f;
 #pragma unroll
@@ -86,9 +116,20 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __res
         const int i = (threadIdx.x + it * blockDim.x) * 4;
         if (i < n) {
             load4(x + i, v[it]);
-            if (d) {
+            if (d.any()) {
                 float dv[4];
-                load4(d + i, dv);
+                if (d.parts > 0) {
+                    float a[4] = {0.f, 0.f, 0.f, 0.f};
+                    for (int s = 0; s < d.parts; ++s) {
+                        load4(d.p + s * d.plane + i, dv);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) a[e] += dv[e];
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) dv[e] = bf16_to_f32(f32_to_bf16(a[e]));
+                } else {
+                    load4(d.d + i, dv);
+                }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[it][e] += dv[e];
                 if (update) store4(x + i, v[it]);
@@ -114,20 +155,20 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const T* __res
 }
 
 template <typename T>
-static void launch_add_rmsnorm(float* resid, const T* delta, const float* weight, T* out, const int* rows,
-                               int out_rows, int total_rows, int n, float eps, hipStream_t s) {
+static void launch_add_rmsnorm(float* resid, const void* delta, int parts, const float* weight, T* out,
+                               const int* rows, int out_rows, int total_rows, int n, float eps, hipStream_t s) {
     const int groups = n / 4;
     if (n % 4 == 0 && groups <= 4096) {
         int threads = groups <= 1024 ? (groups + 63) / 64 * 64 : 1024;
         if (groups <= 1024)
-            add_rmsnorm_vec_kernel<T, 1><<<out_rows, threads, 0, s>>>(resid, delta, weight, out, rows, n, eps, total_rows);
+            add_rmsnorm_vec_kernel<T, 1><<<out_rows, threads, 0, s>>>(resid, delta, parts, weight, out, rows, n, eps, total_rows);
         else if (groups <= 2048)
-            add_rmsnorm_vec_kernel<T, 2><<<out_rows, threads, 0, s>>>(resid, delta, weight, out, rows, n, eps, total_rows);
+            add_rmsnorm_vec_kernel<T, 2><<<out_rows, threads, 0, s>>>(resid, delta, parts, weight, out, rows, n, eps, total_rows);
         else
-            add_rmsnorm_vec_kernel<T, 4><<<out_rows, threads, 0, s>>>(resid, delta, weight, out, rows, n, eps, total_rows);
+            add_rmsnorm_vec_kernel<T, 4><<<out_rows, threads, 0, s>>>(resid, delta, parts, weight, out, rows, n, eps, total_rows);
         return;
     }
-    add_rmsnorm_kernel<T><<<out_rows, n >= 2048 ? 512 : 256, 0, s>>>(resid, delta, weight, out, rows, n, eps, total_rows);
+    add_rmsnorm_kernel<T><<<out_rows, n >= 2048 ? 512 : 256, 0, s>>>(resid, delta, parts, weight, out, rows, n, eps, total_rows);
 }
 
 template <typename T>
@@ -172,18 +213,20 @@ extern "C" int tli_embed(const void* table, const int* ids, float* out, int rows
     return tli_check_launch("embed");
 }
 
+// parts > 0: `delta` holds float32 partial sums [parts][total_rows][n] (bfloat16 rows only).
 extern "C" int tli_add_rmsnorm(float* resid, const void* delta, const float* weight, void* out,
                                const int* rows, int out_rows, int total_rows, int n, float eps,
-                               int dtype, void* stream) {
+                               int dtype, int parts, void* stream) {
     if (out_rows <= 0) return 0;
     if (n <= 0) return tli_fail("add_rmsnorm: bad row size %d", n);
+    if (parts < 0 || (parts > 0 && (dtype != TLI_BF16 || !delta)))
+        return tli_fail("add_rmsnorm: partial sums (%d) go with bfloat16 rows only", parts);
     hipStream_t s = (hipStream_t)stream;
     if (dtype == TLI_F32)
-        launch_add_rmsnorm<float>(resid, (const float*)delta, weight, (float*)out, rows, out_rows,
-                                  total_rows, n, eps, s);
+        launch_add_rmsnorm<float>(resid, delta, 0, weight, (float*)out, rows, out_rows, total_rows, n, eps, s);
     else if (dtype == TLI_BF16)
-        launch_add_rmsnorm<bf16_t>(resid, (const bf16_t*)delta, weight, (bf16_t*)out, rows, out_rows,
-                                   total_rows, n, eps, s);
+        launch_add_rmsnorm<bf16_t>(resid, delta, parts, weight, (bf16_t*)out, rows, out_rows, total_rows, n,
+                                   eps, s);
     else
         return tli_fail("add_rmsnorm: unknown dtype %d", dtype);
     return tli_check_launch("add_rmsnorm");

@@ -250,7 +250,7 @@ static int launch_mid(const bf16_t* x, const bf16_t* w, void* y, float* part, in
     else
         gemm_mid_kernel<RT, WAVES, DEPTH, float, false><<<grid, WAVES * 64, 0, s>>>(x, w, (float*)y, part, M, N, K, splits, steps_per_split);
     if (tli_check_launch("gemm_mid")) return 1;
-    if (splits > 1) {
+    if (splits > 1 && y) {
         const size_t total = (size_t)M * (gated ? N / 2 : N);
         const unsigned blocks = (unsigned)((total + 255) / 256);
         if (y_dtype == TLI_BF16)
@@ -279,7 +279,9 @@ extern "C" int tli_gemm_mid_splits(int N, int K, int gated) {
 
 // y[M,N] = x[M,K] . W^T for 1 <= M <= 64, W in the decode layout (`gated` as tiled = 2 of
 // tli_gemm_skinny_bf16: y is [M, N/2] bfloat16).  `part`: splits*M*N floats when
-// splits > 1 (splits as returned by tli_gemm_mid_splits, or forced by the caller);
+// splits > 1 (splits as returned by tli_gemm_mid_splits, or forced by the caller); with
+// y null the partial sums [splits][M][N] are left for the consumer to add (tli_gemm_mid_reduce,
+// or tli_add_rmsnorm);
 // cfg 0 picks the launch shape, else DEPTH*100 + RT*10 + WAVES.
 extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* part, int M, int N, int K,
                                  int y_dtype, int gated, int splits, int cfg, void* stream) {
@@ -291,6 +293,7 @@ extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* p
         return tli_fail("gemm_mid: a gated product needs N %% 32 == 0 and bfloat16 output");
     if (splits < 1 || splits > 64) return tli_fail("gemm_mid: %d splits", splits);
     if (splits > 1 && !part) return tli_fail("gemm_mid: splits need a buffer for partial sums");
+    if (!y && (splits < 2 || gated)) return tli_fail("gemm_mid: only a plain product with split k can leave its partial sums");
     if (((uintptr_t)x | (uintptr_t)w) & 15) return tli_fail("gemm_mid: operands must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xp = (const bf16_t*)x;
@@ -303,4 +306,20 @@ extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* p
         MID_CASE(2, 2, 4) MID_CASE(4, 2, 4) MID_CASE(2, 2, 8)
         default: return tli_fail("gemm_mid: unknown configuration %d", cfg);
     }
+}
+
+// y[M,N] = sum over the partial products in `part` [splits][M][N], in split order.
+extern "C" int tli_gemm_mid_reduce(const float* part, void* y, int M, int N, int splits, int y_dtype, void* stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (!part || !y || splits < 1) return tli_fail("gemm_mid_reduce: bad arguments");
+    hipStream_t s = (hipStream_t)stream;
+    const size_t total = (size_t)M * N;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    if (y_dtype == TLI_BF16)
+        gemm_mid_reduce_kernel<bf16_t><<<blocks, 256, 0, s>>>(part, (bf16_t*)y, M, N, splits, 0);
+    else if (y_dtype == TLI_F32)
+        gemm_mid_reduce_kernel<float><<<blocks, 256, 0, s>>>(part, (float*)y, M, N, splits, 0);
+    else
+        return tli_fail("gemm_mid_reduce: bad output dtype %d", y_dtype);
+    return tli_check_launch("gemm_mid_reduce");
 }

@@ -49,7 +49,7 @@ def load_library():
         "tli_abi_version": [],
         "tli_embed": [P, P, P, I, I, I, I, P],
         "tli_feed_tokens": [P, P, P, I, I, P],
-        "tli_add_rmsnorm": [P, P, P, P, P, I, I, I, F, I, P],
+        "tli_add_rmsnorm": [P, P, P, P, P, I, I, I, F, I, I, P],
         "tli_swiglu": [P, P, I, I, I, P],
         "tli_qkv_to_cache": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I, I, I, I, P],
         "tli_attention_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
@@ -57,6 +57,7 @@ def load_library():
         "tli_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, I, P],
         "tli_gemm_mid_bf16": [P, P, P, P, I, I, I, I, I, I, I, P],
         "tli_gemm_mid_splits": [I, I, I],
+        "tli_gemm_mid_reduce": [P, P, I, I, I, I, P],
         "tli_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
         "tli_qkv_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I,
                                           F, I, I, I, P],
@@ -76,6 +77,19 @@ def load_library():
 
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
+
+
+class DeferredSum:
+    """A matrix product whose k range was split, left as float32 partial sums
+    [splits, rows, cols].  ``HipOps.linear(..., deferred=True)`` may return one
+    instead of a tensor; ``add_rmsnorm`` takes it as the delta and adds the parts
+    itself (rounding the sum to ``dtype`` as the product's own reduction would),
+    anything else calls ``HipOps.resolve`` first."""
+
+    def __init__(self, parts: torch.Tensor, dtype: torch.dtype):
+        self.parts = parts
+        self.dtype = dtype
+        self.shape = tuple(parts.shape[1:])
 
 
 class HipOps:
@@ -150,11 +164,29 @@ class HipOps:
                    num_rows, hidden, vocab, _dtype_code(table.dtype), self._stream())
         return out
 
+    def resolve(self, y):
+        """The tensor of a product that ``linear`` may have left as partial sums."""
+        if not isinstance(y, DeferredSum):
+            return y
+        splits, M, N = y.parts.shape
+        out = torch.empty((M, N), dtype=y.dtype, device=self.device)
+        self._call(self.lib.tli_gemm_mid_reduce, y.parts.data_ptr(), out.data_ptr(), M, N, splits,
+                   _dtype_code(y.dtype), self._stream())
+        return out
+
     def add_rmsnorm(self, resid, delta, weight, eps, out_dtype, rows=None, num_rows=None):
         total, n = resid.shape
         self._want(resid, "residual", torch.float32)
         self._want(weight, "norm weight", torch.float32, (n,))
-        if delta is not None:
+        parts = 0
+        if isinstance(delta, DeferredSum):
+            if delta.dtype != out_dtype or out_dtype != torch.bfloat16:
+                delta = self.resolve(delta)
+            else:
+                parts = delta.parts.shape[0]
+                delta = delta.parts
+                self._want(delta, "partial sums of the residual delta", torch.float32, (parts, total, n))
+        if delta is not None and not parts:
             self._want(delta, "residual delta", out_dtype, (total, n))
         out_rows = total
         if rows is not None:
@@ -165,7 +197,7 @@ class HipOps:
         out = torch.empty((out_rows, n), dtype=out_dtype, device=self.device)
         self._call(self.lib.tli_add_rmsnorm, resid.data_ptr(), _ptr(delta), weight.data_ptr(),
                    out.data_ptr(), _ptr(rows), out_rows, total, n, float(eps),
-                   _dtype_code(out_dtype), self._stream())
+                   _dtype_code(out_dtype), parts, self._stream())
         return out
 
     def tile_matrix(self, w: torch.Tensor) -> Optional[torch.Tensor]:
@@ -185,9 +217,10 @@ class HipOps:
         t = w.view(n16 // 16, 16, k128 // 128, 4, 4, 8)          # [nb, r, kb, c, j, e]
         return t.permute(0, 2, 4, 3, 1, 5).contiguous()           # [nb, kb, j, c, r, e]
 
-    def linear(self, x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None):
+    def linear(self, x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None, deferred: bool = False):
         """y = x W^T.  ``w`` is a [N, K] tensor or a ``Matrix`` (row-major tensor plus
-        its decode layout)."""
+        its decode layout).  ``deferred``: the caller hands the result to ``add_rmsnorm``
+        (or to ``resolve``) and so also takes a ``DeferredSum``."""
         tiled = getattr(w, "tiled", None)
         w = getattr(w, "w", w)
         M, K = x.shape
@@ -207,7 +240,7 @@ class HipOps:
                 # few rows (decode), or float32 logits: the weight-streaming MFMA kernel,
                 # 64 rows at a time
                 if tiled is not None and self.MID_ROWS_FROM <= M <= self.SKINNY_ROWS:
-                    return self._linear_mid(x, tiled, y, M, N, K, 0)
+                    return self._linear_mid(x, tiled, y, M, N, K, 0, deferred)
                 wp = w if tiled is None else tiled
                 for m0 in range(0, M, self.SKINNY_ROWS):
                     m1 = min(M, m0 + self.SKINNY_ROWS)
@@ -223,16 +256,18 @@ class HipOps:
                    _dtype_code(x.dtype), _dtype_code(w.dtype), _dtype_code(out_dtype), self._stream())
         return y
 
-    def _linear_mid(self, x, tiled, y, M, N, K, gated):
+    def _linear_mid(self, x, tiled, y, M, N, K, gated, deferred=False):
         """17..64 rows: the kernel that shares x through LDS, k cut into ranges when the
-        output alone gives too few workgroups."""
+        output alone gives too few workgroups.  ``deferred``: the partial sums of the
+        ranges are left for the consumer to add, which saves the pass that adds them."""
         splits = self.mid_splits or self.lib.tli_gemm_mid_splits(N, K, gated)
         part = None
         if splits > 1:
-            part = torch.empty((splits * M * N,), dtype=torch.float32, device=self.device)
-        self._call(self.lib.tli_gemm_mid_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), _ptr(part),
-                   M, N, K, _dtype_code(y.dtype), gated, splits, self.mid_cfg, self._stream())
-        return y
+            part = torch.empty((splits, M, N), dtype=torch.float32, device=self.device)
+        leave = deferred and splits > 1 and not gated and y.dtype == torch.bfloat16
+        self._call(self.lib.tli_gemm_mid_bf16, x.data_ptr(), tiled.data_ptr(), None if leave else y.data_ptr(),
+                   _ptr(part), M, N, K, _dtype_code(y.dtype), gated, splits, self.mid_cfg, self._stream())
+        return DeferredSum(part, y.dtype) if leave else y
 
     def linear_plain(self, x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
         """The plain tiled kernel for any sizes and dtypes: the reference beside the tuned ones."""

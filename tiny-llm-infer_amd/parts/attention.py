@@ -77,7 +77,7 @@ class PagedAttention(Mixer):
             None if self.q_norm is None else (self.q_norm.weight, self.q_norm.eps),
             None if self.k_norm is None else (self.k_norm.weight, self.k_norm.eps),
             rot, self.scale, self.window)
-        return ops.linear(o, self.w_o)
+        return ops.linear(o, self.w_o, deferred=True)       # goes to the next norm as the residual delta
 
 
 register_part("mixer", "paged_attention", PagedAttention)

@@ -130,12 +130,15 @@ class Mixer(Part):
 
     def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
         """x: normalised rows [T, hidden] in the run dtype; returns what is
-        added to the residual, same shape."""
+        added to the residual, same shape: a tensor, or whatever
+        ``ops.linear(..., deferred=True)`` returned (a norm's ``forward`` takes
+        either as its delta; ``ops.resolve`` makes a tensor of it)."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
     def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
+        """As ``Mixer.forward``."""
         raise NotImplementedError
 
 

@@ -35,7 +35,7 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
         ops = self.env.ops
-        return ops.linear(ops.linear_swiglu(x, self.w_gate_up), self.w_down)
+        return ops.linear(ops.linear_swiglu(x, self.w_gate_up), self.w_down, deferred=True)   # a delta for the next norm
 
 
 register_part("ffn", "swiglu", SwiGLU)
