@@ -30,6 +30,7 @@
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;       // 16 bytes in flight, as a first-class vector
 
 union Frag {
     uint4 u;
@@ -711,15 +712,20 @@ __device__ __forceinline__ void prefill_lds_block(
     const int full_lo = window > 0 ? max(0, wave_last - window + 1) : 0, full_hi = wave_first;
 
     // staging plan of this thread: chunk e is key row (tid + 256 e) / (HD/8) of the block
-    // for keys, and dim row (tid + 256 e) / (KB/8) for values; fixed over the blocks
+    // for keys, and dim row (tid + 256 e) / (KB/8) for values; fixed over the blocks.
+    // (A thread without a chunk e asks for chunk 0 once more and does not store it: no
+    // load below is under a branch, or the compiler would wait for all loads in flight at
+    // the next use and the prefetching would be undone.)
     int k_key[MAXC], k_dch[MAXC], k_lds[MAXC], v_lds[MAXC];
+    bool mine[MAXC];
     size_t v_dim_off[MAXC];
     const int v_g8 = tid % (KB / 8);                  // this thread's group of 8 keys in every value row
     const size_t head_k = (size_t)kv_head * page_size * HD, page_k = (size_t)kv_heads * page_size * HD;
     const size_t head_v = (size_t)kv_head * HD * page_size, page_v = (size_t)kv_heads * HD * page_size;
 #pragma unroll
     for (int e = 0; e < MAXC; ++e) {
-        const int idx = tid + e * 256;
+        mine[e] = K_CHUNKS % 256 == 0 || tid + e * 256 < K_CHUNKS;
+        const int idx = mine[e] ? tid + e * 256 : 0;
         k_key[e] = idx / (HD / 8);
         k_dch[e] = (idx % (HD / 8)) * 8;
         k_lds[e] = k_key[e] * K_PITCH + k_dch[e];
@@ -727,31 +733,37 @@ __device__ __forceinline__ void prefill_lds_block(
         v_lds[e] = d * V_PITCH + v_g8 * 8;
         v_dim_off[e] = (size_t)d * page_size;
     }
-    uint4 kreg[MAXC], vreg[MAXC];
+    u32x4 kreg[MAXC], vreg[MAXC];
+    // The pages of a block are looked up one block before its keys and values are asked
+    // for, so that an address never waits for a table entry.  A key without a page (past
+    // the table, or released) reads page 0: it lies outside what any row sees.
+    int k_page[MAXC], v_page;
     auto page_of = [&](int key) {
-        const int pidx = key >> page_shift;
-        int page = pidx < table_width ? table[pidx] : 0;
-        return (page < 0 || page >= num_pages) ? 0 : page;
+        const int page = table[min(key >> page_shift, table_width - 1)];
+        return (unsigned)page < (unsigned)num_pages ? page : 0;
+    };
+    auto lookup = [&](int t0) {
+#pragma unroll
+        for (int e = 0; e < MAXC; ++e) k_page[e] = page_of(t0 + k_key[e]);
+        v_page = page_of(t0 + v_g8 * 8);
     };
     auto fetch = [&](int t0) {
         const int vkey = t0 + v_g8 * 8;
-        const bf16_t* vbase = v_cache + (size_t)page_of(vkey) * page_v + head_v + (vkey & (page_size - 1));
+        const bf16_t* vbase = v_cache + (size_t)v_page * page_v + head_v + (vkey & (page_size - 1));
 #pragma unroll
         for (int e = 0; e < MAXC; ++e) {
-            if (K_CHUNKS % 256 == 0 || tid + e * 256 < K_CHUNKS) {
-                const int key = t0 + k_key[e];
-                kreg[e] = *reinterpret_cast<const uint4*>(
-                    k_cache + (size_t)page_of(key) * page_k + head_k + (size_t)(key & (page_size - 1)) * HD + k_dch[e]);
-                vreg[e] = *reinterpret_cast<const uint4*>(vbase + v_dim_off[e]);
-            }
+            const int key = t0 + k_key[e];
+            kreg[e] = *reinterpret_cast<const u32x4*>(
+                k_cache + (size_t)k_page[e] * page_k + head_k + (size_t)(key & (page_size - 1)) * HD + k_dch[e]);
+            vreg[e] = *reinterpret_cast<const u32x4*>(vbase + v_dim_off[e]);
         }
     };
     auto stage = [&]() {
 #pragma unroll
         for (int e = 0; e < MAXC; ++e) {
-            if (K_CHUNKS % 256 == 0 || tid + e * 256 < K_CHUNKS) {
-                *reinterpret_cast<uint4*>(ks + k_lds[e]) = kreg[e];
-                *reinterpret_cast<uint4*>(vs + v_lds[e]) = vreg[e];
+            if (mine[e]) {
+                *reinterpret_cast<u32x4*>(ks + k_lds[e]) = kreg[e];
+                *reinterpret_cast<u32x4*>(vs + v_lds[e]) = vreg[e];
             }
         }
     };
@@ -764,12 +776,16 @@ __device__ __forceinline__ void prefill_lds_block(
     const int vt_off = r * V_PITCH + 8 * c;
 
     int t0 = (wg_lo / KB) * KB;
+    const int t_last = (wg_last / KB) * KB;             // the last block; asked for again rather than branching
+    lookup(t0);
     fetch(t0);
+    lookup(min(t0 + KB, t_last));
     for (; t0 <= wg_last; t0 += KB) {
         __syncthreads();                 // everyone has finished reading the previous block
         stage();
         __syncthreads();
-        if (t0 + KB <= wg_last) fetch(t0 + KB);
+        fetch(min(t0 + KB, t_last));
+        lookup(min(t0 + 2 * KB, t_last));
 #pragma unroll
         for (int sub = 0; sub < KB / 32; ++sub) {
             const int s0 = t0 + sub * 32;
@@ -996,15 +1012,17 @@ extern "C" int tli_attention_prefill_bf16(
     const int rq = group >= 16 ? 1 : 16 / group;
     const int shift = log2_exact(page_size);
     if (page_size >= 8 && direct != 1) {
-        // through LDS: two column tiles a wave for head sizes up to 128 when the portions are
-        // long enough to fill the chip that way; blocks of 64 keys (32 for large heads)
-        bool two = head_dim <= 128 && (long)rows * kv_heads * head_tiles >= (long)8 * rq * 512;
+        // through LDS, blocks of 64 keys (32 for large heads).  Two column tiles a wave (which
+        // leaves room for one workgroup a compute unit) when pairs of its row blocks, a long
+        // one with a short one, still fill the chip; else one tile a wave, two workgroups a unit.
+        const long blocks2 = (rows + 8 * rq - 1) / (8 * rq) + num_seqs;
+        bool two = head_dim <= 128 && blocks2 * kv_heads * head_tiles >= 512;
         if (direct == 2) two = false;
         if (direct == 3 || direct >= 4) two = head_dim <= 128;
         const int rows_per_block = 4 * rq * (two ? 2 : 1);
         const long blocks = (rows + rows_per_block - 1) / rows_per_block + num_seqs;   // upper bound
         if (blocks > 2147483647L) return tli_fail("attention_prefill: too many rows");
-        int pair = blocks * kv_heads * head_tiles >= 1024 ? 1 : 2;
+        int pair = two ? 1 : (blocks * kv_heads * head_tiles >= 1024 ? 1 : 2);
         if (direct >= 4) pair = direct - 4;               // measurements: 4, 5, 6 force the pairing mode
         dim3 grid((unsigned)(pair == 1 ? (blocks + 1) / 2 : blocks), kv_heads * head_tiles);
         const int kb = head_dim <= 128 ? 64 : 32;
