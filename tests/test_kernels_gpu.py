@@ -398,30 +398,37 @@ def test_qkv_to_cache(ops, dtype, case):
     assert torch.equal(step.cache.k.cpu()[untouched], before_k.cpu()[untouched])
 
 
-RAW_DECODE_CASES = [
-    # heads, kv_heads, head_dim, norms, rotation, page, seq_lens, window, writes
-    (32, 8, 128, True, True, 16, [1500, 40, 129, 1, 640], None, True),     # keys split over workgroups
-    (8, 8, 64, True, True, 8, [130, 257, 16, 17], 19, True),
-    (5, 1, 256, False, True, 16, [90, 33], None, True),
-    (6, 2, 192, True, False, 4, [70, 5], 64, True),
-    (16, 1, 64, True, True, 16, [48, 1], None, False),                      # reads another layer's cache
+RAW_CASES = [
+    # heads, kv_heads, head_dim, norms, rotation, page, seq_lens, new rows, window, writes
+    (32, 8, 128, True, True, 16, [1500, 40, 129, 1, 640], [1] * 5, None, True),     # decode, keys split over workgroups
+    (8, 8, 64, True, True, 8, [130, 257, 16, 17], [1] * 4, 19, True),
+    (5, 1, 256, False, True, 16, [90, 33], [1, 1], None, True),
+    (6, 2, 192, True, False, 4, [70, 5], [1, 1], 64, True),
+    (16, 1, 64, True, True, 16, [48, 1], [1, 1], None, False),                      # reads another layer's cache
+    # portions of prompts beside single rows
+    (32, 8, 128, True, True, 16, [300, 64, 1, 77], [130, 64, 1, 1], None, True),
+    (8, 8, 64, True, True, 8, [130, 257], [130, 2], 19, True),
+    (6, 3, 256, True, True, 16, [90, 17], [7, 17], 64, True),
+    (4, 2, 128, False, False, 32, [45], [45], None, True),
+    (16, 1, 64, True, True, 16, [48, 9], [5, 9], None, False),
 ]
 
 
-@pytest.mark.parametrize("case", RAW_DECODE_CASES)
-def test_decode_attention_from_raw_projections(ops, case):
-    """The decode kernel that norms and rotates q and k itself and writes the row's
-    key and value: against float64 mathematics, and the cache it leaves against
-    the two-kernel path's."""
-    heads, kv_heads, hd, norms, rotation, page, seq_lens, window, writes = case
+@pytest.mark.parametrize("case", RAW_CASES)
+def test_attention_from_raw_projections(ops, case):
+    """The attention kernels that norm and rotate q (and for a decode step k, writing the
+    row's key and value) themselves: against float64 mathematics, and the cache they
+    leave against the two-kernel path's."""
+    heads, kv_heads, hd, norms, rotation, page, seq_lens, new_counts, window, writes = case
     dtype = torch.bfloat16
     B = len(seq_lens)
     num_pages = sum((n + page - 1) // page for n in seq_lens) + 3
-    step, tables, pos, seq = make_step(seq_lens, [1] * B, page, num_pages, 7, kv_heads, hd, dtype, window)
+    step, tables, pos, seq = make_step(seq_lens, new_counts, page, num_pages, 7, kv_heads, hd, dtype, window)
     ks, vs = fill_cache(step, tables, seq_lens, kv_heads, hd, dtype, 300)
     step.cache.writes = writes
+    T = len(pos)
     qd, kd = heads * hd, kv_heads * hd
-    qkv = rnd((B, qd + 2 * kd), dtype, 21)
+    qkv = rnd((T, qd + 2 * kd), dtype, 21)
     qw, kw = 1 + rnd((hd,), torch.float32, 22, 0.2), 1 + rnd((hd,), torch.float32, 23, 0.2)
     eps_q, eps_k = 1e-5, 3e-6
     qn = (qw.to(DEV), eps_q) if norms else None
@@ -450,9 +457,9 @@ def test_decode_attention_from_raw_projections(ops, case):
         assert torch.equal(k1, k0) and torch.equal(v1, v0)
     # float64
     x = qkv.double()
-    qq = x[:, :qd].reshape(B, heads, hd)
-    kk = x[:, qd:qd + kd].reshape(B, kv_heads, hd)
-    vv = x[:, qd + kd:].reshape(B, kv_heads, hd)
+    qq = x[:, :qd].reshape(T, heads, hd)
+    kk = x[:, qd:qd + kd].reshape(T, kv_heads, hd)
+    vv = x[:, qd + kd:].reshape(T, kv_heads, hd)
     if norms:
         qq = qw.double() * qq / torch.sqrt((qq * qq).mean(-1, keepdim=True) + eps_q)
         kk = kw.double() * kk / torch.sqrt((kk * kk).mean(-1, keepdim=True) + eps_k)
@@ -463,11 +470,11 @@ def test_decode_attention_from_raw_projections(ops, case):
             a, b = t[..., :half], t[..., half:]
             return torch.cat([a * c - b * sn, a * sn + b * c], -1)
         qq, kk = rot(qq), rot(kk)
-    if writes:                      # the row's own key and value replace what the cache held there
-        for i in range(B):
-            ks[i][-1] = kk[i].to(dtype)
-            vs[i][-1] = vv[i].to(dtype)
-    want = ref_attention(qq.reshape(B, qd).to(dtype), ks, vs, pos, seq, heads, kv_heads, scale, window)
+    if writes:                      # the rows' own keys and values replace what the cache held there
+        for r in range(T):
+            ks[seq[r]][pos[r]] = kk[r].to(dtype)
+            vs[seq[r]][pos[r]] = vv[r].to(dtype)
+    want = ref_attention(qq.reshape(T, qd).to(dtype), ks, vs, pos, seq, heads, kv_heads, scale, window)
     close(out, want, dtype, "attention from raw projections")
     close(out2, want, dtype, "attention through two kernels")
 

@@ -656,7 +656,7 @@ __device__ __forceinline__ void prefill_lds_block(
     const bf16_t* __restrict__ v_cache, const int* __restrict__ row_start,
     const int* __restrict__ seq_start, int num_seqs, const int* __restrict__ tables, int table_width,
     int page_size, int page_shift, int num_pages, int heads, int kv_heads, float scale_log2, int window,
-    int rq, int block, int head_index) {
+    int rq, int block, int head_index, const RawQkv& raw) {
     constexpr int HD = ND * 16;
     constexpr int K_PITCH = HD + 8;                   // elements per key row in LDS
     constexpr int V_PITCH = KB + 8;                   // elements per value (dim) row in LDS
@@ -701,7 +701,17 @@ __device__ __forceinline__ void prefill_lds_block(
         tile_init(t[ct]);
         t[ct].pos = live[ct] ? pos : -1;
         t[ct].lo = live[ct] ? (window > 0 ? max(0, pos - window + 1) : 0) : 0;
-        tile_load_q(t[ct], q + ((size_t)row[ct] * heads + head) * HD, HD, live[ct]);
+        if (NJ * 2 == ND && raw.qkv) {
+            // the query from the raw projections: this row's head, normed and rotated here
+            // (an idle column computes on the first row of the portion; it is masked)
+            const int at = live[ct] ? pos : start;
+            const float* cos_row = raw.cos ? raw.cos + (size_t)at * (HD / 2) : nullptr;
+            const float* sin_row = raw.cos ? raw.sin + (size_t)at * (HD / 2) : nullptr;
+            head_from_raw<NJ>(t[ct].q, raw.qkv + ((size_t)row[ct] * (heads + 2 * kv_heads) + head) * HD,
+                              raw.q_norm_w, raw.q_eps, cos_row, sin_row);
+        } else {
+            tile_load_q(t[ct], q + ((size_t)row[ct] * heads + head) * HD, HD, live[ct]);
+        }
     }
     // keys the workgroup walks, and those this wave needs
     const int wg_first = start + block0, wg_last = wg_first + block_rows - 1;
@@ -825,6 +835,8 @@ __device__ __forceinline__ void prefill_lds_block(
     }
 }
 
+// With raw.qkv the queries are taken from the raw projections (normed and rotated here, q
+// is not read); needs head_dim == 32*NJ.
 // grid (row blocks, kv_heads * head_tiles), or with `pair` (ceil(row blocks / 2), ...):
 // row blocks late in a sequence walk more keys than early ones, so when there are
 // workgroups to spare each takes block (last - b) and then block b, and all do about
@@ -836,7 +848,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
                              const int* __restrict__ row_start, const int* __restrict__ seq_start,
                              int num_seqs, const int* __restrict__ tables, int table_width, int page_size,
                              int page_shift, int num_pages, int heads, int kv_heads,
-                             float scale_log2, int window, int rq, int pair) {
+                             float scale_log2, int window, int rq, int pair, RawQkv raw) {
     const int rows_per_block = 4 * CT * rq;
     int total = 0;
     for (int seq = 0; seq < num_seqs; ++seq)
@@ -864,19 +876,19 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
         (void)linear;
         prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                           table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                          scale_log2, window, rq, rb, hd_i);
+                                          scale_log2, window, rq, rb, hd_i, raw);
         return;
     }
     const int first = blockIdx.x, second = pair ? total - 1 - first : first;
     if (first >= total || first > second) return;
     prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                       table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                      scale_log2, window, rq, second, blockIdx.y);
+                                      scale_log2, window, rq, second, blockIdx.y, raw);
     if (second != first) {
         __syncthreads();
         prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                           table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                          scale_log2, window, rq, first, blockIdx.y);
+                                          scale_log2, window, rq, first, blockIdx.y, raw);
     }
 }
 
@@ -1000,17 +1012,21 @@ extern "C" int tli_qkv_attention_decode_bf16(
 // Rows of a sequence are contiguous and ascend in position; row_start has num_seqs+1 entries.
 // direct = 1: every wave reads its keys and values straight from the cache (no LDS staging);
 // 0: through LDS, tiles per wave by shape; 2, 3: through LDS with one, two tiles per wave.
-extern "C" int tli_attention_prefill_bf16(
+static int launch_prefill(
     const void* q, void* out, const void* k_cache, const void* v_cache, const int* row_start,
     const int* seq_start, int num_seqs, int rows, const int* tables, int table_width, int page_size,
     int num_pages, int heads, int kv_heads, int head_dim, float scale, int window, int direct,
-    void* stream) {
+    const RawQkv* raw_in, void* stream) {
     if (rows <= 0 || num_seqs <= 0) return 0;
     if (check_common("attention_prefill", heads, kv_heads, head_dim, page_size, table_width, num_pages)) return 1;
     hipStream_t s = (hipStream_t)stream;
     const int group = heads / kv_heads, head_tiles = (group + 15) / 16;
     const int rq = group >= 16 ? 1 : 16 / group;
     const int shift = log2_exact(page_size);
+    if (raw_in && (head_dim % 64 || page_size < 8 || direct == 1))
+        return tli_fail("attention_prefill from raw projections: head_dim %d must be a multiple of 64, pages "
+                        "of at least 8 (%d), through LDS", head_dim, page_size);
+    const RawQkv raw = raw_in ? *raw_in : RawQkv{};
     if (page_size >= 8 && direct != 1) {
         // through LDS, blocks of 64 keys (32 for large heads).  Two column tiles a wave (which
         // leaves room for one workgroup a compute unit) when pairs of its row blocks, a long
@@ -1030,7 +1046,7 @@ extern "C" int tli_attention_prefill_bf16(
 #define ARGS (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, row_start, \
              seq_start, num_seqs, tables, table_width, page_size, shift, num_pages, heads, kv_heads
 #define TAIL scale * LOG2E, window, rq
-#define TAIL_LDS scale * LOG2E, window, rq, pair
+#define TAIL_LDS scale * LOG2E, window, rq, pair, raw
 #define CALL(NJ, ND)                                                                                    \
     if (ND <= 8 && two) attention_prefill_lds_kernel<NJ, (ND <= 8 ? ND : 1), 2, 64><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS); \
     else if (ND <= 8) attention_prefill_lds_kernel<NJ, (ND <= 8 ? ND : 1), 1, 64><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS);   \
@@ -1052,4 +1068,29 @@ extern "C" int tli_attention_prefill_bf16(
 #undef TAIL_LDS
     }
     return tli_check_launch("attention_prefill");
+}
+
+extern "C" int tli_attention_prefill_bf16(
+    const void* q, void* out, const void* k_cache, const void* v_cache, const int* row_start,
+    const int* seq_start, int num_seqs, int rows, const int* tables, int table_width, int page_size,
+    int num_pages, int heads, int kv_heads, int head_dim, float scale, int window, int direct,
+    void* stream) {
+    return launch_prefill(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, rows, tables, table_width,
+                          page_size, num_pages, heads, kv_heads, head_dim, scale, window, direct, nullptr, stream);
+}
+
+// The same with the queries taken from the raw projections qkv [rows][(heads + 2 kv_heads) * head_dim]
+// (per-head norm if q_norm_w, rotation of the whole head if cos_table), the keys and values
+// already in the cache.  head_dim a multiple of 64, pages of at least 8, direct != 1.
+extern "C" int tli_qkv_attention_prefill_bf16(
+    const void* qkv, void* out, const void* k_cache, const void* v_cache, const int* row_start,
+    const int* seq_start, int num_seqs, int rows, const int* tables, int table_width, int page_size,
+    int num_pages, int heads, int kv_heads, int head_dim, const float* q_norm_w, float q_eps,
+    const float* cos_table, const float* sin_table, float scale, int window, int direct, void* stream) {
+    if (!qkv) return tli_fail("attention_prefill from raw projections: no projections");
+    if ((cos_table == nullptr) != (sin_table == nullptr)) return tli_fail("attention_prefill: cos without sin");
+    const RawQkv raw{(const bf16_t*)qkv, q_norm_w, nullptr, cos_table, sin_table, q_eps, 0.f, 0};
+    return launch_prefill(nullptr, out, k_cache, v_cache, row_start, seq_start, num_seqs, rows, tables,
+                          table_width, page_size, num_pages, heads, kv_heads, head_dim, scale, window, direct,
+                          &raw, stream);
 }

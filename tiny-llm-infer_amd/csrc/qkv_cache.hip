@@ -113,11 +113,11 @@ qkv_to_cache_wide_kernel(
     int heads, int kv_heads,
     const float* __restrict__ q_norm_w, float q_eps, const float* __restrict__ k_norm_w, float k_eps,
     const float* __restrict__ cos_table, const float* __restrict__ sin_table, int table_positions,
-    int write_cache) {
+    int write_cache, int first_unit) {
     constexpr int HD = 64 * EPL;
     const int row = blockIdx.x;
     const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE;
-    const int h = blockIdx.y * QKV_WAVES + wave;
+    const int h = first_unit + blockIdx.y * QKV_WAVES + wave;      // first_unit = heads: keys and values only
     if (h >= heads + 2 * kv_heads) return;
     const int q_dim = heads * HD, kv_dim = kv_heads * HD;
     const int pos = positions[row];
@@ -205,13 +205,21 @@ extern "C" int tli_qkv_to_cache(
     const int units = heads + 2 * kv_heads;
     if ((units + QKV_WAVES - 1) / QKV_WAVES > 65535) return tli_fail("qkv_to_cache: too many heads");
     dim3 grid(rows, (units + QKV_WAVES - 1) / QKV_WAVES);
-    if (dtype == TLI_BF16 && head_dim % 64 == 0 && head_dim <= 256 && head_dim != 192 &&
-        (!cos_table || rotary_dim == head_dim)) {
+    const bool wide = dtype == TLI_BF16 && head_dim % 64 == 0 && head_dim <= 256 && head_dim != 192 &&
+                      (!cos_table || rotary_dim == head_dim);
+    // without q_out only keys and values are done (the attention kernel takes q from qkv itself)
+    const int first_unit = q_out ? 0 : heads;
+    if (!q_out) {
+        if (!wide) return tli_fail("qkv_to_cache: keys and values alone only for bfloat16 heads of 64, 128 or 256");
+        if (!write_cache) return 0;
+        grid.y = (2 * kv_heads + QKV_WAVES - 1) / QKV_WAVES;
+    }
+    if (wide) {
 #define WIDE(EPL)                                                                                        \
     qkv_to_cache_wide_kernel<EPL><<<grid, threads, 0, s>>>(                                              \
         (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, positions, seq_of_row,   \
         tables, table_width, page_size, num_pages, heads, kv_heads, q_norm_w, q_eps, k_norm_w, k_eps,    \
-        cos_table, sin_table, table_positions, write_cache)
+        cos_table, sin_table, table_positions, write_cache, first_unit)
         if (head_dim == 64) WIDE(1);
         else if (head_dim == 128) WIDE(2);
         else WIDE(4);

@@ -62,6 +62,7 @@ def load_library():
         "tli_qkv_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I,
                                           F, I, I, I, P],
         "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, I, P],
+        "tli_qkv_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, P, F, P, P, F, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
         "tli_sample_scratch_bytes": [I],
     }
@@ -307,11 +308,13 @@ class HipOps:
                    _dtype_code(gu.dtype), self._stream())
         return out
 
-    def qkv_to_cache(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary):
+    def qkv_to_cache(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary, queries=True):
+        """Norms and rotation of q and k, k and v into the cache; returns q.  Without
+        ``queries`` only the keys and values are done (bfloat16 heads of 64, 128, 256)."""
         T = step.num_rows
         q_dim, kv_dim = heads * head_dim, kv_heads * head_dim
         self._want(qkv, "qkv", None, (T, q_dim + 2 * kv_dim))
-        q = torch.empty((T, q_dim), dtype=qkv.dtype, device=self.device)
+        q = torch.empty((T, q_dim), dtype=qkv.dtype, device=self.device) if queries else None
         qw, qe = q_norm if q_norm is not None else (None, 0.0)
         kw, ke = k_norm if k_norm is not None else (None, 0.0)
         for w in (qw, kw):
@@ -335,7 +338,7 @@ class HipOps:
             self._check_cache(kc, vc, g, kv_heads, head_dim, qkv.dtype, step)
             k_ptr, v_ptr, tab_ptr = kc.data_ptr(), vc.data_ptr(), g.tables.data_ptr()
             width, page, pages = g.table_width, g.page_size, kc.shape[0]
-        self._call(self.lib.tli_qkv_to_cache, qkv.data_ptr(), q.data_ptr(), k_ptr, v_ptr,
+        self._call(self.lib.tli_qkv_to_cache, qkv.data_ptr(), _ptr(q), k_ptr, v_ptr,
                    step.positions.data_ptr(), step.seq_of_row.data_ptr(), tab_ptr, width, page, pages,
                    T, heads, kv_heads, head_dim, _ptr(qw), float(qe), _ptr(kw), float(ke),
                    _ptr(cos), _ptr(sin), rd, npos, write, _dtype_code(qkv.dtype), self._stream())
@@ -377,10 +380,15 @@ class HipOps:
         and k, k and v into the cache, attention over the cache.  A decode step (one
         row a sequence) does all of it in the attention kernel where the sizes allow;
         other steps run qkv_to_cache and paged_attention."""
-        fused = (qkv.dtype == torch.bfloat16 and step.max_rows_per_seq == 1 and cache is not None
-                 and head_dim % 64 == 0 and head_dim <= 256 and heads // kv_heads <= 16
-                 and cache.group.page_size >= 4 and not self.force_plain and not self.unfused_decode
-                 and (rotary is None or rotary[2] == head_dim))
+        fusable = (qkv.dtype == torch.bfloat16 and cache is not None and head_dim % 64 == 0
+                   and head_dim <= 256 and not self.force_plain and not self.unfused_decode
+                   and (rotary is None or rotary[2] == head_dim))
+        if (fusable and step.max_rows_per_seq > 1 and head_dim != 192 and cache.group.page_size >= 8
+                and self.prefill_direct != 1):
+            return self._qkv_attention_prefill(qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm,
+                                               rotary, scale, window)
+        fused = (fusable and step.max_rows_per_seq == 1 and heads // kv_heads <= 16
+                 and cache.group.page_size >= 4)
         if not fused:
             q = self.qkv_to_cache(qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary)
             return self.paged_attention(q, step, cache, heads, kv_heads, head_dim, scale, window)
@@ -409,6 +417,25 @@ class HipOps:
                    head_dim, _ptr(qw), float(qe), _ptr(kw), float(ke), _ptr(cos), _ptr(sin),
                    1 if cache.writes else 0, float(scale), int(window or 0), splits, per_split,
                    self._stream())
+        return out
+
+    def _qkv_attention_prefill(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary,
+                               scale, window):
+        """Portions of prompts: keys and values go into the cache in one pass, the
+        attention kernel norms and rotates its queries itself (a query is read by
+        one wave only, so nothing is done twice and q is never written)."""
+        T = step.num_rows
+        self.qkv_to_cache(qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary, queries=False)
+        kc, vc, g = cache.k, cache.v, cache.group
+        self._check_cache(kc, vc, g, kv_heads, head_dim, qkv.dtype, step)
+        qw, qe = q_norm if q_norm is not None else (None, 0.0)
+        cos, sin = (rotary[0], rotary[1]) if rotary is not None else (None, None)
+        out = torch.empty((T, heads * head_dim), dtype=qkv.dtype, device=self.device)
+        self._call(self.lib.tli_qkv_attention_prefill_bf16, qkv.data_ptr(), out.data_ptr(), kc.data_ptr(),
+                   vc.data_ptr(), step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs,
+                   T, g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], heads, kv_heads,
+                   head_dim, _ptr(qw), float(qe), _ptr(cos), _ptr(sin), float(scale), int(window or 0),
+                   int(self.prefill_direct), self._stream())
         return out
 
     def _decode_splits(self, step, g, heads, kv_heads, head_dim, window):
