@@ -113,12 +113,13 @@ qkv_to_cache_wide_kernel(
     int heads, int kv_heads,
     const float* __restrict__ q_norm_w, float q_eps, const float* __restrict__ k_norm_w, float k_eps,
     const float* __restrict__ cos_table, const float* __restrict__ sin_table, int table_positions,
-    int write_cache, int first_unit) {
+    int write_cache, int first_unit, int end_unit) {
     constexpr int HD = 64 * EPL;
     const int row = blockIdx.x;
     const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE;
-    const int h = first_unit + blockIdx.y * QKV_WAVES + wave;      // first_unit = heads: keys and values only
-    if (h >= heads + 2 * kv_heads) return;
+    // units first_unit .. end_unit-1 of: q heads, k heads, v heads
+    const int h = first_unit + blockIdx.y * QKV_WAVES + wave;
+    if (h >= end_unit) return;
     const int q_dim = heads * HD, kv_dim = kv_heads * HD;
     const int pos = positions[row];
     const bf16_t* src = qkv + (size_t)row * (q_dim + 2 * kv_dim) + (size_t)h * HD + lane * EPL;
@@ -185,13 +186,92 @@ qkv_to_cache_wide_kernel(
     }
 }
 
+// The values of a step's rows into the cache, for steps that bring many rows a sequence: a
+// workgroup takes up to G consecutive positions of one sequence that share a page and one kv
+// head; a thread reads one dim of each of them (a wave reads whole rows) and writes them as one
+// run of consecutive slots, where the kernels above write every (row, dim) as 2 bytes of its own.
+// grid (groups upper bound, kv_heads).
+template <int G>
+__global__ void values_to_cache_kernel(
+    const bf16_t* __restrict__ qkv, bf16_t* __restrict__ v_cache, const int* __restrict__ row_start,
+    const int* __restrict__ seq_start, int num_seqs, const int* __restrict__ tables, int table_width,
+    int page_size, int num_pages, int heads, int kv_heads, int head_dim) {
+    int grp = blockIdx.x, seq = 0, start = 0, first_row = 0, n_rows = 0;
+    for (; seq < num_seqs; ++seq) {
+        first_row = row_start[seq];
+        n_rows = row_start[seq + 1] - first_row;
+        start = seq_start[seq];
+        const int groups = n_rows > 0 ? (start + n_rows - 1) / G - start / G + 1 : 0;
+        if (grp < groups) break;
+        grp -= groups;
+    }
+    if (seq >= num_seqs) return;
+    const int g0 = start / G + grp;
+    const int p_lo = max(start, g0 * G), p_hi = min(start + n_rows, (g0 + 1) * G);
+    const int n = p_hi - p_lo;
+    const int page = tables[(size_t)seq * table_width + p_lo / page_size];
+    if (page < 0 || page >= num_pages) return;
+    const int slot0 = p_lo % page_size, kvh = blockIdx.y;
+    const size_t stride = (size_t)(heads + 2 * kv_heads) * head_dim;
+    const bf16_t* src = qkv + (size_t)(first_row + p_lo - start) * stride + (size_t)(heads + kv_heads + kvh) * head_dim;
+    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+        bf16_t vals[G];
+#pragma unroll
+        for (int j = 0; j < G; ++j) vals[j] = j < n ? src[(size_t)j * stride + d] : (bf16_t)0;
+        bf16_t* dst = v_cache + (((size_t)page * kv_heads + kvh) * head_dim + d) * page_size + slot0;
+        if (n == G) {               // a whole group: its slots start at a multiple of G
+            uint32_t w[G / 2];
+#pragma unroll
+            for (int j = 0; j < G / 2; ++j) w[j] = (uint32_t)vals[2 * j] | ((uint32_t)vals[2 * j + 1] << 16);
+            if (G == 16) {
+                reinterpret_cast<uint4*>(dst)[0] = make_uint4(w[0], w[1], w[2], w[3]);
+                reinterpret_cast<uint4*>(dst)[1] = make_uint4(w[4 % (G / 2)], w[5 % (G / 2)], w[6 % (G / 2)], w[7 % (G / 2)]);
+            } else if (G == 8) {
+                reinterpret_cast<uint4*>(dst)[0] = make_uint4(w[0], w[1], w[2], w[3]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < G / 2; ++j) reinterpret_cast<uint32_t*>(dst)[j] = w[j];
+            }
+        } else {
+            for (int j = 0; j < n; ++j) dst[j] = vals[j];
+        }
+    }
+}
+
+// rows: the step's rows; row_start/seq_start as the prefill attention takes them.  bfloat16.
+extern "C" int tli_values_to_cache(
+    const void* qkv, void* v_cache, const int* row_start, const int* seq_start, int num_seqs, int rows,
+    const int* tables, int table_width, int page_size, int num_pages, int heads, int kv_heads,
+    int head_dim, void* stream) {
+    if (rows <= 0 || num_seqs <= 0) return 0;
+    if (head_dim <= 0 || heads <= 0 || kv_heads <= 0 || kv_heads > 65535) return tli_fail("values_to_cache: bad head sizes");
+    if (page_size < 2 || (page_size & (page_size - 1)) || table_width <= 0 || num_pages <= 0)
+        return tli_fail("values_to_cache: bad cache geometry (pages of a power of two, at least 2)");
+    hipStream_t s = (hipStream_t)stream;
+    const int G = page_size >= 16 ? 16 : page_size;
+    const long groups = (long)rows / G + 2L * num_seqs;           // upper bound
+    if (groups > 2147483647L) return tli_fail("values_to_cache: too many rows");
+    dim3 grid((unsigned)groups, kv_heads);
+    const int threads = head_dim <= 64 ? 64 : (head_dim <= 128 ? 128 : 256);
+#define VALUES(GG)                                                                                       \
+    values_to_cache_kernel<GG><<<grid, threads, 0, s>>>((const bf16_t*)qkv, (bf16_t*)v_cache, row_start, \
+        seq_start, num_seqs, tables, table_width, page_size, num_pages, heads, kv_heads, head_dim)
+    if (G == 16) VALUES(16);
+    else if (G == 8) VALUES(8);
+    else if (G == 4) VALUES(4);
+    else VALUES(2);
+#undef VALUES
+    return tli_check_launch("values_to_cache");
+}
+
+// skip_values: the values are written by tli_values_to_cache instead.
 extern "C" int tli_qkv_to_cache(
     const void* qkv, void* q_out, void* k_cache, void* v_cache, const int* positions,
     const int* seq_of_row, const int* tables, int table_width, int page_size, int num_pages,
     int rows, int heads, int kv_heads, int head_dim,
     const float* q_norm_w, float q_eps, const float* k_norm_w, float k_eps,
     const float* cos_table, const float* sin_table, int rotary_dim, int table_positions,
-    int write_cache, int dtype, void* stream) {
+    int write_cache, int skip_values, int dtype, void* stream) {
     if (rows <= 0) return 0;
     if (head_dim <= 0 || head_dim > QKV_MAX_HEAD_DIM)
         return tli_fail("qkv_to_cache: head_dim %d is outside 1..%d", head_dim, QKV_MAX_HEAD_DIM);
@@ -208,18 +288,18 @@ extern "C" int tli_qkv_to_cache(
     const bool wide = dtype == TLI_BF16 && head_dim % 64 == 0 && head_dim <= 256 && head_dim != 192 &&
                       (!cos_table || rotary_dim == head_dim);
     // without q_out only keys and values are done (the attention kernel takes q from qkv itself)
-    const int first_unit = q_out ? 0 : heads;
-    if (!q_out) {
-        if (!wide) return tli_fail("qkv_to_cache: keys and values alone only for bfloat16 heads of 64, 128 or 256");
-        if (!write_cache) return 0;
-        grid.y = (2 * kv_heads + QKV_WAVES - 1) / QKV_WAVES;
+    const int first_unit = q_out ? 0 : heads, end_unit = heads + (skip_values ? 1 : 2) * kv_heads;
+    if (!q_out || skip_values) {
+        if (!wide) return tli_fail("qkv_to_cache: a part of the heads only for bfloat16 heads of 64, 128 or 256");
+        if (!q_out && !write_cache) return 0;
+        grid.y = (end_unit - first_unit + QKV_WAVES - 1) / QKV_WAVES;
     }
     if (wide) {
 #define WIDE(EPL)                                                                                        \
     qkv_to_cache_wide_kernel<EPL><<<grid, threads, 0, s>>>(                                              \
         (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, positions, seq_of_row,   \
         tables, table_width, page_size, num_pages, heads, kv_heads, q_norm_w, q_eps, k_norm_w, k_eps,    \
-        cos_table, sin_table, table_positions, write_cache, first_unit)
+        cos_table, sin_table, table_positions, write_cache, first_unit, end_unit)
         if (head_dim == 64) WIDE(1);
         else if (head_dim == 128) WIDE(2);
         else WIDE(4);

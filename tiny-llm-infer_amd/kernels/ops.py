@@ -51,7 +51,8 @@ def load_library():
         "tli_feed_tokens": [P, P, P, I, I, P],
         "tli_add_rmsnorm": [P, P, P, P, P, I, I, I, F, I, I, P],
         "tli_swiglu": [P, P, I, I, I, P],
-        "tli_qkv_to_cache": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I, I, I, I, P],
+        "tli_qkv_to_cache": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I, I, I, I, I, P],
+        "tli_values_to_cache": [P, P, P, P, I, I, P, I, I, I, I, I, I, P],
         "tli_attention_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
         "tli_gemm_plain": [P, P, P, I, I, I, I, I, I, P],
         "tli_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, I, P],
@@ -310,7 +311,8 @@ class HipOps:
 
     def qkv_to_cache(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary, queries=True):
         """Norms and rotation of q and k, k and v into the cache; returns q.  Without
-        ``queries`` only the keys and values are done (bfloat16 heads of 64, 128, 256)."""
+        ``queries`` only the keys and values are done (bfloat16 heads of 64, 128, 256),
+        the values by a kernel of their own that writes runs of slots."""
         T = step.num_rows
         q_dim, kv_dim = heads * head_dim, kv_heads * head_dim
         self._want(qkv, "qkv", None, (T, q_dim + 2 * kv_dim))
@@ -341,7 +343,12 @@ class HipOps:
         self._call(self.lib.tli_qkv_to_cache, qkv.data_ptr(), _ptr(q), k_ptr, v_ptr,
                    step.positions.data_ptr(), step.seq_of_row.data_ptr(), tab_ptr, width, page, pages,
                    T, heads, kv_heads, head_dim, _ptr(qw), float(qe), _ptr(kw), float(ke),
-                   _ptr(cos), _ptr(sin), rd, npos, write, _dtype_code(qkv.dtype), self._stream())
+                   _ptr(cos), _ptr(sin), rd, npos, write, 0 if queries else 1, _dtype_code(qkv.dtype),
+                   self._stream())
+        if write and not queries:
+            self._call(self.lib.tli_values_to_cache, qkv.data_ptr(), v_ptr, step.row_start.data_ptr(),
+                       step.seq_start.data_ptr(), step.num_seqs, T, tab_ptr, width, page, pages, heads,
+                       kv_heads, head_dim, self._stream())
         return q
 
     def _check_cache(self, kc, vc, g, kv_heads, head_dim, dtype, step):
