@@ -30,6 +30,13 @@ TINY = {
               use_sliding_window=True, sliding_window=19,
               layer_types=["sliding_attention", "full_attention", "sliding_attention", "full_attention"],
               seed=37, page_size=32),
+    # heads of 64: the attention kernels that take q (and for decode steps k and v) from the
+    # raw projections themselves; one windowed layer, one not
+    "D": dict(hidden_size=128, intermediate_size=192, num_hidden_layers=2, num_attention_heads=4,
+              num_key_value_heads=2, head_dim=64, vocab_size=320, max_position_embeddings=512,
+              rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+              use_sliding_window=True, sliding_window=24,
+              layer_types=["sliding_attention", "full_attention"], seed=41, page_size=8),
 }
 
 

@@ -61,7 +61,7 @@ def oracle(model_folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("cut", ["whole", "decode", "portions", "mixed"])
 def test_cuts_match_plain(model_folders, oracle, name, dtype, cut):
     reqs, want = oracle[name]
