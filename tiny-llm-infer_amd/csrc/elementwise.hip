@@ -109,13 +109,14 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const void* __
     float* x = resid + (size_t)r * n;
     const RowDelta<T> d = row_delta<T>(delta, parts, r, n, total_rows);
     const bool update = (rows == nullptr) && d.any();
-    float v[IT][4];
+    float v[IT][4], w[IT][4];
     float ss = 0.f;
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
         const int i = (threadIdx.x + it * blockDim.x) * 4;
         if (i < n) {
             load4(x + i, v[it]);
+            load4(weight + i, w[it]);         // asked for now: after the sum it would be one more wait for memory
             if (d.any()) {
                 float dv[4];
                 if (d.parts > 0) {
@@ -145,10 +146,9 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const void* __
     for (int it = 0; it < IT; ++it) {
         const int i = (threadIdx.x + it * blockDim.x) * 4;
         if (i < n) {
-            float w[4], y[4];
-            load4(weight + i, w);
+            float y[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) y[e] = w[e] * v[it][e] * scale;
+            for (int e = 0; e < 4; ++e) y[e] = w[it][e] * v[it][e] * scale;
             store4(o + i, y);
         }
     }
