@@ -84,6 +84,18 @@ def test_temperature_tokens_do_not_depend_on_the_batch(model_folders):
     assert [r.token_ids for r in greedy] != [r.token_ids for r in together]
 
 
+def test_counters(model_folders):
+    eng = _engine(model_folders["A"], "A", num_kv_blocks=40, enable_prefix_caching=True)
+    prompt = random_prompt(256, 20, 3)
+    eng.generate([prompt, prompt[:17] + [1, 2]], SamplingParams(max_tokens=5))
+    st = eng.stats()
+    assert st["generated_tokens"] == 10 and st["steps"] >= 5
+    assert st["waiting"] == 0 and st["running"] == 0 and st["preemptions"] == 0
+    assert st["pages"] == 40 and st["pages_taken_total"] > 0
+    eng.generate([prompt], SamplingParams(max_tokens=2))
+    assert eng.stats()["prefix_pages_reused"] >= 2          # whole pages of the same prompt
+
+
 def test_prefix_caching_gives_the_same_tokens_and_skips_work(model_folders):
     folder = model_folders["A"]
     shared = random_prompt(256, 40, 9)

@@ -208,6 +208,10 @@ def run_benchmark(argv: List[str]) -> int:
         print(f"aggregate_runs={args.repeats} output_tokens={total_tokens} elapsed_seconds={total_time:.4f} "
               f"output_tokens_per_second={total_tokens / total_time:.2f} "
               f"median_output_tokens_per_second={statistics.median(rates):.2f}")
+    st = engine.stats()
+    print(f"engine_steps={st['steps']} preemptions={st['preemptions']} "
+          f"pages_free={min(st['pages_free'])}/{st['pages']} prefix_pages_reused={st['prefix_pages_reused']}",
+          file=sys.stderr)
     return 0
 
 

@@ -127,6 +127,25 @@ class LLMEngine:
     def is_eos(self, token: int) -> bool:
         return token in self.eos_token_ids
 
+    def stats(self) -> dict:
+        """Counters since construction (the reference counts generated tokens only,
+        engine/include/llm_engine.h:46)."""
+        cache = self.runner.cache
+        with self._lock:
+            return {
+                "steps": self.num_steps,
+                "steps_launched_ahead": self.num_steps_ahead,
+                "generated_tokens": self.total_generated_tokens,
+                "preemptions": self.scheduler.num_preemptions,
+                "waiting": len(self.scheduler.waiting),
+                "running": len(self.scheduler.running),
+                "pages": cache.num_pages,
+                "pages_free": cache.free_pages(),          # one count per group of layers
+                "pages_taken_total": cache.pages_taken_total,
+                "prefix_pages_reused": cache.prefix_hits,
+                "recorded_decode_shapes": len(self.runner.graphs),
+            }
+
     # ---- one step -------------------------------------------------------------------
     def _launch(self, plan: BatchPlan, ahead_of: Optional["_Inflight"] = None) -> "_Inflight":
         """Put one planned step on the device: the batch, then the sampling.  Nothing
