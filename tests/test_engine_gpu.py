@@ -180,6 +180,27 @@ def test_recorded_decode_steps_equal_eager_ones(model_folders):
     assert compared > 30 and fast.graph_replays == compared and len(fast.graphs) >= 3
 
 
+def test_decode_steps_are_padded_to_few_sizes(model_folders):
+    """Seven requests that finish one after the other: the recorded decode steps come in
+    the sizes 8, 4, 2 and 1 only (steps of other sizes are filled with rows of no
+    request), and the tokens are those of an engine that records nothing."""
+    from tiny_llm_infer_amd.sampling.params import SamplingParams
+    folder = model_folders["D"]
+    prompts = [random_prompt(320, 6 + 3 * i, 70 + i) for i in range(7)]
+    params = [SamplingParams(max_tokens=4 + 5 * i, ignore_eos=True) for i in range(7)]
+    args = dict(max_num_seqs=8, max_num_batched_tokens=128, max_model_len=128)
+    eng = _engine(folder, "D", "bfloat16", **args)
+    got = eng.generate(prompts, params)
+    assert eng.runner.graph_replays > 20
+    assert {k[0] for k in eng.runner.graphs} == {8, 4, 2, 1}
+    plain = _engine(folder, "D", "bfloat16", **args)
+    plain.runner.use_graphs = False
+    want = plain.generate(prompts, params)
+    assert [r.token_ids for r in got] == [r.token_ids for r in want]
+    eng.runner.cache.check()
+    assert all(f == eng.runner.cache.num_pages for f in eng.runner.cache.free_pages())
+
+
 def test_prefix_caching_on_the_gpu(model_folders):
     """Requests that share a prompt prefix take its pages over instead of computing
     them; the tokens are those of an engine without the cache."""

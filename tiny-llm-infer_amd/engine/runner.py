@@ -47,6 +47,12 @@ def _pad4(n: int) -> int:
     return (n + 3) & ~3
 
 
+def _decode_bucket(n: int) -> int:
+    """Recorded decode steps come in these numbers of rows: powers of two up to 64 (up to
+    16 rows, and from 17 to 64, the matrix products cost the same), then multiples of 32."""
+    return _pow2_at_least(n, 1) if n <= 64 else (n + 31) // 32 * 32
+
+
 class StepInputs:
     """One host staging buffer and one device buffer that hold every integer
     input of a step; a step costs one host-to-device copy.  The layout depends
@@ -113,16 +119,19 @@ class ModelRunner:
             n, heads, hd = len(g.cache_layers), g.need.num_kv_heads, g.need.head_dim
             # keys [.., slot, head_dim]; values transposed [.., head_dim, slot]: both are
             # then contiguous along the index the matrix cores contract over
-            k = torch.zeros((n, num_pages, heads, page_size, hd), dtype=env.dtype, device=env.device)
-            v = torch.zeros((n, num_pages, heads, hd, page_size), dtype=env.dtype, device=env.device)
+            # (one page and one state slot more than the manager hands out: what the
+            # padding rows of a recorded decode step write to)
+            k = torch.zeros((n, num_pages + 1, heads, page_size, hd), dtype=env.dtype, device=env.device)
+            v = torch.zeros((n, num_pages + 1, heads, hd, page_size), dtype=env.dtype, device=env.device)
             self.group_tensors.append((k, v))
+        self.pad_page, self.pad_slot = num_pages, max_requests
         self.states: List[Optional[torch.Tensor]] = []
         for need in model.state_needs():
             self.states.append(None if need is None else torch.zeros(
-                (max_requests,) + tuple(need.shape), dtype=need.dtype, device=env.device))
+                (max_requests + 1,) + tuple(need.shape), dtype=need.dtype, device=env.device))
         max_width = _pow2_at_least((self.max_model_len + page_size - 1) // page_size)
-        self.inputs = StepInputs(env.device, max_batch_tokens, max_requests,
-                                 len(self.cache.groups), max_width)
+        self.inputs = StepInputs(env.device, max(max_batch_tokens, _decode_bucket(max_requests)),
+                                 _decode_bucket(max_requests), len(self.cache.groups), max_width)
         self.steps_run = 0
         # Decode steps (one token for every request, every logit wanted) launch the same
         # kernels with the same arguments whenever (requests, table width, reach) agree:
@@ -180,7 +189,11 @@ class ModelRunner:
         if rows > self.max_batch_tokens:
             raise StepError(f"{rows} tokens in one step, at most {self.max_batch_tokens}")
 
-    def _pack(self, entries: Sequence[StepEntry], feed: Optional[torch.Tensor] = None) -> StepView:
+    def _pack(self, entries: Sequence[StepEntry], feed: Optional[torch.Tensor] = None, pad_to: int = 0) -> StepView:
+        """``pad_to``: a decode step is filled up to this many rows with rows of no
+        request (token 0 at position 0 of a one-token sequence that lives in the spare
+        page and the spare state slot), so that steps of a few different sizes cover
+        every number of requests."""
         page = self.page_size
         rcs = [self.cache.get(e.key) for e in entries]
         starts = [rc.num_tokens for rc in rcs]
@@ -189,7 +202,8 @@ class ModelRunner:
         rows, seqs = sum(counts), len(entries)
         wanted = sum(len(e.want) for e in entries)
         width = _pow2_at_least(max(max((len(tab) for tab in rc.tables), default=1) for rc in rcs))
-        lay = self.inputs.layout(rows, seqs, wanted, width)
+        pads = max(0, pad_to - seqs)
+        lay = self.inputs.layout(rows + pads, seqs + pads, wanted + pads, width)
         buf = self.inputs.begin()
         # every field is put together as one list and written with one assignment
         tok, pos, sor, sample, row_start, src = [], [], [], [], [0], []
@@ -203,6 +217,18 @@ class ModelRunner:
             sample.extend(r + int(w) for w in e.want)
             r += n
             row_start.append(r)
+        slots = [rc.slot for rc in rcs]
+        if pads:
+            tok.extend([0] * pads)
+            src.extend([-1] * pads)
+            pos.extend([0] * pads)
+            sor.extend(range(seqs, seqs + pads))
+            sample.extend(range(rows, rows + pads))
+            row_start.extend(range(rows + 1, rows + pads + 1))
+            starts = starts + [0] * pads
+            totals = totals + [1] * pads
+            counts = counts + [1] * pads
+            slots = slots + [self.pad_slot] * pads
         buf[lay["token_ids"]] = tok
         buf[lay["token_from"]] = src
         buf[lay["positions"]] = pos
@@ -210,18 +236,21 @@ class ModelRunner:
         buf[lay["row_start"]] = row_start
         buf[lay["seq_start"]] = starts
         buf[lay["seq_len"]] = totals
-        buf[lay["slots"]] = [rc.slot for rc in rcs]
-        if wanted:
+        buf[lay["slots"]] = slots
+        if wanted + pads:
             buf[lay["sample_rows"]] = sample
+        pad_row = [self.pad_page] + [-1] * (width - 1)
         for g in range(len(self.cache.groups)):
             flat = []
             for rc in rcs:
                 tab = rc.tables[g]
                 flat.extend(tab)
                 flat.extend([-1] * (width - len(tab)))
+            flat.extend(pad_row * pads)
             buf[lay[f"tables{g}"]] = flat
         self.inputs.upload(lay["_end"].stop)
         dev = self.inputs.dev
+        rows, seqs = rows + pads, seqs + pads
         if feed is not None:
             self.env.ops.feed_tokens(dev[lay["token_ids"]], dev[lay["token_from"]], feed, rows)
         groups = []
@@ -236,7 +265,7 @@ class ModelRunner:
             seq_start=dev[lay["seq_start"]], seq_len=dev[lay["seq_len"]],
             slots=dev[lay["slots"]], sample_rows=dev[lay["sample_rows"]],
             h_row_start=row_start, h_seq_start=starts, h_seq_len=totals,
-            h_slots=[rc.slot for rc in rcs], max_rows_per_seq=max(counts),
+            h_slots=slots, max_rows_per_seq=max(counts),
             max_seq_len=max(totals), reach=max(128, 1 << (max(totals) - 1).bit_length()),
             groups=groups)
 
@@ -301,11 +330,12 @@ class ModelRunner:
             self.cache.reserve(e.key, self.cache.get(e.key).num_tokens + len(e.tokens))
         if feed is None and any(e.token_from is not None for e in entries):
             raise StepError("an entry takes its token from the device but no tensor was given")
-        view = self._pack(entries, feed)
         wanted = sum(len(e.want) for e in entries)
-        if self.use_graphs and view.max_rows_per_seq == 1 and wanted == len(entries):
-            logits = self._replay(view, wanted)
+        if self.use_graphs and wanted == len(entries) and all(len(e.tokens) == 1 for e in entries):
+            view = self._pack(entries, feed, pad_to=_decode_bucket(len(entries)))
+            logits = self._replay(view, view.num_rows)[:wanted]
         else:
+            view = self._pack(entries, feed)
             logits = self.forward(view, wanted)
         for e in entries:
             self.cache.advance(e.key, self.cache.get(e.key).num_tokens + len(e.tokens))
