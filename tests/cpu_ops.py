@@ -24,7 +24,7 @@ class CpuOps:
     def embed(self, table, token_ids, num_rows):
         return table[token_ids.long()].to(torch.float32)
 
-    def add_rmsnorm(self, resid, delta, weight, eps, out_dtype, rows=None, num_rows=None):
+    def add_rmsnorm(self, resid, delta, weight, eps, out_dtype, rows=None, num_rows=None, lazy=False):
         if rows is None:
             if delta is not None:
                 resid += delta.to(torch.float32)

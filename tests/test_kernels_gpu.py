@@ -529,6 +529,59 @@ def test_partial_sums_as_residual_delta(ops):
     assert torch.equal(o3, o1[rows.long()])
 
 
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("hidden", [200, 4096])
+def test_products_that_take_the_norm_in(ops, M, hidden):
+    """A decode step's output projection adds into the residual and leaves the next norm's
+    rows with their factor owed; the products that follow apply it.  Against float64
+    mathematics and against the same done with a norm kernel between the products."""
+    from tiny_llm_infer_amd.kernels.ops import NormedRows, PendingProduct
+    from tiny_llm_infer_amd.parts.base import BuildEnv
+    from tiny_llm_infer_amd.parts.linear import GatedMatrix, Matrix
+    env = BuildEnv(dtype=torch.bfloat16, device=torch.device(DEV), ops=ops, max_model_len=64)
+    K, N2, inter, eps = 320, 96, 64, 1e-5
+    bf = torch.bfloat16
+    x = rnd((M, K), bf, 1)
+    wo, wn = rnd((hidden, K), bf, 2, 0.05), rnd((N2, hidden), bf, 3, 0.05)
+    wg, wu = rnd((inter, hidden), bf, 4, 0.05), rnd((inter, hidden), bf, 5, 0.05)
+    nw = 1 + rnd((hidden,), torch.float32, 6, 0.2)
+    resid0 = rnd((M, hidden), torch.float32, 7)
+    Wo, Wn, Wg = Matrix(wo.to(DEV), env), Matrix(wn.to(DEV), env), GatedMatrix(wg.to(DEV), wu.to(DEV), env)
+    # float64
+    h = resid0.double() + x.double() @ wo.double().t()
+    n = nw.double() * h / torch.sqrt((h * h).mean(-1, keepdim=True) + eps)
+    want_z = n @ wn.double().t()
+    g, u = n @ wg.double().t(), n @ wu.double().t()
+    want_act = g / (1 + torch.exp(-g)) * u
+    # a norm kernel between the products
+    ops.separate_norms = True
+    try:
+        ra = resid0.clone().to(DEV)
+        y = ops.linear(x.to(DEV), Wo, deferred=True)
+        assert isinstance(y, torch.Tensor)
+        na = ops.add_rmsnorm(ra, y, nw.to(DEV), eps, bf, lazy=True)
+        za, acta = ops.linear(na, Wn), ops.linear_swiglu(na, Wg)
+    finally:
+        ops.separate_norms = False
+    # the norm taken into the products
+    rb = resid0.clone().to(DEV)
+    p = ops.linear(x.to(DEV), Wo, deferred=True)
+    assert isinstance(p, PendingProduct)
+    nb = ops.add_rmsnorm(rb, p, nw.to(DEV), eps, bf, lazy=True)
+    assert isinstance(nb, NormedRows) and tuple(nb.ssq.shape) == ((hidden + 15) // 16, M)
+    zb, actb = ops.linear(nb, Wn), ops.linear_swiglu(nb, Wg)
+    close(rb, h, torch.float32, "residual", scale=float(h.abs().max()) * 4)     # bfloat16 inputs, float32 sums
+    close(ra, h, bf, "residual through a bfloat16 delta")
+    assert float((nb.ssq.sum(0).double().cpu() - (h * h).sum(-1)).abs().max()) <= 1e-4 * float((h * h).sum(-1).max())
+    for got, want, what in ((zb, want_z, "product of normed rows"), (actb, want_act, "gated product of normed rows"),
+                            (za, want_z, "the same with a norm kernel"), (acta, want_act, "gated, with a norm kernel")):
+        close(got, want, bf, what)
+    # without lazy the product is run as it is
+    rc = resid0.clone().to(DEV)
+    nc = ops.add_rmsnorm(rc, ops.linear(x.to(DEV), Wo, deferred=True), nw.to(DEV), eps, bf)
+    assert torch.equal(nc, na) and torch.equal(rc, ra)
+
+
 # ------------------------------------------------------------------ sampling --
 def test_greedy_takes_the_lowest_index_on_ties(ops):
     logits = torch.zeros(3, 5000)

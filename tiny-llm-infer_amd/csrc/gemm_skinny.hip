@@ -18,6 +18,21 @@
 // A workgroup owns 16*RT output columns; its waves take the 128-wide k steps in
 // turn and their partial sums are added through LDS in wave order, so the
 // result does not depend on the launch.
+//
+// Two variants take the RMS norms of a decoder block into the products around them, so
+// that a decode step needs no norm kernel between its products.  With h the float32
+// residual, w the norm's weights and r = 1/sqrt(mean(h^2) + eps) of a row, the normed row
+// is w*h*r, and (w*h*r) . W^T = r * ((w*h) . W^T): the scalar r can wait until after the
+// product.
+//   FUSE_RESIDUAL (output projections): h += x . W^T in float32, then the product writes
+//       bfloat16(w*h) for the next product and, for every 16 columns, the rows' partial
+//       sums of h^2.
+//   FUSE_RSTD (the products that read normed rows): x is such a bfloat16(w*h); the rows'
+//       partial sums are added in order, and the outputs are scaled by r (before the
+//       SwiGLU of a gated matrix).
+// Sums, r and the residual are float32 (kernels/src/rmsnorm_kernel_cpu.cpp:27-43); the
+// rounding to bfloat16 happens once, as for a separate norm, only before r is applied
+// instead of after (a scalar factor does not change the relative rounding error).
 #include "common.h"
 #include <type_traits>
 
@@ -33,10 +48,25 @@ __device__ __forceinline__ uint4 load16_or_zero(const bf16_t* p, bool ok) {
     return ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
 }
 
-template <int RT, int MT, int WAVES, typename TO, bool TILED = false, bool GATED = false, int DEPTH = 2>
+#define FUSE_NONE 0
+#define FUSE_RSTD 1
+#define FUSE_RESIDUAL 2
+
+struct SkinnyFuse {
+    const float* ssq_in;      // FUSE_RSTD: [parts_in][M] partial sums of squares of the rows of x's source
+    int parts_in;
+    float eps;
+    float* resid;             // FUSE_RESIDUAL: [M][N] float32, updated in place
+    const float* norm_w;      // [N] weights of the norm that follows
+    bf16_t* xw;               // [M][N] bfloat16(norm_w * resid)
+    float* ssq_out;           // [ceil(N/16)][M]
+};
+
+template <int RT, int MT, int WAVES, typename TO, bool TILED = false, bool GATED = false, int DEPTH = 2,
+          int FUSE = FUSE_NONE>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* __restrict__ y,
-                   int M, int N, int K) {
+                   int M, int N, int K, SkinnyFuse fuse) {
     __shared__ float red[WAVES][RT * MT][64][4];
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int r = lane % 16, c = lane / 16;
@@ -128,6 +158,45 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
         }
     };
     prologue(prologue, std::integral_constant<int, 0>{});
+    // (asked for behind the first W fragments, needed only after the last)
+    // FUSE_RSTD: the partial sums of squares are shared out over the waves and lane groups
+    // (part p to wave (p / 4) % WAVES, lane group p % 4), asked for eight at a time without
+    // a branch, and added up over the workgroup only after the main loop
+    float ssq_mine[MT];
+    if (FUSE == FUSE_RSTD) {
+        constexpr int STEP = 4 * WAVES;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const int row = min(m * 16 + r, M - 1);
+            float a = 0.f;
+            for (int p0 = wave * 4 + c; p0 < fuse.parts_in; p0 += 8 * STEP) {
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int p = p0 + e * STEP;
+                    v[e] = fuse.ssq_in[(size_t)min(p, fuse.parts_in - 1) * M + row] * (p < fuse.parts_in ? 1.f : 0.f);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a += v[e];
+            }
+            ssq_mine[m] = quad_rows_sum(a);            // over the four lane groups
+        }
+    }
+    float h_old[4] = {0.f, 0.f, 0.f, 0.f}, nw[4] = {0.f, 0.f, 0.f, 0.f};
+    if (FUSE == FUSE_RESIDUAL) {
+        static_assert(FUSE != FUSE_RESIDUAL || (MT == 1 && RT <= WAVES), "one tile a wave at most");
+        {   // wave t < RT finishes tile t: its residual values and norm weights (the other
+            // waves ask for the same as wave 0, which costs nothing and keeps the loads
+            // free of branches; rows and columns past the end repeat the last)
+            const int n0 = n_base + (wave < RT ? wave : 0) * 16 + c * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int col = min(n0 + e, N - 1);
+                h_old[e] = fuse.resid[(size_t)min(r, M - 1) * N + col];
+                nw[e] = fuse.norm_w[col];
+            }
+        }
+    }
     int i = 0;
     for (; i + 2 * (DEPTH - 1) < mine; i += DEPTH)
         round(round, i, std::integral_constant<int, 0>{}, std::true_type{});
@@ -156,7 +225,21 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
         for (int m = 0; m < MT; ++m)
 #pragma unroll
             for (int i = 0; i < 4; ++i) red[wave][t * MT + m][lane][i] = acc[t][m][i];
+    __shared__ float ssq_red[FUSE == FUSE_RSTD ? WAVES : 1][MT][16];
+    if (FUSE == FUSE_RSTD && c == 0) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) ssq_red[wave][m][r] = ssq_mine[m];
+    }
     __syncthreads();
+    float rstd[MT];
+    if (FUSE == FUSE_RSTD) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            float a = 0.f;
+            for (int wv = 0; wv < WAVES; ++wv) a += ssq_red[wv][m][r];
+            rstd[m] = 1.0f / sqrtf(a / (float)K + fuse.eps);
+        }
+    }
     if (GATED) {
         // row tiles come in pairs (gate rows, up rows of the same 16 outputs): the
         // epilogue writes silu(gate) * up, N/2 columns (kernels/src/swiglu_kernel_cpu.cpp:20-24)
@@ -172,6 +255,13 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
                 }
             const int row = m * 16 + r;
             const int n0 = (blockIdx.x * (RT / 2) + tp) * 16 + c * 4;
+            if (FUSE == FUSE_RSTD) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    g[i] *= rstd[m];
+                    u[i] *= rstd[m];
+                }
+            }
             if (row < M) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
@@ -190,6 +280,25 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
             for (int i = 0; i < 4; ++i) s[i] += red[wv][tile][lane][i];
         const int row = m * 16 + r;
         const int n0 = n_base + t * 16 + c * 4;
+        if (FUSE == FUSE_RESIDUAL) {
+            // (MT == 1 and tile == wave: the values asked for at the start are this tile's)
+            float ssq = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (row < M && n0 + i < N) {
+                    const float h = h_old[i] + s[i];
+                    fuse.resid[(size_t)row * N + n0 + i] = h;
+                    fuse.xw[(size_t)row * N + n0 + i] = f32_to_bf16(nw[i] * h);
+                    ssq += h * h;
+                }
+            ssq = quad_rows_sum(ssq);                  // over the tile's 16 columns
+            if (c == 0 && row < M) fuse.ssq_out[(size_t)(blockIdx.x * RT + t) * M + row] = ssq;
+            continue;
+        }
+        if (FUSE == FUSE_RSTD) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[i] *= rstd[m];
+        }
         if (row < M) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -208,17 +317,17 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, void* y, int M, int N
     const int blocks = (N + 16 * RT - 1) / (16 * RT);
     constexpr int D = (MT == 1 && RT <= 2) ? PIPE_DEPTH : 2;    // deep prefetch where the registers allow
     if (tiled == 2) {       // gated: pairs of row tiles, silu(gate)*up written as bfloat16
-        gemm_skinny_kernel<RT, MT, WAVES, bf16_t, true, true, D><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
+        gemm_skinny_kernel<RT, MT, WAVES, bf16_t, true, true, D><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K, SkinnyFuse{});
     } else if (tiled) {
         if (y_dtype == TLI_BF16)
-            gemm_skinny_kernel<RT, MT, WAVES, bf16_t, true, false, D><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
+            gemm_skinny_kernel<RT, MT, WAVES, bf16_t, true, false, D><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K, SkinnyFuse{});
         else
-            gemm_skinny_kernel<RT, MT, WAVES, float, true, false, D><<<blocks, WAVES * 64, 0, s>>>(x, w, (float*)y, M, N, K);
+            gemm_skinny_kernel<RT, MT, WAVES, float, true, false, D><<<blocks, WAVES * 64, 0, s>>>(x, w, (float*)y, M, N, K, SkinnyFuse{});
     } else {
         if (y_dtype == TLI_BF16)
-            gemm_skinny_kernel<RT, MT, WAVES, bf16_t, false><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K);
+            gemm_skinny_kernel<RT, MT, WAVES, bf16_t, false><<<blocks, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, M, N, K, SkinnyFuse{});
         else
-            gemm_skinny_kernel<RT, MT, WAVES, float, false><<<blocks, WAVES * 64, 0, s>>>(x, w, (float*)y, M, N, K);
+            gemm_skinny_kernel<RT, MT, WAVES, float, false><<<blocks, WAVES * 64, 0, s>>>(x, w, (float*)y, M, N, K, SkinnyFuse{});
     }
     return tli_check_launch("gemm_skinny");
 }
@@ -266,5 +375,51 @@ extern "C" int tli_gemm_skinny_bf16(const void* x, const void* w, void* y, int M
         case 2: return pick_skinny<2>(xp, wp, y, M, N, K, y_dtype, tiled, s, cfg);
         case 3: return pick_skinny<3>(xp, wp, y, M, N, K, y_dtype, tiled, s, cfg);
         default: return pick_skinny<4>(xp, wp, y, M, N, K, y_dtype, tiled, s, cfg);
+    }
+}
+
+template <int RT, int WAVES>
+static int launch_skinny_fused(const bf16_t* x, const bf16_t* w, bf16_t* y, int M, int N, int K, int gated,
+                               const SkinnyFuse& f, hipStream_t s) {
+    const int blocks = (N + 16 * RT - 1) / (16 * RT);
+    if (f.resid)
+        gemm_skinny_kernel<RT, 1, WAVES, bf16_t, true, false, PIPE_DEPTH, FUSE_RESIDUAL><<<blocks, WAVES * 64, 0, s>>>(x, w, y, M, N, K, f);
+    else if (gated)
+        gemm_skinny_kernel<RT, 1, WAVES, bf16_t, true, true, PIPE_DEPTH, FUSE_RSTD><<<blocks, WAVES * 64, 0, s>>>(x, w, y, M, N, K, f);
+    else
+        gemm_skinny_kernel<RT, 1, WAVES, bf16_t, true, false, PIPE_DEPTH, FUSE_RSTD><<<blocks, WAVES * 64, 0, s>>>(x, w, y, M, N, K, f);
+    return tli_check_launch("gemm_skinny (norm taken in)");
+}
+
+// The product with a norm taken in (see the top of this file), for up to 16 rows and W in the
+// decode layout.  Either  resid != null:  resid[M,N] += x . W^T (float32), xw[M,N] =
+// bfloat16(norm_w * resid), ssq_out[ceil(N/16)][M] = partial sums of resid^2 (y is not used);
+// or  ssq_in != null:  y = (x . W^T) / sqrt(sum(ssq_in[parts_in][M]) / K + eps), through the
+// SwiGLU of a gated matrix if `gated` (y then [M, N/2]).
+extern "C" int tli_gemm_skinny_fused_bf16(const void* x, const void* w, void* y, int M, int N, int K, int gated,
+                                          const float* ssq_in, int parts_in, float eps, float* resid,
+                                          const float* norm_w, void* xw, float* ssq_out, int cfg, void* stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16) return tli_fail("gemm_skinny with a norm: %d rows, at most 16", M);
+    if (K <= 0 || K % 8) return tli_fail("gemm_skinny: K = %d must be a positive multiple of 8", K);
+    if ((resid != nullptr) == (ssq_in != nullptr))
+        return tli_fail("gemm_skinny with a norm: give either the residual to add into or the sums of squares of x");
+    if (resid && (gated || !norm_w || !xw || !ssq_out)) return tli_fail("gemm_skinny into the residual: missing arguments");
+    if (ssq_in && (parts_in <= 0 || !y)) return tli_fail("gemm_skinny with sums of squares: missing arguments");
+    if (gated && N % 32) return tli_fail("gemm_skinny: a gated product needs N %% 32 == 0");
+    if (((uintptr_t)x | (uintptr_t)w) & 15) return tli_fail("gemm_skinny: operands must be 16-byte aligned");
+    const SkinnyFuse f{ssq_in, parts_in, eps, resid, norm_w, (bf16_t*)xw, ssq_out};
+    hipStream_t s = (hipStream_t)stream;
+    const bf16_t* xp = (const bf16_t*)x;
+    const bf16_t* wp = (const bf16_t*)w;
+    const long tiles = (N + 15) / 16;
+    if (cfg == 0) cfg = tiles <= 256 ? 18 : (tiles < 1024 ? 28 : 24);
+    if (gated && cfg < 20) cfg = 24;
+    switch (cfg) {
+        case 14: return launch_skinny_fused<1, 4>(xp, wp, (bf16_t*)y, M, N, K, gated, f, s);
+        case 18: return launch_skinny_fused<1, 8>(xp, wp, (bf16_t*)y, M, N, K, gated, f, s);
+        case 24: return launch_skinny_fused<2, 4>(xp, wp, (bf16_t*)y, M, N, K, gated, f, s);
+        case 28: return launch_skinny_fused<2, 8>(xp, wp, (bf16_t*)y, M, N, K, gated, f, s);
+        default: return tli_fail("gemm_skinny: unknown configuration %d", cfg);
     }
 }

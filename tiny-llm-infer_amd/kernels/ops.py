@@ -22,6 +22,29 @@ class KernelError(RuntimeError):
     pass
 
 
+class PendingProduct:
+    """x W^T not run yet: what ``linear(..., deferred=True)`` returns for a decode step's
+    few rows.  ``add_rmsnorm(..., lazy=True)`` runs it with the residual sum and the
+    norm taken into the product; anything else runs it as it is (``resolve``)."""
+
+    def __init__(self, x: torch.Tensor, matrix):
+        self.x, self.matrix = x, matrix
+        self.shape = (x.shape[0], matrix.w.shape[0])
+        self.dtype = x.dtype
+
+
+class NormedRows:
+    """Rows of a norm whose scalar factor is still owed: ``xw`` = bfloat16(weight * h)
+    [rows, n] and ``ssq`` [parts, rows], partial sums of h^2 in float32; the normed rows
+    are xw / sqrt(sum(ssq) / n + eps).  ``linear`` and ``linear_swiglu`` take it as their
+    input and apply the factor to their outputs."""
+
+    def __init__(self, xw: torch.Tensor, ssq: torch.Tensor, eps: float):
+        self.xw, self.ssq, self.eps = xw, ssq, float(eps)
+        self.shape = tuple(xw.shape)
+        self.dtype = xw.dtype
+
+
 def _dtype_code(dtype: torch.dtype) -> int:
     if dtype == torch.float32:
         return F32
@@ -56,6 +79,7 @@ def load_library():
         "tli_attention_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
         "tli_gemm_plain": [P, P, P, I, I, I, I, I, I, P],
         "tli_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, I, P],
+        "tli_gemm_skinny_fused_bf16": [P, P, P, I, I, I, I, P, I, F, P, P, P, P, I, P],
         "tli_gemm_mid_bf16": [P, P, P, P, I, I, I, I, I, I, I, P],
         "tli_gemm_mid_splits": [I, I, I],
         "tli_gemm_mid_reduce": [P, P, I, I, I, I, P],
@@ -109,6 +133,7 @@ class HipOps:
             raise KernelError("no GPU is visible to torch; this engine has no CPU path")
         self.lib = load_library()
         self.force_plain = False     # tests: run the plain attention kernel for bfloat16 too
+        self.separate_norms = False  # tests: decode steps run their norms as kernels of their own
         self.unfused_decode = False  # tests: decode steps through qkv_to_cache and paged_attention too
         self.prefill_direct = 0      # tests: 1 = the prefill attention kernel without LDS staging; 2, 3 = with, 1 or 2 tiles a wave
         self.mid_cfg = 0             # measurements: launch shape and k ranges of the 17..64-row kernel
@@ -167,7 +192,11 @@ class HipOps:
         return out
 
     def resolve(self, y):
-        """The tensor of a product that ``linear`` may have left as partial sums."""
+        """The tensor of a product that ``linear(..., deferred=True)`` left unfinished."""
+        if isinstance(y, PendingProduct):
+            return self.linear(y.x, y.matrix)
+        if isinstance(y, NormedRows):
+            raise KernelError("normed rows that still owe their factor go to linear or linear_swiglu")
         if not isinstance(y, DeferredSum):
             return y
         splits, M, N = y.parts.shape
@@ -176,10 +205,16 @@ class HipOps:
                    _dtype_code(y.dtype), self._stream())
         return out
 
-    def add_rmsnorm(self, resid, delta, weight, eps, out_dtype, rows=None, num_rows=None):
+    def add_rmsnorm(self, resid, delta, weight, eps, out_dtype, rows=None, num_rows=None, lazy=False):
+        """``lazy``: the caller hands the result to ``linear`` or ``linear_swiglu`` only and so
+        also takes ``NormedRows``."""
         total, n = resid.shape
         self._want(resid, "residual", torch.float32)
         self._want(weight, "norm weight", torch.float32, (n,))
+        if isinstance(delta, PendingProduct):
+            if lazy and rows is None and not self.separate_norms:
+                return self._product_into_residual(delta, resid, weight, eps)
+            delta = self.resolve(delta)
         parts = 0
         if isinstance(delta, DeferredSum):
             if delta.dtype != out_dtype or out_dtype != torch.bfloat16:
@@ -223,7 +258,12 @@ class HipOps:
         """y = x W^T.  ``w`` is a [N, K] tensor or a ``Matrix`` (row-major tensor plus
         its decode layout).  ``deferred``: the caller hands the result to ``add_rmsnorm``
         (or to ``resolve``) and so also takes a ``DeferredSum``."""
+        if isinstance(x, NormedRows):
+            return self._linear_normed(x, w, getattr(w, "tiled", None), 0, out_dtype)
         tiled = getattr(w, "tiled", None)
+        if (deferred and tiled is not None and x.dtype == torch.bfloat16 and 0 < x.shape[0] <= 16
+                and out_dtype in (None, torch.bfloat16) and not self.separate_norms):
+            return PendingProduct(x, w)
         w = getattr(w, "w", w)
         M, K = x.shape
         N, K2 = w.shape
@@ -258,6 +298,37 @@ class HipOps:
                    _dtype_code(x.dtype), _dtype_code(w.dtype), _dtype_code(out_dtype), self._stream())
         return y
 
+    def _product_into_residual(self, p: PendingProduct, resid, weight, eps) -> NormedRows:
+        """resid += x W^T, and the rows of the norm that follows, its factor still owed."""
+        x, m = p.x, p.matrix
+        M, K = x.shape
+        N = m.w.shape[0]
+        self._want(x, "linear input", torch.bfloat16, (M, m.w.shape[1]))
+        if tuple(resid.shape) != (M, N):
+            raise KernelError(f"the product gives {(M, N)}, the residual is {tuple(resid.shape)}")
+        xw = torch.empty((M, N), dtype=torch.bfloat16, device=self.device)
+        ssq = torch.empty(((N + 15) // 16, M), dtype=torch.float32, device=self.device)
+        self._call(self.lib.tli_gemm_skinny_fused_bf16, x.data_ptr(), m.tiled.data_ptr(), None, M, N, K, 0,
+                   None, 0, 0.0, resid.data_ptr(), weight.data_ptr(), xw.data_ptr(), ssq.data_ptr(), 0,
+                   self._stream())
+        return NormedRows(xw, ssq, eps)
+
+    def _linear_normed(self, x: NormedRows, m, tiled, gated: int, out_dtype=None):
+        """y = normed rows . W^T with the rows' factor applied to the outputs."""
+        M, K = x.xw.shape
+        if tiled is None:
+            raise KernelError("normed rows that still owe their factor need a matrix in the decode layout")
+        if out_dtype not in (None, torch.bfloat16):
+            raise KernelError("normed rows that still owe their factor give bfloat16 products")
+        rows_out = m.w.shape[0]
+        if m.w.shape[1] != K:
+            raise KernelError(f"linear: input has {K} columns, the matrix {m.w.shape[1]}")
+        N = 2 * m.inter if gated else rows_out
+        y = torch.empty((M, m.inter if gated else N), dtype=torch.bfloat16, device=self.device)
+        self._call(self.lib.tli_gemm_skinny_fused_bf16, x.xw.data_ptr(), tiled.data_ptr(), y.data_ptr(), M, N, K,
+                   gated, x.ssq.data_ptr(), x.ssq.shape[0], x.eps, None, None, None, None, 0, self._stream())
+        return y
+
     def _linear_mid(self, x, tiled, y, M, N, K, gated, deferred=False):
         """17..64 rows: the kernel that shares x through LDS, k cut into ranges when the
         output alone gives too few workgroups.  ``deferred``: the partial sums of the
@@ -287,6 +358,8 @@ class HipOps:
         """silu(x gate^T) * (x up^T) for a ``GatedMatrix``.  Few rows: one pass of
         the weight-streaming kernel over the interleaved layout, the activation in
         its epilogue.  Otherwise the stacked product, then the activation."""
+        if isinstance(x, NormedRows):
+            return self._linear_normed(x, m, getattr(m, "gated", None), 1)
         M, K = x.shape
         gated = getattr(m, "gated", None)
         if gated is not None and 0 < M <= self.SKINNY_ROWS and x.dtype == torch.bfloat16:

@@ -68,6 +68,10 @@ class PagedAttention(Mixer):
     def cache_need(self) -> Optional[CacheNeed]:
         return CacheNeed(self.kv_heads, self.head_dim, self.window)
 
+    @property
+    def takes_normed_rows(self) -> bool:       # x goes to the q/k/v product only
+        return getattr(self.w_qkv, "tiled", None) is not None
+
     def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
         ops = self.env.ops
         qkv = ops.linear(x, self.w_qkv)

@@ -122,6 +122,10 @@ class Norm(Part):
 
 
 class Mixer(Part):
+    # True if ``forward`` hands x to ``ops.linear`` / ``ops.linear_swiglu`` only: the norm
+    # before it may then leave its scalar factor to that product (``lazy`` norms)
+    takes_normed_rows = False
+
     def cache_need(self) -> Optional[CacheNeed]:
         return None
 
@@ -137,6 +141,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    takes_normed_rows = False        # as for a mixer
+
     def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
         """As ``Mixer.forward``."""
         raise NotImplementedError

@@ -32,9 +32,11 @@ class PreNormBlock(Block):
 
     def forward(self, resid: torch.Tensor, pending: Optional[torch.Tensor],
                 step: StepView) -> torch.Tensor:
-        n = self.norm_mixer.forward(resid, pending)
+        # (a part that gives its input to matrix products only lets the norm before it be
+        # taken into those products)
+        n = self.norm_mixer.forward(resid, pending, **({"lazy": True} if self.mixer.takes_normed_rows else {}))
         a = self.mixer.forward(n, step)
-        m = self.norm_ffn.forward(resid, a)
+        m = self.norm_ffn.forward(resid, a, **({"lazy": True} if self.ffn.takes_normed_rows else {}))
         return self.ffn.forward(m, step)
 
 

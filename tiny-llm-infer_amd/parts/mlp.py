@@ -33,6 +33,10 @@ class SwiGLU(FeedForward):
         self.w_gate_up = GatedMatrix(weights[n["gate"]], weights[n["up"]], env)
         self.w_down = as_matrix(weights[n["down"]], env)
 
+    @property
+    def takes_normed_rows(self) -> bool:       # x goes to the gate/up product only
+        return getattr(self.w_gate_up, "gated", None) is not None
+
     def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
         ops = self.env.ops
         return ops.linear(ops.linear_swiglu(x, self.w_gate_up), self.w_down, deferred=True)   # a delta for the next norm

@@ -30,9 +30,11 @@ class RMSNorm(Norm):
         # vectors are held in float32: exact for 16-bit storage, unchanged for 32-bit
         self.weight = weights[self.weight_name].to(torch.float32).contiguous()
 
-    def forward(self, resid, delta, rows=None, num_rows=None):
+    def forward(self, resid, delta, rows=None, num_rows=None, lazy=False):
+        """``lazy``: the rows go to matrix products only, which may then apply the rows'
+        scalar factor themselves (the kernel library decides; see its ``add_rmsnorm``)."""
         return self.env.ops.add_rmsnorm(resid, delta, self.weight, self.eps, self.env.dtype,
-                                        rows=rows, num_rows=num_rows)
+                                        rows=rows, num_rows=num_rows, **({"lazy": True} if lazy else {}))
 
 
 register_part("norm", "rmsnorm", RMSNorm)
