@@ -842,7 +842,7 @@ __device__ __forceinline__ void prefill_lds_block(
 // workgroups to spare each takes block (last - b) and then block b, and all do about
 // the same work.
 template <int NJ, int ND, int CT, int KB>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, (CT == 2 && ND <= 8) ? 2 : 1)
 attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                              const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                              const int* __restrict__ row_start, const int* __restrict__ seq_start,
@@ -1028,9 +1028,9 @@ static int launch_prefill(
                         "of at least 8 (%d), through LDS", head_dim, page_size);
     const RawQkv raw = raw_in ? *raw_in : RawQkv{};
     if (page_size >= 8 && direct != 1) {
-        // through LDS, blocks of 64 keys (32 for large heads).  Two column tiles a wave (which
-        // leaves room for one workgroup a compute unit) when pairs of its row blocks, a long
-        // one with a short one, still fill the chip; else one tile a wave, two workgroups a unit.
+        // through LDS, blocks of 64 keys (32 for large heads).  Two column tiles a wave when
+        // that still gives two workgroups for every compute unit (long row blocks are then
+        // placed beside short ones); else one tile a wave.
         const long blocks2 = (rows + 8 * rq - 1) / (8 * rq) + num_seqs;
         bool two = head_dim <= 128 && blocks2 * kv_heads * head_tiles >= 512;
         if (direct == 2) two = false;
@@ -1038,7 +1038,7 @@ static int launch_prefill(
         const int rows_per_block = 4 * rq * (two ? 2 : 1);
         const long blocks = (rows + rows_per_block - 1) / rows_per_block + num_seqs;   // upper bound
         if (blocks > 2147483647L) return tli_fail("attention_prefill: too many rows");
-        int pair = two ? 1 : (blocks * kv_heads * head_tiles >= 1024 ? 1 : 2);
+        int pair = two ? 2 : (blocks * kv_heads * head_tiles >= 1024 ? 1 : 2);
         if (direct >= 4) pair = direct - 4;               // measurements: 4, 5, 6 force the pairing mode
         dim3 grid((unsigned)(pair == 1 ? (blocks + 1) / 2 : blocks), kv_heads * head_tiles);
         const int kb = head_dim <= 128 ? 64 : 32;
