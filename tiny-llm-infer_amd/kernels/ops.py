@@ -124,6 +124,7 @@ class HipOps:
     SKINNY_ROWS = 64
     MID_ROWS_FROM = 17           # from this many rows the x-sharing kernel multiplies
     DECODE_WORKGROUPS = 512      # aim of the decode attention's key splitting
+    DECODE_SPLIT_KEYS = 512      # a split walks at least this many keys
 
     def __init__(self, device):
         self.device = torch.device(device)
@@ -525,7 +526,7 @@ class HipOps:
         reach = step.reach if not window else min(step.reach, (window + 31) // 32 * 32 + 32)
         groups = T * kv_heads * ((heads // kv_heads + 15) // 16)
         # a split costs a merge pass: only worth it when a workgroup would walk many keys
-        splits = max(1, min((self.DECODE_WORKGROUPS + groups - 1) // groups, reach // 512, 64))
+        splits = max(1, min((self.DECODE_WORKGROUPS + groups - 1) // groups, reach // self.DECODE_SPLIT_KEYS, 64))
         # (a split's block table entries are kept in LDS: at most 2046 pages a split)
         splits = max(splits, -(-reach // (2046 * g.page_size // 128 * 128)))
         per_split = ((reach + splits - 1) // splits + 127) // 128 * 128
