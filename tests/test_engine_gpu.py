@@ -132,6 +132,28 @@ def test_command_line_bench(model_folders):
     assert out[-1].startswith("aggregate_runs=2")
 
 
+def test_command_line_plain_kernels_and_prefill_only(model_folders):
+    """--kernels plain runs bfloat16 through the plain kernels: the first tokens are those
+    of the tuned kernels; --bench --prefill-only counts prompt tokens."""
+    folder = model_folders["D"]
+    prompt = ",".join(map(str, random_prompt(320, 21, 4)))
+    outs = []
+    for kernels in ("tuned", "plain"):
+        cmd = [sys.executable, os.path.join(ROOT, "bin", "model_main"), "--infer", "--model", folder,
+               "--dtype", "bfloat16", "--max-new-tokens", "4", "--max-seq-len", "64", "--num-kv-blocks", "16",
+               "--page-size", "8", "--ignore-eos", "--kernels", kernels, "--prompt-ids", prompt]
+        proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        outs.append(list(map(int, proc.stdout.split())))
+    assert len(outs[0]) == 4 and outs[0][0] == outs[1][0]
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "model_main"), "--bench", "--model", folder, "--prefill-only",
+           "--num-seqs", "3", "--min-input-len", "20", "--max-input-len", "40", "--warmup", "0", "--repeats", "1",
+           "--max-seq-len", "64"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.startswith("run=0 prompt_tokens=") and "median_prompt_tokens_per_second=" in proc.stdout
+
+
 def test_the_library_is_needed():
     from tiny_llm_infer_amd.kernels.ops import HipOps, KernelError
     with pytest.raises(KernelError):

@@ -137,6 +137,17 @@ def test_trace_run_program(model_folders, tmp_path):
                 outputs[s["step"]] = np.fromfile(path, dtype="<f4").reshape(-1, vocab)
         got = collect(steps, outputs)
         _check(got, want, dtype, f"trace_run {dtype}")
+    # `model_main --replay` is the same program; with --kernels plain bfloat16 goes through the plain kernels
+    out_dir = tmp_path / "plain"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "model_main"), "--replay", "--model", model_folders[name],
+         "--dtype", "bfloat16", "--out", str(out_dir), "--max-tokens", "192", "--kernels", "plain"],
+        input="".join(json.dumps(s) + "\n" for s in steps), text=True,
+        stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    outputs = {s["step"]: np.fromfile(out_dir / f"{s['step']}.f32", dtype="<f4").reshape(-1, vocab)
+               for s in steps if sum(len(e["want"]) for e in s["entries"])}
+    _check(collect(steps, outputs), want, "bfloat16", "model_main --replay --kernels plain")
 
 
 def test_real_layer_sizes(tmp_path):

@@ -36,6 +36,8 @@ def _common(ap: argparse.ArgumentParser) -> None:
                     help="with --config: draw seeded random weights instead of reading a checkpoint")
     ap.add_argument("--config", help="a config.json, for --random-weights")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--kernels", default="tuned", choices=["tuned", "plain"],
+                    help="plain: the simple twins of the tuned kernels (bfloat16 too)")
 
 
 def _device(name: str) -> str:
@@ -63,10 +65,13 @@ def _load(args, max_seq_len: int):
             data = json.load(fh)
         arch = architecture_of(data, args.config)
         cfg = arch.read_config(data, args.config)
-        return random_model(arch.name, cfg, args.seed, args.dtype, device, max_seq_len)
+        model = random_model(arch.name, cfg, args.seed, args.dtype, device, max_seq_len)
+        _kernels(model, args.kernels)
+        return model
     if not args.model:
         raise SystemExit2("--model is required (or --config with --random-weights)")
     model, _ = load_model(args.model, args.dtype, device, max_seq_len)
+    _kernels(model, args.kernels)
     return model
 
 
@@ -156,7 +161,11 @@ def run_benchmark(argv: List[str]) -> int:
     ap.add_argument("--repeats", type=int, default=3)
     ap.add_argument("--max-token-id", type=int, default=10000)
     ap.add_argument("--manifest-prefix", default=None)
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="one new token a request: measures prompt tokens a second")
     args = ap.parse_args(argv)
+    if args.prefill_only:
+        args.min_output_len = args.max_output_len = 1
     max_seq_len = args.max_seq_len or 256
     if args.max_input_len + args.max_output_len > max_seq_len + 1:
         raise SystemExit2("max-input-len + max-output-len must be at most max-seq-len + 1")
@@ -191,6 +200,8 @@ def run_benchmark(argv: List[str]) -> int:
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         out_tokens = sum(len(r.token_ids) for r in results)
+        if args.prefill_only:
+            out_tokens = sum(len(p) for p, _ in reqs)          # the tokens that were run
         if args.manifest_prefix and not warm:
             with open(f"{args.manifest_prefix}.run{run - args.warmup}.json", "w") as fh:
                 json.dump({"seed": seed, "requests": [
@@ -202,12 +213,14 @@ def run_benchmark(argv: List[str]) -> int:
         rates.append(out_tokens / dt)
         total_tokens += out_tokens
         total_time += dt
-        print(f"run={run - args.warmup} output_tokens={out_tokens} elapsed_seconds={dt:.4f} "
-              f"output_tokens_per_second={out_tokens / dt:.2f}")
+        what = "prompt" if args.prefill_only else "output"
+        print(f"run={run - args.warmup} {what}_tokens={out_tokens} elapsed_seconds={dt:.4f} "
+              f"{what}_tokens_per_second={out_tokens / dt:.2f}")
     if rates:
-        print(f"aggregate_runs={args.repeats} output_tokens={total_tokens} elapsed_seconds={total_time:.4f} "
-              f"output_tokens_per_second={total_tokens / total_time:.2f} "
-              f"median_output_tokens_per_second={statistics.median(rates):.2f}")
+        what = "prompt" if args.prefill_only else "output"
+        print(f"aggregate_runs={args.repeats} {what}_tokens={total_tokens} elapsed_seconds={total_time:.4f} "
+              f"{what}_tokens_per_second={total_tokens / total_time:.2f} "
+              f"median_{what}_tokens_per_second={statistics.median(rates):.2f}")
     st = engine.stats()
     print(f"engine_steps={st['steps']} preemptions={st['preemptions']} "
           f"pages_free={min(st['pages_free'])}/{st['pages']} prefix_pages_reused={st['prefix_pages_reused']}",
@@ -215,9 +228,62 @@ def run_benchmark(argv: List[str]) -> int:
     return 0
 
 
-USAGE = """usage: model_main --infer [options] | --bench [options]
+REPLAY_HELP = """Trace replay: feed given token ids through a model step by step and write
+the logits at the wanted places.  Nothing is sampled.
+
+    trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
+
+Steps are read from standard input, one JSON object a line:
+    {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
+For a step in which something is wanted, OUT/<step>.f32 holds the logits at the
+wanted places as little-endian float32 [wanted, vocab].  After every step a
+line "done <step>" is printed."""
+
+
+def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
+    """``bin/trace_run`` and ``model_main --replay``: the model, step function, cache and
+    kernels that generation uses, driven by a trace instead of a scheduler."""
+    ap = argparse.ArgumentParser(prog=prog, description=REPLAY_HELP,
+                                 formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
+    ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
+    ap.add_argument("--max-tokens", type=int, required=True,
+                    help="most tokens live requests hold at any time (each rounded up to 64)")
+    ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--max-live", type=int, default=4, help="most requests live at a time")
+    ap.add_argument("--max-step-tokens", type=int, default=8192, help="most tokens in one step")
+    ap.add_argument("--device", default="cuda:0")
+    ap.add_argument("--kernels", default="tuned", choices=["tuned", "plain"],
+                    help="plain: the simple twins of the tuned kernels (bfloat16 too)")
+    args = ap.parse_args(argv)
+    if 64 % args.page_size:
+        ap.error("--page-size must divide 64")
+    print("[trace_run] loading the kernel library (compiled at the first call)", file=sys.stderr, flush=True)
+    from .engine.loading import load_model
+    from .engine.replay import Replayer
+    from .engine.runner import ModelRunner
+    model, cfg = load_model(args.model, args.dtype, _device(args.device))
+    _kernels(model, args.kernels)
+    pages = max(1, (args.max_tokens + args.page_size - 1) // args.page_size)
+    runner = ModelRunner(model, model.env, page_size=args.page_size, num_pages=pages,
+                         max_requests=args.max_live, max_batch_tokens=args.max_step_tokens)
+    print(f"[trace_run] ready: {type(cfg).__name__}, {args.dtype}, {pages} pages of {args.page_size}",
+          file=sys.stderr, flush=True)
+    Replayer(runner, args.out).run_stream(sys.stdin, ack=sys.stdout)
+    return 0
+
+
+def _kernels(model, which: str) -> None:
+    """--kernels plain: every product, attention and norm through the plain kernels."""
+    if which == "plain":
+        model.env.ops.use_plain_kernels()
+
+
+USAGE = """usage: model_main --infer [options] | --bench [options] | --replay [options]
   --infer   generate for --prompt-ids (repeatable) and print completion token ids
   --bench   measure output tokens a second over synthetic requests
+  --replay  feed a trace of token ids from standard input, write logits (as bin/trace_run)
   add --help after the mode for its options"""
 
 
@@ -230,6 +296,9 @@ def main(argv=None) -> int:
         if "--bench" in argv:
             argv.remove("--bench")
             return run_benchmark(argv)
+        if "--replay" in argv:
+            argv.remove("--replay")
+            return run_replay(argv)
         print(USAGE, file=sys.stderr)
         return 2
     except SystemExit2 as exc:

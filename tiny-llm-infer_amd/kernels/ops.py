@@ -134,12 +134,18 @@ class HipOps:
             raise KernelError("no GPU is visible to torch; this engine has no CPU path")
         self.lib = load_library()
         self.force_plain = False     # tests: run the plain attention kernel for bfloat16 too
+        self.plain_products = False  # every matrix product through the plain kernel
         self.separate_norms = False  # tests: decode steps run their norms as kernels of their own
         self.unfused_decode = False  # tests: decode steps through qkv_to_cache and paged_attention too
         self.prefill_direct = 0      # tests: 1 = the prefill attention kernel without LDS staging; 2, 3 = with, 1 or 2 tiles a wave
         self.mid_cfg = 0             # measurements: launch shape and k ranges of the 17..64-row kernel
         self.mid_splits = 0
         self.skinny_cfg = 0          # measurements: force a launch shape of the weight-streaming kernel
+
+    def use_plain_kernels(self) -> None:
+        """Every product, attention and norm through the plain kernels, bfloat16 too
+        (what the float32 path runs): to tell a fault of a tuned kernel from one elsewhere."""
+        self.force_plain = self.plain_products = self.separate_norms = self.unfused_decode = True
 
     # ---- helpers ----------------------------------------------------------
     def _stream(self):
@@ -261,6 +267,8 @@ class HipOps:
         (or to ``resolve``) and so also takes a ``DeferredSum``."""
         if isinstance(x, NormedRows):
             return self._linear_normed(x, w, getattr(w, "tiled", None), 0, out_dtype)
+        if self.plain_products:
+            return self.linear_plain(x, getattr(w, "w", w), out_dtype)
         tiled = getattr(w, "tiled", None)
         if (deferred and tiled is not None and x.dtype == torch.bfloat16 and 0 < x.shape[0] <= 16
                 and out_dtype in (None, torch.bfloat16) and not self.separate_norms):
@@ -362,7 +370,7 @@ class HipOps:
         if isinstance(x, NormedRows):
             return self._linear_normed(x, m, getattr(m, "gated", None), 1)
         M, K = x.shape
-        gated = getattr(m, "gated", None)
+        gated = getattr(m, "gated", None) if not self.plain_products else None
         if gated is not None and 0 < M <= self.SKINNY_ROWS and x.dtype == torch.bfloat16:
             self._want(x, "linear input", torch.bfloat16, (M, m.w.shape[1]))
             y = torch.empty((M, m.inter), dtype=x.dtype, device=self.device)
