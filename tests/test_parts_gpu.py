@@ -234,3 +234,177 @@ def test_toy_mixer_with_state_of_its_own(tmp_path):
         for k in reqs:
             assert np.abs(got[k] - want[k]).max() <= 2e-5 * max(1.0, np.abs(want[k]).max())
         assert runner.cache.free_slots() == 4
+
+
+# ------------------------------------------------- toy routing, toy rotation ---
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routed_feed_forward_and_another_rotation(tmp_path, dtype):
+    """Defined here and registered without a change to the framework: a feed-forward
+    that routes every row to experts, and a rotary encoding with its own angles
+    (positions scaled, only a part of the head rotated).  The toy architecture puts them
+    beside the framework's attention and SwiGLU, chooses parts layer by layer, runs block
+    0 twice (each run with a cache layer of its own) and lets the second run of block 1
+    read the keys and values that its first run wrote.  All cuts against a plain version
+    written here."""
+    import numpy as np
+
+    from helpers import collect, trace_mixed, trace_portions, trace_prefill_then_decode, trace_whole
+    from tiny_llm_infer_amd import register_architecture
+    from tiny_llm_infer_amd.config import BlockSpec, JsonReader, LayerCall, ModelSpec, PartSpec
+    from tiny_llm_infer_amd.engine.loading import load_model, write_random_model
+    from tiny_llm_infer_amd.engine.replay import Replayer
+    from tiny_llm_infer_amd.engine.runner import ModelRunner
+    from tiny_llm_infer_amd.parts import FeedForward, PositionEncoding, register_part
+    from tiny_llm_infer_amd.weights import TensorDecl
+
+    def toy_angles(rd, base, scale, n):
+        i = np.arange(rd // 2, dtype=np.float64)
+        return (np.arange(n, dtype=np.float64) * scale)[:, None] * (base ** (-i / (rd // 2)))[None, :]
+
+    class ScaledRotation(PositionEncoding):
+        """angle[p, i] = scale * p * base^(-i / (rd/2)); pairs (i, i + rd/2) of the first rd dims."""
+        def load(self, weights, env):
+            super().load(weights, env)
+            p = self.spec.params
+            a = toy_angles(p["rotary_dim"], p["base"], p["scale"], min(p["max_positions"], env.max_model_len))
+            self.cos = torch.from_numpy(np.cos(a).astype(np.float32)).to(env.device)
+            self.sin = torch.from_numpy(np.sin(a).astype(np.float32)).to(env.device)
+
+        def rotary(self):
+            return self.cos, self.sin, self.spec.params["rotary_dim"]
+
+    class RoutedExperts(FeedForward):
+        """Router logits x Wr^T and their softmax in float32; the top_k experts of a row, each
+        W2_e silu(W1_e x), weighted by their probabilities (not renormalised)."""
+        def __init__(self, spec):
+            super().__init__(spec)
+            p = spec.params
+            self.n, self.inter, self.experts, self.top_k = p["size"], p["inter"], p["experts"], p["top_k"]
+
+        def tensors(self):
+            nm = self.spec.names
+            out = [TensorDecl(nm["router"], (self.experts, self.n))]
+            for e in range(self.experts):
+                out += [TensorDecl(f"{nm['experts']}.{e}.w1", (self.inter, self.n)),
+                        TensorDecl(f"{nm['experts']}.{e}.w2", (self.n, self.inter))]
+            return out
+
+        def load(self, weights, env):
+            super().load(weights, env)
+            nm = self.spec.names
+            self.router = weights[nm["router"]].float()
+            self.w1 = [weights[f"{nm['experts']}.{e}.w1"].to(env.dtype).contiguous() for e in range(self.experts)]
+            self.w2 = [weights[f"{nm['experts']}.{e}.w2"].to(env.dtype).contiguous() for e in range(self.experts)]
+
+        def forward(self, x, step):
+            ops = self.env.ops
+            prob = torch.softmax(x.float() @ self.router.t(), dim=-1)
+            top = torch.topk(prob, self.top_k, dim=-1).indices
+            out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+            for e in range(self.experts):
+                rows = (top == e).any(dim=-1).nonzero().flatten()
+                if rows.numel() == 0:
+                    continue
+                h = ops.linear(x[rows].contiguous(), self.w1[e]).float()           # the framework's products
+                y = ops.linear((h * torch.sigmoid(h)).to(x.dtype), self.w2[e]).float()
+                out[rows] += prob[rows, e:e + 1] * y
+            return out.to(x.dtype)
+
+    register_part("position", "toy_scaled_rotation", ScaledRotation, replace=True)
+    register_part("ffn", "toy_routed_experts", RoutedExperts, replace=True)
+
+    size, heads, kv, hd, inter, vocab, experts = 128, 4, 2, 64, 96, 211, 3
+    top_k = 1 if dtype == "float32" else experts          # in bfloat16 a near tie of the router could go either way
+    rot = [dict(rotary_dim=64, base=500.0, scale=0.5), dict(rotary_dim=32, base=10000.0, scale=1.0)]
+    windows = [None, 21]
+
+    class ToyConfig:
+        def __init__(self, d):
+            JsonReader(d).integer("top_k")
+            self.d = d
+
+        def to_dict(self):
+            return self.d
+
+    def toy_spec(c):
+        rms = lambda n, name: PartSpec("rmsnorm", {"size": n, "eps": 1e-5}, {"weight": name})
+
+        def attention(i):
+            return PartSpec("paged_attention",
+                            {"hidden_size": size, "num_heads": heads, "num_kv_heads": kv, "head_dim": hd,
+                             "scale": hd ** -0.5, "window": windows[i]},
+                            {k: f"l{i}.{k}" for k in "qkvo"},
+                            {"position": PartSpec("toy_scaled_rotation", dict(rot[i], max_positions=512)),
+                             "q_norm": rms(hd, f"l{i}.qn"), "k_norm": rms(hd, f"l{i}.kn")})
+        ffn0 = PartSpec("toy_routed_experts", {"size": size, "inter": inter, "experts": experts,
+                                               "top_k": c.d["top_k"]}, {"router": "l0.router", "experts": "l0.expert"})
+        ffn1 = PartSpec("swiglu", {"hidden_size": size, "intermediate_size": inter},
+                        {"gate": "l1.g", "up": "l1.u", "down": "l1.d"})
+        blocks = tuple(BlockSpec("prenorm", attention(i), ffn, {"mixer": rms(size, f"l{i}.n1"), "ffn": rms(size, f"l{i}.n2")})
+                       for i, ffn in enumerate((ffn0, ffn1)))
+        # block 0 with cache layer 0, block 1 with cache layer 1, block 0 again with cache layer 2,
+        # block 1 again reading cache layer 1
+        schedule = (LayerCall(0, 0), LayerCall(1, 1), LayerCall(0, 2), LayerCall(1, 1, False))
+        return ModelSpec("ToyMixLM", size, vocab, 512,
+                         PartSpec("token_embedding", {"vocab_size": vocab, "hidden_size": size}, {"weight": "emb"}),
+                         blocks, schedule, rms(size, "norm"),
+                         PartSpec("linear_head", {"vocab_size": vocab, "hidden_size": size, "tied": False},
+                                  {"weight": "head"}))
+
+    register_architecture("ToyMixLM", lambda d, origin: ToyConfig(d), toy_spec, replace=True)
+    cfg = {"architectures": ["ToyMixLM"], "top_k": top_k}
+    folder = write_random_model(str(tmp_path / "toymix"), "ToyMixLM", ToyConfig(cfg), seed=9)
+    w = {k: v for k, v in P.read_safetensors(str(tmp_path / "toymix" / "model.safetensors")).items()}
+
+    # ---- the plain version, whole sequences, float64
+    def rotate(x, i, T):
+        rd = rot[i]["rotary_dim"]
+        a = torch.from_numpy(toy_angles(rd, rot[i]["base"], rot[i]["scale"], T))
+        cos, sin = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
+        first, second, rest = x[..., :rd // 2], x[..., rd // 2:rd], x[..., rd:]
+        return torch.cat([first * cos - second * sin, first * sin + second * cos, rest], -1)
+
+    def plain(ids):
+        T = len(ids)
+        h = w["emb"][torch.tensor(ids)]
+        kept = {}
+        for call, (i, reads_old) in enumerate(((0, False), (1, False), (0, False), (1, True))):
+            n = P.rmsnorm(h, w[f"l{i}.n1"], 1e-5)
+            q = P.rmsnorm(P.linear(n, w[f"l{i}.q"]).reshape(T, heads, hd), w[f"l{i}.qn"], 1e-5)
+            q = rotate(q, i, T)
+            if reads_old:
+                k, v = kept[i]
+            else:
+                k = rotate(P.rmsnorm(P.linear(n, w[f"l{i}.k"]).reshape(T, kv, hd), w[f"l{i}.kn"], 1e-5), i, T)
+                v = P.linear(n, w[f"l{i}.v"]).reshape(T, kv, hd)
+                kept[i] = (k, v)
+            o = P.causal_attention(q, k, v, hd ** -0.5, windows[i])
+            r = h + P.linear(o.reshape(T, heads * hd), w[f"l{i}.o"])
+            m = P.rmsnorm(r, w[f"l{i}.n2"], 1e-5)
+            if i == 0:
+                prob = torch.softmax(m @ w["l0.router"].t(), -1)
+                top = torch.topk(prob, top_k, -1).indices
+                y = torch.zeros_like(m)
+                for e in range(experts):
+                    a = P.linear(m, w[f"l0.expert.{e}.w1"])
+                    ye = P.linear(a / (1 + torch.exp(-a)), w[f"l0.expert.{e}.w2"])
+                    y += torch.where((top == e).any(-1, keepdim=True), prob[:, e:e + 1] * ye, torch.zeros_like(ye))
+                h = r + y
+            else:
+                h = r + P.linear(P.swiglu(P.linear(m, w["l1.g"]), P.linear(m, w["l1.u"])), w["l1.d"])
+        return P.linear(P.rmsnorm(h, w["norm"], 1e-5), w["head"]).numpy()
+
+    rng = np.random.default_rng(4)
+    reqs = {f"m{i}": rng.integers(0, vocab, n).tolist() for i, n in enumerate([37, 58, 12, 45])}
+    want = {k: plain(v) for k, v in reqs.items()}
+    model, _ = load_model(folder, dtype, DEV)
+    assert len(model.cache_needs()) == 3                      # three cache layers for four runs of two blocks
+    bound = 2e-5 if dtype == "float32" else 4e-2
+    for steps in (trace_whole(reqs), trace_prefill_then_decode(reqs), trace_portions(reqs, 7),
+                  trace_mixed(reqs, 192, seed=8)):
+        runner = ModelRunner(model, model.env, page_size=8, num_pages=24, max_requests=4, max_batch_tokens=256)
+        rp = Replayer(runner)
+        got = collect(steps, {s["step"]: rp.run_step(s) for s in steps})
+        for k in reqs:
+            assert np.abs(got[k] - want[k]).max() <= bound * max(1.0, np.abs(want[k]).max()), (dtype, k)
+        runner.cache.check()
