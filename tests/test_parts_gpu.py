@@ -55,6 +55,35 @@ def test_rope_part_tables(envs, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tied", [True, False])
+def test_embedding_and_head_parts(envs, dtype, tied):
+    """Rows of the table become the float32 residual; the head gives float32 logits
+    from its own matrix, or from the embedding's when the model ties them."""
+    from tiny_llm_infer_amd.config import PartSpec
+    from tiny_llm_infer_amd.parts import build_part
+    vocab, hidden = 301, 80
+    emb = build_part("embedding", PartSpec("token_embedding", {"vocab_size": vocab, "hidden_size": hidden},
+                                           {"weight": "emb"}))
+    head = build_part("head", PartSpec("linear_head", {"vocab_size": vocab, "hidden_size": hidden, "tied": tied},
+                                       {"weight": "emb" if tied else "head"}))
+    decls = emb.tensors() + ([] if tied else head.tensors())
+    w = _weights(decls, dtype, seed=8)
+    emb.load(w, envs[dtype])
+    head.load(w, envs[dtype], share_with=emb if tied else None)
+    ids = torch.tensor([300, 0, 17, 17, 42], dtype=torch.int32)
+    resid = emb.forward(ids.to(DEV), 5)
+    assert resid.dtype == torch.float32
+    assert torch.equal(resid.cpu(), w["emb"].cpu().float()[ids.long()])
+    x = rnd((3, hidden), dtype, 9)
+    logits = head.forward(x.to(DEV))
+    assert logits.dtype == torch.float32 and tuple(logits.shape) == (3, vocab)
+    matrix = w["emb" if tied else "head"].cpu().double()
+    close(logits, P.linear(x.double(), matrix), torch.float32 if dtype == torch.float32 else dtype, "head")
+    if tied:
+        assert head.weight.w.data_ptr() == emb.table.data_ptr()       # one copy of the matrix
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_swiglu_part(envs, dtype):
     from tiny_llm_infer_amd.config import PartSpec
     from tiny_llm_infer_amd.parts import build_part
