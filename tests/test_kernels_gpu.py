@@ -479,6 +479,28 @@ def test_attention_from_raw_projections(ops, case):
     close(out2, want, dtype, "attention through two kernels")
 
 
+@pytest.mark.parametrize("hd,counts", [(128, [1, 1]), (128, [20, 1]), (48, [5, 1])])
+def test_values_enter_the_cache_finite(ops, hd, counts):
+    """Infinities and NaNs among the values become 0 on their way into the cache (every
+    kernel that writes values), and the attention output of the other rows stays finite."""
+    heads, kv_heads, page = 4, 2, 16
+    seq_lens = [40, 23]
+    dtype = torch.bfloat16
+    step, tables, pos, seq = make_step(seq_lens, counts, page, 8, 5, kv_heads, hd, dtype)
+    fill_cache(step, tables, seq_lens, kv_heads, hd, dtype, 70)
+    T = len(pos)
+    qd, kd = heads * hd, kv_heads * hd
+    qkv = rnd((T, qd + 2 * kd), dtype, 71)
+    qkv[0, qd + kd + 3] = float("inf")
+    qkv[T - 1, qd + kd + hd + 5] = float("nan")
+    out = ops.qkv_attention(qkv.to(DEV), step, step.cache, heads, kv_heads, hd, None, None, None, hd ** -0.5, None)
+    assert bool(torch.isfinite(step.cache.v).all())
+    p0, p1 = int(tables[seq[0], pos[0] // page]), int(tables[seq[T - 1], pos[T - 1] // page])
+    assert float(step.cache.v[p0, 0, 3, pos[0] % page]) == 0.0
+    assert float(step.cache.v[p1, 1, 5, pos[T - 1] % page]) == 0.0
+    assert bool(torch.isfinite(out).all())
+
+
 def test_rotation_pairs_halves_not_neighbours(ops):
     """A head with only element i set: after the rotation at a position whose
     angle for pair i is 90 degrees, the value has moved to element i + d/2."""

@@ -454,7 +454,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
                 } else if (wave == 1) {
                     const bf16_t* src = raw_row + (size_t)(heads + kv_heads + kv_head) * head_dim;
                     bf16_t* dst = v_cache + ((size_t)page * kv_heads + kv_head) * head_dim * page_size + slot;
-                    for (int d = lane; d < head_dim; d += 64) dst[(size_t)d * page_size] = src[d];
+                    for (int d = lane; d < head_dim; d += 64) dst[(size_t)d * page_size] = cache_value(src[d]);
                 }
             }
         }

@@ -39,6 +39,12 @@ __device__ __forceinline__ float to_f32(bf16_t v) { return bf16_to_f32(v); }
 __device__ __forceinline__ void from_f32(float* p, float v) { *p = v; }
 __device__ __forceinline__ void from_f32(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 
+// A value on its way into the cache: infinities and NaNs become 0.  The MFMA attention
+// kernels multiply values of keys that a row does not see by a weight of exactly 0, which
+// only gives 0 for finite values; a page is used again by other requests.
+__device__ __forceinline__ bf16_t cache_value(bf16_t v) { return (v & 0x7F80u) == 0x7F80u ? (bf16_t)0 : v; }
+__device__ __forceinline__ float cache_value(float v) { return (__float_as_uint(v) & 0x7F800000u) == 0x7F800000u ? 0.f : v; }
+
 // Makes LDS writes of this wavefront's lanes visible to its other lanes.
 __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -60,7 +60,7 @@ __global__ void qkv_to_cache_kernel(
         const int g = h - heads - kv_heads;
         const T* vsrc = src_row + q_dim + kv_dim + (size_t)g * head_dim;
         for (int d = lane; d < head_dim; d += TLI_WAVE)
-            v_cache[v_base + ((size_t)g * head_dim + d) * page_size] = vsrc[d];
+            v_cache[v_base + ((size_t)g * head_dim + d) * page_size] = cache_value(vsrc[d]);
         return;
     }
     {
@@ -151,7 +151,7 @@ qkv_to_cache_wide_kernel(
         const int g = h - heads - kv_heads;
         bf16_t* dst = v_cache + ((size_t)page * kv_heads + g) * HD * page_size + (pos % page_size);
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) dst[(size_t)(lane * EPL + e) * page_size] = src[e];
+        for (int e = 0; e < EPL; ++e) dst[(size_t)(lane * EPL + e) * page_size] = cache_value(src[e]);
         return;
     }
     const float* nw = is_q ? q_norm_w : k_norm_w;
@@ -217,7 +217,7 @@ __global__ void values_to_cache_kernel(
     for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
         bf16_t vals[G];
 #pragma unroll
-        for (int j = 0; j < G; ++j) vals[j] = j < n ? src[(size_t)j * stride + d] : (bf16_t)0;
+        for (int j = 0; j < G; ++j) vals[j] = j < n ? cache_value(src[(size_t)j * stride + d]) : (bf16_t)0;
         bf16_t* dst = v_cache + (((size_t)page * kv_heads + kvh) * head_dim + d) * page_size + slot0;
         if (n == G) {               // a whole group: its slots start at a multiple of G
             uint32_t w[G / 2];
