@@ -80,13 +80,31 @@ __device__ __forceinline__ void tile_load_q(Tile<NJ, ND>& t, const bf16_t* q_hea
     }
 }
 
+// The base of a column's exponentials (the value that exp2 subtracts; in units of log2)
+// follows the column's maximum lazily: it stays as long as no column of the wave has a
+// maximum more than 2^LAZY_BITS above its base, which bounds the weights by 2^LAZY_BITS
+// instead of 1 (harmless in float32 sums and in bfloat16 weights) and saves most of the
+// rescaling of the accumulators.  m: the base so far (-inf: nothing seen), m_now: this
+// block's maximum.  Returns the factor that sums under the old base take under the new
+// one (1 if the base stayed) and updates m.
+#define LAZY_BITS 8.0f
+__device__ __forceinline__ float tile_new_base(float& m, float m_now) {
+    const float m_new = fmaxf(m, m_now);
+    // (-inf) - (-inf) is NaN and compares false: a column that has seen nothing stays
+    if (__builtin_amdgcn_ballot_w64(m_new - m > LAZY_BITS) == 0) return 1.0f;
+    const float base = (m_new == -INFINITY) ? 0.f : m_new;
+    const float corr = __builtin_amdgcn_exp2f(m - base);         // exp2(-inf) = 0 the first time
+    m = m_new;
+    return corr;
+}
+
 // Scores, softmax update and output accumulation of one column tile for 32 keys
 // whose fragments are given.  Row 4c+i of score tile u (and k-slot 4u+i of lane
 // group c in the output MFMA) is the key  key_c0 + u*u_stride + i.
-// The running maximum is kept in units of log2: scores are multiplied by
-// scale*log2(e) and exponentials are exp2 (one v_exp_f32 each).  MASK = false
-// skips the comparison with lo..pos when the caller knows every key is seen by
-// every live column.
+// The base of the exponentials is kept in units of log2: a weight is
+// exp2(score * scale*log2(e) - base), one fused multiply-add and one v_exp_f32.
+// MASK = false skips the comparison with lo..pos when the caller knows every key is
+// seen by every live column (an idle column then computes on zeros; it is never stored).
 template <int NJ, int ND, bool MASK>
 __device__ __forceinline__ void tile_consume(Tile<NJ, ND>& t, const Frag (&ka)[2][NJ], const Frag (&vt)[ND],
                                              int key_c0, int u_stride, float scale_log2) {
@@ -106,26 +124,23 @@ __device__ __forceinline__ void tile_consume(Tile<NJ, ND>& t, const Frag (&ka)[2
     for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            float v = s[u][i] * scale_log2;
+            float v = s[u][i];
             if (MASK) {
                 const int key = key_c0 + u * u_stride + i;
                 v = (key >= t.lo && key <= t.pos) ? v : -INFINITY;
-            } else if (t.pos < 0) {
-                v = -INFINITY;                                   // an idle column
             }
             p[u][i] = v;
             mx = fmaxf(mx, v);
         }
     mx = quad_rows_max(mx);
-    const float m_new = fmaxf(t.m, mx);
-    const float base = (m_new == -INFINITY) ? 0.f : m_new;      // nothing seen yet: all p become 0
-    const float corr = __builtin_amdgcn_exp2f(t.m - base);      // exp2(-inf) = 0 on the first block
+    const float corr = tile_new_base(t.m, mx * scale_log2);
+    const float base = (t.m == -INFINITY) ? 0.f : t.m;          // nothing seen yet: all p become 0
     float sum = 0.f;
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            p[u][i] = __builtin_amdgcn_exp2f(p[u][i] - base);
+            p[u][i] = __builtin_amdgcn_exp2f(fmaf(p[u][i], scale_log2, -base));
             sum += p[u][i];
         }
     Frag pb;
@@ -133,9 +148,8 @@ __device__ __forceinline__ void tile_consume(Tile<NJ, ND>& t, const Frag (&ka)[2
                       pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
     sum = quad_rows_sum(sum);
     t.l = t.l * corr + sum;
-    t.m = m_new;
     // ---- output ----------------------------------------------------------------
-    // the accumulators are rescaled only if some column's maximum moved
+    // the accumulators are rescaled only if the base moved
     if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt)
@@ -175,33 +189,29 @@ __device__ __forceinline__ void tiles_consume(Tile<NJ, ND> (&tiles)[CT], const F
         for (int u = 0; u < 2; ++u)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float v = s[ct][u][i] * scale_log2;
+                float v = s[ct][u][i];
                 if (MASK) {
                     const int key = key_c0 + u * u_stride + i;
                     v = (key >= t.lo && key <= t.pos) ? v : -INFINITY;
-                } else if (t.pos < 0) {
-                    v = -INFINITY;
                 }
                 p[u][i] = v;
                 mx = fmaxf(mx, v);
             }
         mx = quad_rows_max(mx);
-        const float m_new = fmaxf(t.m, mx);
-        const float base = (m_new == -INFINITY) ? 0.f : m_new;
-        corr[ct] = __builtin_amdgcn_exp2f(t.m - base);
+        corr[ct] = tile_new_base(t.m, mx * scale_log2);
+        const float base = (t.m == -INFINITY) ? 0.f : t.m;
         float sum = 0.f;
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                p[u][i] = __builtin_amdgcn_exp2f(p[u][i] - base);
+                p[u][i] = __builtin_amdgcn_exp2f(fmaf(p[u][i], scale_log2, -base));
                 sum += p[u][i];
             }
         pb[ct].u = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
                               pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
         sum = quad_rows_sum(sum);
         t.l = t.l * corr[ct] + sum;
-        t.m = m_new;
     }
     bool moved = false;
 #pragma unroll
