@@ -150,19 +150,25 @@ def test_trace_run_program(model_folders, tmp_path):
     _check(collect(steps, outputs), want, "bfloat16", "model_main --replay --kernels plain")
 
 
-def test_real_layer_sizes(tmp_path):
+@pytest.mark.parametrize("sizes", [
+    dict(hidden_size=4096, intermediate_size=12288, num_attention_heads=32, num_key_value_heads=8),   # Qwen3-8B
+    # the width and the head grouping of Qwen3-14B (5 query heads a kv head) and of Qwen3-32B (8),
+    # fewer heads and a narrower feed-forward to keep the plain implementation's time down
+    dict(hidden_size=5120, intermediate_size=1536, num_attention_heads=10, num_key_value_heads=2),
+    dict(hidden_size=5120, intermediate_size=2560, num_attention_heads=16, num_key_value_heads=2),
+], ids=["8B", "14B-like", "32B-like"])
+def test_real_layer_sizes(tmp_path, sizes):
     """Qwen3-8B layer sizes (hidden 4096, 32 query / 8 kv heads of 128, intermediate
     12288) with random weights, one layer and a small vocabulary to keep the plain
     implementation's time down: all cuts in float32 and in bfloat16, through the
     kernels' full-size code paths (decode layout, MFMA attention, recorded decode
-    steps)."""
+    steps).  Also the width and head grouping of the larger models."""
     from tiny_llm_infer_amd.config import Qwen3Config
     from tiny_llm_infer_amd.engine.loading import load_model, write_random_model
     from tiny_llm_infer_amd.engine.runner import ModelRunner
     cfg = Qwen3Config.from_dict(dict(
-        architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_size=4096, intermediate_size=12288,
-        num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8, head_dim=128, vocab_size=2048,
-        max_position_embeddings=4096, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False))
+        architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=1, head_dim=128, vocab_size=2048,
+        max_position_embeddings=4096, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False, **sizes))
     folder = write_random_model(str(tmp_path / "big"), "Qwen3ForCausalLM", cfg, seed=5)
     reqs = {f"r{i}": random_prompt(2048, n, 300 + i) for i, n in enumerate([150, 97, 40])}
     want = plain_logits(folder, reqs)
@@ -174,6 +180,6 @@ def test_real_layer_sizes(tmp_path):
             runner = ModelRunner(model, model.env, page_size=16, num_pages=24, max_requests=4,
                                  max_batch_tokens=512)
             got = collect(steps, _replay(runner, steps))
-            worst = _check(got, want, dtype, f"8B layer sizes/{dtype}/{cut}")
-            print(f"8B layer sizes {dtype} {cut}: worst relative error {worst:.2e}")
+            worst = _check(got, want, dtype, f"{sizes['hidden_size']} wide/{dtype}/{cut}")
+            print(f"{sizes['hidden_size']} wide, {sizes['num_attention_heads']} heads, {dtype} {cut}: worst relative error {worst:.2e}")
             runner.cache.check()
