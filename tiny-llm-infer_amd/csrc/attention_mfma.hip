@@ -847,10 +847,10 @@ __device__ __forceinline__ void prefill_lds_block(
 
 // With raw.qkv the queries are taken from the raw projections (normed and rotated here, q
 // is not read); needs head_dim == 32*NJ.
-// grid (row blocks, kv_heads * head_tiles), or with `pair` (ceil(row blocks / 2), ...):
-// row blocks late in a sequence walk more keys than early ones, so when there are
-// workgroups to spare each takes block (last - b) and then block b, and all do about
-// the same work.
+// grid (row blocks, kv_heads * head_tiles).  Row blocks late in a sequence walk more keys
+// than early ones; `pair` says how the work is evened out: 1: (ceil(row blocks / 2), ...)
+// workgroups that each take block (last - b) and then block b; 2: long blocks placed beside
+// short ones on a compute unit; 3: long blocks first; 0: as the grid says.
 template <int NJ, int ND, int CT, int KB>
 __global__ void __launch_bounds__(256, (CT == 2 && ND <= 8) ? 2 : 1)
 attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
@@ -884,6 +884,18 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
             hd_i = blockIdx.y;
         }
         (void)linear;
+        prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+                                          table_width, page_size, page_shift, num_pages, heads, kv_heads,
+                                          scale_log2, window, rq, rb, hd_i, raw);
+        return;
+    }
+    if (pair == 3) {
+        // Long row blocks first: workgroups are handed out in the order of their index as
+        // compute units become free, so the short blocks fill the gaps the long ones leave.
+        // The heads vary fastest, so that what runs at the same time walks similar key ranges.
+        if (blockIdx.x >= total) return;                      // the grid's slack
+        const int idx = blockIdx.y * total + blockIdx.x;      // index among the real workgroups
+        const int rb = total - 1 - idx / head_count, hd_i = idx % head_count;
         prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                           table_width, page_size, page_shift, num_pages, heads, kv_heads,
                                           scale_log2, window, rq, rb, hd_i, raw);
@@ -1039,17 +1051,19 @@ static int launch_prefill(
     const RawQkv raw = raw_in ? *raw_in : RawQkv{};
     if (page_size >= 8 && direct != 1) {
         // through LDS, blocks of 64 keys (32 for large heads).  Two column tiles a wave when
-        // that still gives two workgroups for every compute unit (long row blocks are then
-        // placed beside short ones); else one tile a wave.
+        // that still gives two workgroups for every compute unit (long row blocks then come
+        // first); else one tile a wave.
         const long blocks2 = (rows + 8 * rq - 1) / (8 * rq) + num_seqs;
         bool two = head_dim <= 128 && blocks2 * kv_heads * head_tiles >= 512;
         if (direct == 2) two = false;
-        if (direct == 3 || direct >= 4) two = head_dim <= 128;
+        if (direct == 3 || (direct >= 4 && direct <= 7)) two = head_dim <= 128;
+        if (direct == 8) two = false;
         const int rows_per_block = 4 * rq * (two ? 2 : 1);
         const long blocks = (rows + rows_per_block - 1) / rows_per_block + num_seqs;   // upper bound
         if (blocks > 2147483647L) return tli_fail("attention_prefill: too many rows");
-        int pair = two ? 2 : (blocks * kv_heads * head_tiles >= 1024 ? 1 : 2);
-        if (direct >= 4) pair = direct - 4;               // measurements: 4, 5, 6 force the pairing mode
+        int pair = two ? 3 : (blocks * kv_heads * head_tiles >= 1024 ? 1 : 2);
+        if (direct >= 4 && direct <= 7) pair = direct - 4;        // measurements: 4..7 force the pairing mode, two tiles
+        if (direct == 8) pair = 3;                                // one tile, long blocks first
         dim3 grid((unsigned)(pair == 1 ? (blocks + 1) / 2 : blocks), kv_heads * head_tiles);
         const int kb = head_dim <= 128 ? 64 : 32;
         const size_t lds = ((size_t)kb * (head_dim + 8) + (size_t)head_dim * (kb + 8)) * sizeof(bf16_t);
