@@ -144,7 +144,7 @@ def main():
         pre = float("nan")
     else:
         prefill_once()
-        pre = min(prefill_once() for _ in range(3))
+        pre = min(prefill_once() for _ in range(5))
     T = args.prefill_tokens
     pre_flops = step_flops(cfg_json, layers, T, T * (T + 1) / 2.0, 1)
 
