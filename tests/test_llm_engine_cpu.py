@@ -135,3 +135,20 @@ def test_steps_put_on_the_device_ahead_change_nothing(model_folders):
         assert eng.runner.cache.free_pages() == [64, 64] and eng.is_finished()
     assert [r.token_ids for r in outs[0]] == [r.token_ids for r in outs[1]]
     assert len(outs[1][0].token_ids) <= 5 and len(outs[1][2].token_ids) <= 3
+
+
+def test_requests_that_arrive_while_others_are_served(model_folders):
+    """Continuous batching as the benchmark mode drives it: a request joins every
+    few steps; each one's greedy tokens are those it gets alone."""
+    from tiny_llm_infer_amd.cli import _generate_arriving
+    folder = model_folders["B"]
+    cfg, w = plain_qwen3.read_model(folder)
+    prompts = [random_prompt(384, n, 70 + n) for n in (3, 21, 9, 30, 14)]
+    want = [plain_qwen3.greedy(cfg, w, p, 10) for p in prompts]
+    eng = _engine(folder, "B", max_num_seqs=3)
+    params = SamplingParams(max_tokens=10, ignore_eos=True)
+    for interval in (1, 4, 40):              # 40: the engine runs dry between arrivals
+        got = _generate_arriving(eng, [(p, params) for p in prompts], interval)
+        assert [r.token_ids for r in got] == want
+        assert [r.prompt_token_ids for r in got] == prompts
+        eng.runner.cache.check()

@@ -149,6 +149,22 @@ def make_benchmark_requests(num_seqs, min_in, max_in, min_out, max_out, max_toke
     return reqs
 
 
+def _generate_arriving(engine, requests, interval: int):
+    """Continuous batching: request i joins ``interval`` engine steps after request i-1
+    (at once if the engine has run dry), while the earlier ones are being served."""
+    import copy
+    results, admitted, steps = [], 0, 0
+    while admitted < len(requests) or not engine.is_finished():
+        while admitted < len(requests) and (steps >= interval * admitted or engine.is_finished()):
+            prompt, sampling = requests[admitted]
+            engine.add_request(prompt, copy.copy(sampling))
+            admitted += 1
+        results.extend(engine.step())
+        steps += 1
+    results.sort(key=lambda r: r.request_id)
+    return results
+
+
 def run_benchmark(argv: List[str]) -> int:
     ap = argparse.ArgumentParser(prog="model_main --bench")
     _common(ap)
@@ -163,6 +179,10 @@ def run_benchmark(argv: List[str]) -> int:
     ap.add_argument("--manifest-prefix", default=None)
     ap.add_argument("--prefill-only", action="store_true",
                     help="one new token a request: measures prompt tokens a second")
+    ap.add_argument("--arrival-interval", type=int, default=0,
+                    help="engine steps between one request's arrival and the next (0: all are there at the start)")
+    ap.add_argument("--kv-from-free-memory", action="store_true",
+                    help="with --num-kv-blocks 0: as many pages as --gpu-memory-utilization leaves room for")
     args = ap.parse_args(argv)
     if args.prefill_only:
         args.min_output_len = args.max_output_len = 1
@@ -177,7 +197,7 @@ def run_benchmark(argv: List[str]) -> int:
     model = _load(args, max_seq_len)
     page = min(args.page_size, max_seq_len)
     blocks = args.num_kv_blocks
-    if blocks <= 0:
+    if blocks <= 0 and not args.kv_from_free_memory:
         # as the reference: enough for every request's longest possible sequence
         blocks = ((args.max_input_len + args.max_output_len + page - 1) // page) * args.num_seqs
     engine = LLMEngine.from_model(
@@ -196,7 +216,10 @@ def run_benchmark(argv: List[str]) -> int:
                                        args.max_token_id, vocab, seed)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        results = engine.generate([p for p, _ in reqs], [s for _, s in reqs])
+        if args.arrival_interval > 0:
+            results = _generate_arriving(engine, reqs, args.arrival_interval)
+        else:
+            results = engine.generate([p for p, _ in reqs], [s for _, s in reqs])
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         out_tokens = sum(len(r.token_ids) for r in results)
