@@ -90,8 +90,12 @@ def main():
     page = 16
     max_batch = max(64, args.batch)
     budget = max(args.prefill_tokens, 2048)
-    pages = max_batch * ((args.prompt_len + args.steps + args.warmup + 64 + page - 1) // page) \
-        + (args.prefill_tokens + page - 1) // page + 8
+
+    def prefill_steps(batch):
+        """Steps in which the prompts are taken in; those taken in first decode meanwhile."""
+        return (batch * args.prompt_len + budget - 1) // budget + 1
+    pages = max_batch * ((args.prompt_len + args.steps + args.warmup + prefill_steps(max_batch) + 64 + page - 1)
+                         // page) + (args.prefill_tokens + page - 1) // page + 8
     engine = LLMEngine.from_model(model, max_model_len=args.context, page_size=page, num_kv_blocks=pages,
                                   max_num_seqs=max_batch, max_num_batched_tokens=budget)
     rng = random.Random(args.seed)
@@ -99,15 +103,16 @@ def main():
 
     def decode_run(batch, steps, warmup):
         """Prefill ``batch`` prompts, then time ``steps`` decode steps."""
-        # (prompts that were prefilled first decode a few tokens while the others are
-        # prefilled; the margin keeps every request alive through the timed steps)
-        params = SamplingParams(max_tokens=steps + warmup + 17, temperature=0.0, ignore_eos=True)
+        # (the margin keeps every request alive through the timed steps)
+        params = SamplingParams(max_tokens=steps + warmup + prefill_steps(batch) + 16, temperature=0.0,
+                                ignore_eos=True)
         for _ in range(batch):
             engine.add_request([rng.randrange(vocab) for _ in range(args.prompt_len)], params)
         while engine.scheduler.waiting:
             engine.step()
         for _ in range(warmup):
             engine.step()
+        assert len(engine.scheduler.running) == batch
         ctx0 = sum(s.size for s in engine.scheduler.running)
         torch.cuda.synchronize()
         t = time.perf_counter()
@@ -116,6 +121,7 @@ def main():
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         ctx1 = sum(s.size for s in engine.scheduler.running)
+        assert len(engine.scheduler.running) == batch, "a request ended inside the timed steps"
         while not engine.is_finished():
             engine.step()
         return dt, (ctx0 + ctx1) / 2.0
@@ -155,7 +161,7 @@ def main():
             points[f"decode_b{b}"] = round(b * min(args.steps, 32) / d, 2)
 
     out = {
-        "metric": "decode tok/s @ batch 8 (Qwen3-8B shape, bf16, random weights)",
+        "metric": f"decode tok/s @ batch {args.batch} (Qwen3-8B shape, {dkey}, random weights)",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": dkey, "data": "synthetic",
