@@ -275,13 +275,21 @@ ATT_CASES = [
 ]
 
 
-@pytest.mark.parametrize("dtype", DTYPES + ["bfloat16-plain", "bfloat16-direct", "bfloat16-lds1", "bfloat16-lds2"])
+PREFILL_MODES = {"bfloat16-direct": 1, "bfloat16-lds1": 2, "bfloat16-lds2": 3,
+                 # the orders in which workgroups take row blocks (none, pairs in sequence, pairs that
+                 # complement each other, long blocks first), which the launcher picks by the step's size
+                 "bfloat16-order0": 4, "bfloat16-order1": 5, "bfloat16-order2": 6, "bfloat16-order3": 7,
+                 "bfloat16-lds1-order3": 8}
+
+
+@pytest.mark.parametrize("dtype", DTYPES + ["bfloat16-plain"] + list(PREFILL_MODES))
 @pytest.mark.parametrize("case", ATT_CASES)
 def test_paged_attention(ops, dtype, case):
     """float32: the plain kernel.  bfloat16: the MFMA kernels (decode when every
-    sequence brings one row, prefill otherwise), and the plain kernel beside them."""
+    sequence brings one row, prefill otherwise) in each of the prefill kernel's
+    forms, and the plain kernel beside them."""
     ops.force_plain = dtype == "bfloat16-plain"
-    ops.prefill_direct = {"bfloat16-direct": 1, "bfloat16-lds1": 2, "bfloat16-lds2": 3}.get(dtype, 0)
+    ops.prefill_direct = PREFILL_MODES.get(dtype, 0)
     dtype = torch.bfloat16 if isinstance(dtype, str) else dtype
     try:
         _paged_attention_case(ops, dtype, case)
