@@ -88,7 +88,7 @@ def main():
     print(f"[bench] model with {layers} layers on the device in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
 
     page = 16
-    max_batch = max(64, args.batch)
+    max_batch = args.batch if args.no_points else max(64, args.batch)      # the points run 64 requests
     budget = max(args.prefill_tokens, 2048)
 
     def prefill_steps(batch):
