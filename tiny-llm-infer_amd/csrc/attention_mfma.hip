@@ -57,7 +57,8 @@ template <int NJ, int ND>
 struct Tile {
     Frag q[NJ];               // B operand of the score MFMAs: this lane's column, dims of group c
     f32x4 acc[ND];            // O^T[dim = 16*dt + 4c + i][column]
-    float m, l;               // running maximum and sum of this lane's column
+    f32x4 ls;                 // the column's sum of weights, four times (a row of ones times P^T)
+    float m, nb;              // base of the column's exponentials, -inf while nothing is seen; -base (0 then)
     int pos, lo;              // this column sees keys lo..pos (pos < lo: an idle column)
 };
 
@@ -65,9 +66,14 @@ template <int NJ, int ND>
 __device__ __forceinline__ void tile_init(Tile<NJ, ND>& t) {
 #pragma unroll
     for (int d = 0; d < ND; ++d) t.acc[d] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    t.ls = (f32x4){0.f, 0.f, 0.f, 0.f};
     t.m = -INFINITY;
-    t.l = 0.f;
+    t.nb = 0.f;
 }
+
+// The sum of the weights of this lane's column.
+template <int NJ, int ND>
+__device__ __forceinline__ float tile_sum(const Tile<NJ, ND>& t) { return t.ls[0]; }
 
 // Load the query of this lane's column: dims [c*8*NJ + 8j, +8) for j < NJ.
 template <int NJ, int ND>
@@ -80,90 +86,25 @@ __device__ __forceinline__ void tile_load_q(Tile<NJ, ND>& t, const bf16_t* q_hea
     }
 }
 
-// The base of a column's exponentials (the value that exp2 subtracts; in units of log2)
-// follows the column's maximum lazily: it stays as long as no column of the wave has a
-// maximum more than 2^LAZY_BITS above its base, which bounds the weights by 2^LAZY_BITS
-// instead of 1 (harmless in float32 sums and in bfloat16 weights) and saves most of the
-// rescaling of the accumulators.  m: the base so far (-inf: nothing seen), m_now: this
-// block's maximum.  Returns the factor that sums under the old base take under the new
-// one (1 if the base stayed) and updates m.
-#define LAZY_BITS 8.0f
-__device__ __forceinline__ float tile_new_base(float& m, float m_now) {
-    const float m_new = fmaxf(m, m_now);
-    // (-inf) - (-inf) is NaN and compares false: a column that has seen nothing stays
-    if (__builtin_amdgcn_ballot_w64(m_new - m > LAZY_BITS) == 0) return 1.0f;
-    const float base = (m_new == -INFINITY) ? 0.f : m_new;
-    const float corr = __builtin_amdgcn_exp2f(m - base);         // exp2(-inf) = 0 the first time
-    m = m_new;
-    return corr;
-}
-
-// Scores, softmax update and output accumulation of one column tile for 32 keys
-// whose fragments are given.  Row 4c+i of score tile u (and k-slot 4u+i of lane
-// group c in the output MFMA) is the key  key_c0 + u*u_stride + i.
-// The base of the exponentials is kept in units of log2: a weight is
-// exp2(score * scale*log2(e) - base), one fused multiply-add and one v_exp_f32.
+// Scores, softmax update and output accumulation of CT column tiles for 32 keys whose
+// fragments they share.  Row 4c+i of score tile u (and k-slot 4u+i of lane group c in the
+// output MFMA) is the key  key_c0 + u*u_stride + i.
+//
+// A weight is exp2(score * scale*log2(e) - base): one fused multiply-add and one
+// v_exp_f32.  The base of a column follows the column's maximum lazily: it stays as
+// long as no score of the wave lies more than 2^LAZY_BITS above its column's base, which
+// bounds the weights by 2^LAZY_BITS instead of 1 (harmless in float32 sums and in
+// bfloat16 weights).  Whether it may stay is decided from each lane's own 8 scores, so
+// the usual round needs no exchange between lanes at all: only when a base has to move
+// are the columns' maxima gathered over the four lane groups and the accumulators
+// rescaled.  The sum of a column's weights is one more output MFMA, with a row of ones
+// for the values (it adds the weights as rounded to bfloat16, the ones that the
+// values meet).
 // MASK = false skips the comparison with lo..pos when the caller knows every key is
 // seen by every live column (an idle column then computes on zeros; it is never stored).
-template <int NJ, int ND, bool MASK>
-__device__ __forceinline__ void tile_consume(Tile<NJ, ND>& t, const Frag (&ka)[2][NJ], const Frag (&vt)[ND],
-                                             int key_c0, int u_stride, float scale_log2) {
-    // ---- scores ------------------------------------------------------------
-    f32x4 s[2];
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-        s[u] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int j = 0; j < NJ; ++j)
-            s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[u][j].v, t.q[j].v, s[u], 0, 0, 0);
-    }
-    // ---- softmax over this column -------------------------------------------
-    float p[2][4];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float v = s[u][i];
-            if (MASK) {
-                const int key = key_c0 + u * u_stride + i;
-                v = (key >= t.lo && key <= t.pos) ? v : -INFINITY;
-            }
-            p[u][i] = v;
-            mx = fmaxf(mx, v);
-        }
-    mx = quad_rows_max(mx);
-    const float corr = tile_new_base(t.m, mx * scale_log2);
-    const float base = (t.m == -INFINITY) ? 0.f : t.m;          // nothing seen yet: all p become 0
-    float sum = 0.f;
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            p[u][i] = __builtin_amdgcn_exp2f(fmaf(p[u][i], scale_log2, -base));
-            sum += p[u][i];
-        }
-    Frag pb;
-    pb.u = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
-                      pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
-    sum = quad_rows_sum(sum);
-    t.l = t.l * corr + sum;
-    // ---- output ----------------------------------------------------------------
-    // the accumulators are rescaled only if the base moved
-    if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
-#pragma unroll
-        for (int dt = 0; dt < ND; ++dt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) t.acc[dt][i] *= corr;
-    }
-#pragma unroll
-    for (int dt = 0; dt < ND; ++dt)
-        t.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt].v, pb.v, t.acc[dt], 0, 0, 0);
-}
-
-// The same for CT tiles that share the fragments, in phases (all score MFMAs, then all
-// softmax updates, then all output MFMAs), so that one tile's vector arithmetic can
-// run beside another tile's matrix instructions.
+// The phases (all score MFMAs, all softmax arithmetic, all output MFMAs) let one tile's
+// vector arithmetic run beside another tile's matrix instructions.
+#define LAZY_BITS 8.0f
 template <int NJ, int ND, int CT, bool MASK>
 __device__ __forceinline__ void tiles_consume(Tile<NJ, ND> (&tiles)[CT], const Frag (&ka)[2][NJ],
                                               const Frag (&vt)[ND], int key_c0, int u_stride,
@@ -178,57 +119,73 @@ __device__ __forceinline__ void tiles_consume(Tile<NJ, ND> (&tiles)[CT], const F
             for (int j = 0; j < NJ; ++j)
                 s[ct][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[u][j].v, tiles[ct].q[j].v, s[ct][u], 0, 0, 0);
         }
-    Frag pb[CT];
-    float corr[CT];
+    // this lane's maxima, and whether some base has to move
+    float mx[CT];
+    bool move = false;
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         Tile<NJ, ND>& t = tiles[ct];
-        float p[2][4];
-        float mx = -INFINITY;
+        mx[ct] = -INFINITY;
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float v = s[ct][u][i];
                 if (MASK) {
                     const int key = key_c0 + u * u_stride + i;
-                    v = (key >= t.lo && key <= t.pos) ? v : -INFINITY;
+                    s[ct][u][i] = (key >= t.lo && key <= t.pos) ? s[ct][u][i] : -INFINITY;
                 }
-                p[u][i] = v;
-                mx = fmaxf(mx, v);
+                mx[ct] = fmaxf(mx[ct], s[ct][u][i]);
             }
-        mx = quad_rows_max(mx);
-        corr[ct] = tile_new_base(t.m, mx * scale_log2);
-        const float base = (t.m == -INFINITY) ? 0.f : t.m;
-        float sum = 0.f;
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                p[u][i] = __builtin_amdgcn_exp2f(fmaf(p[u][i], scale_log2, -base));
-                sum += p[u][i];
-            }
-        pb[ct].u = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
-                              pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
-        sum = quad_rows_sum(sum);
-        t.l = t.l * corr[ct] + sum;
+        // (nothing seen before and nothing now: -inf + inf is NaN and compares false)
+        move = move || fmaf(mx[ct], scale_log2, -t.m) > LAZY_BITS;
     }
-    bool moved = false;
+    if (__builtin_amdgcn_ballot_w64(move) != 0) {
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) moved = moved || corr[ct] != 1.0f;
-    if (__builtin_amdgcn_ballot_w64(moved) != 0) {
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
+        for (int ct = 0; ct < CT; ++ct) {
+            Tile<NJ, ND>& t = tiles[ct];
+            const float m_new = fmaxf(t.m, quad_rows_max(mx[ct]) * scale_log2);
+            const float base = (m_new == -INFINITY) ? 0.f : m_new;
+            const float corr = __builtin_amdgcn_exp2f(t.m - base);       // exp2(-inf) = 0 the first time
+            t.m = m_new;
+            t.nb = -base;
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) tiles[ct].acc[dt][i] *= corr[ct];
+                for (int i = 0; i < 4; ++i) t.acc[dt][i] *= corr;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) t.ls[i] *= corr;
+        }
     }
+    Frag pb[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const float nb = tiles[ct].nb;
+        float p[2][4];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) p[u][i] = __builtin_amdgcn_exp2f(fmaf(s[ct][u][i], scale_log2, nb));
+        pb[ct].u = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
+                              pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
+    }
+    Frag ones;
+    ones.u = make_uint4(0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u);
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
             tiles[ct].acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt].v, pb[ct].v, tiles[ct].acc[dt], 0, 0, 0);
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+        tiles[ct].ls = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pb[ct].v, tiles[ct].ls, 0, 0, 0);
+}
+
+// The same for one tile.
+template <int NJ, int ND, bool MASK>
+__device__ __forceinline__ void tile_consume(Tile<NJ, ND>& t, const Frag (&ka)[2][NJ], const Frag (&vt)[ND],
+                                             int key_c0, int u_stride, float scale_log2) {
+    Tile<NJ, ND> (&one)[1] = reinterpret_cast<Tile<NJ, ND>(&)[1]>(t);
+    tiles_consume<NJ, ND, 1, MASK>(one, ka, vt, key_c0, u_stride, scale_log2);
 }
 
 // Process the 32 keys t0 .. t0+31 (t0 a multiple of 32) for CT column tiles that
@@ -499,7 +456,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     if (wave > 0) {
         float* dst = lds + ((size_t)(wave - 1) * 64 + lane) * stride;
         dst[0] = t.m;
-        dst[1] = t.l;
+        dst[1] = tile_sum(t);
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
@@ -511,7 +468,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     for (int w = 0; w < 3; ++w) m = fmaxf(m, lds[((size_t)w * 64 + lane) * stride]);
     const float base = (m == -INFINITY) ? 0.f : m;
     float f = __builtin_amdgcn_exp2f(t.m - base);
-    float l = t.l * f;
+    float l = tile_sum(t) * f;
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
@@ -635,7 +592,8 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         if (!live[ct]) continue;
-        const float inv = t[ct].l > 0.f ? 1.0f / t[ct].l : 0.f;
+        const float l = tile_sum(t[ct]);
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
         bf16_t* o = out + ((size_t)row[ct] * heads + head) * head_dim;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt) {
@@ -833,7 +791,201 @@ __device__ __forceinline__ void prefill_lds_block(
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         if (!live[ct]) continue;
-        const float inv = t[ct].l > 0.f ? 1.0f / t[ct].l : 0.f;
+        const float l = tile_sum(t[ct]);
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        bf16_t* o = out + ((size_t)row[ct] * heads + head) * HD;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) {
+            uint2 packed;
+            packed.x = pack_bf16x2(t[ct].acc[dt][0] * inv, t[ct].acc[dt][1] * inv);
+            packed.y = pack_bf16x2(t[ct].acc[dt][2] * inv, t[ct].acc[dt][3] * inv);
+            *reinterpret_cast<uint2*>(o + dt * 16 + 4 * c) = packed;
+        }
+    }
+}
+
+// ------------------------------------- prefill, blocks copied straight into LDS --
+// The same work again for heads of 64 and 128 (ND = 4, 8; NJ = ND/2), with the blocks of
+// 64 keys copied from the cache into LDS by the memory pipeline itself
+// (global_load_lds_dwordx4: lane l of a wave writes the 16 bytes it asked for at LDS
+// base + 16 l), into one of two buffers: the next block is on its way while this one is
+// multiplied, no register holds it meanwhile, and one barrier a block is enough.
+//
+// Such a copy leaves no room for padding between rows, so rows are swizzled instead: a
+// lane chooses which 16 bytes of the cache it asks for, and asks for those that belong at
+// its place.  Keys: row = key, 16-byte chunk q of the row lies at chunk q ^ f(key) with
+// f(key) = (key & 3) | ((key >> 3) & 3) << 2 (halved for rows of 8 chunks): the 16 lanes
+// that read one chunk column for an MFMA operand (keys 8 (r/4) + 4 u + r%4) then hit 16
+// different bank groups.  Values: row = dim, 64 keys = 8 chunks, chunk q at q ^ (dim >> 1 & 7).
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+template <int NJ, int ND, int CT>
+__device__ __forceinline__ void prefill_dma_block(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int* __restrict__ row_start,
+    const int* __restrict__ seq_start, int num_seqs, const int* __restrict__ tables, int table_width,
+    int page_size, int page_shift, int num_pages, int heads, int kv_heads, float scale_log2, int window,
+    int rq, int block, int head_index, const RawQkv& raw) {
+    static_assert(ND == 2 * NJ && (ND == 4 || ND == 8), "heads of 64 or 128");
+    constexpr int KB = 64;
+    constexpr int HD = ND * 16;
+    constexpr int CR = HD / 8;                        // 16-byte chunks of a key row
+    constexpr int CV = KB / 8;                        // 16-byte chunks of a value (dim) row
+    constexpr int KI = KB * CR / 256, VI = HD * CV / 256;       // copies a wave issues for a block
+    constexpr int TILE = KB * HD;                     // elements of a block's keys (and of its values)
+    extern __shared__ uint4 lds_raw[];
+    bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw); // buffer b: keys at b * 2 TILE, values TILE further
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
+    const int group = heads / kv_heads;
+    const int head_tiles = (group + 15) / 16;
+    const int kv_head = head_index / head_tiles, head_tile = head_index % head_tiles;
+    const int heads_here = min(16, group - head_tile * 16);
+    const int rows_per_wave = CT * rq, rows_per_block = 4 * rows_per_wave;
+    int seq = 0, first_row = 0, n_rows = 0;
+    for (; seq < num_seqs; ++seq) {
+        first_row = row_start[seq];
+        n_rows = row_start[seq + 1] - first_row;
+        const int blocks = (n_rows + rows_per_block - 1) / rows_per_block;
+        if (block < blocks) break;
+        block -= blocks;
+    }
+    if (seq >= num_seqs) return;                      // the whole workgroup leaves together
+    const int start = seq_start[seq];
+    const int block0 = block * rows_per_block;        // first row of the workgroup in the portion
+    const int block_rows = min(rows_per_block, n_rows - block0);
+    const int local0 = block0 + wave * rows_per_wave;
+    const int wave_rows = max(0, min(rows_per_wave, n_rows - local0));
+    const int col_row = r / heads_here, col_head = head_tile * 16 + r % heads_here;
+    const int head = kv_head * group + col_head;
+    const int* table = tables + (size_t)seq * table_width;
+
+    Tile<NJ, ND> t[CT];
+    bool live[CT];
+    int row[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int local = ct * rq + col_row;
+        live[ct] = col_row < rq && local < wave_rows;
+        row[ct] = first_row + (live[ct] ? local0 + local : 0);
+        const int pos = start + local0 + local;
+        tile_init(t[ct]);
+        t[ct].pos = live[ct] ? pos : -1;
+        t[ct].lo = live[ct] ? (window > 0 ? max(0, pos - window + 1) : 0) : 0;
+        if (raw.qkv) {
+            const int at = live[ct] ? pos : start;
+            const float* cos_row = raw.cos ? raw.cos + (size_t)at * (HD / 2) : nullptr;
+            const float* sin_row = raw.cos ? raw.sin + (size_t)at * (HD / 2) : nullptr;
+            head_from_raw<NJ>(t[ct].q, raw.qkv + ((size_t)row[ct] * (heads + 2 * kv_heads) + head) * HD,
+                              raw.q_norm_w, raw.q_eps, cos_row, sin_row);
+        } else {
+            tile_load_q(t[ct], q + ((size_t)row[ct] * heads + head) * HD, HD, live[ct]);
+        }
+    }
+    const int wg_first = start + block0, wg_last = wg_first + block_rows - 1;
+    const int wg_lo = window > 0 ? max(0, wg_first - window + 1) : 0;
+    const int wave_first = start + local0, wave_last = wave_first + wave_rows - 1;
+    const int wave_lo = window > 0 ? max(0, wave_first - window + 1) : 0;
+    const int full_lo = window > 0 ? max(0, wave_last - window + 1) : 0, full_hi = wave_first;
+
+    // what this lane asks for in copy e of a block: for keys the row k_row[e] and the
+    // elements from k_col[e]; for values the dim row v_dim[e] and always the same 8 keys
+    auto swz_key = [](int key) {
+        const int f = (key & 3) | (((key >> 3) & 3) << 2);
+        return CR == 16 ? f : f >> 1;
+    };
+    int k_row[KI], k_col[KI];
+    size_t v_off[VI];
+#pragma unroll
+    for (int e = 0; e < KI; ++e) {
+        const int slot = (e * 4 + wave) * 64 + lane;
+        k_row[e] = slot / CR;
+        k_col[e] = ((slot % CR) ^ swz_key(k_row[e])) * 8;
+    }
+    const int v_key8 = ((lane % CV) ^ ((((wave * 64 + lane) / CV) >> 1) & 7)) * 8;     // the same for every e
+#pragma unroll
+    for (int e = 0; e < VI; ++e) v_off[e] = (size_t)(((e * 4 + wave) * 64 + lane) / CV) * page_size;
+    const size_t head_k = (size_t)kv_head * page_size * HD, page_k = (size_t)kv_heads * page_size * HD;
+    const size_t head_v = (size_t)kv_head * HD * page_size, page_v = (size_t)kv_heads * HD * page_size;
+    int k_page[KI], v_page;
+    auto page_of = [&](int key) {
+        const int page = table[min(key >> page_shift, table_width - 1)];
+        return (unsigned)page < (unsigned)num_pages ? page : 0;      // no page: page 0, masked below
+    };
+    auto lookup = [&](int t0) {
+#pragma unroll
+        for (int e = 0; e < KI; ++e) k_page[e] = page_of(t0 + k_row[e]);
+        v_page = page_of(t0 + v_key8);
+    };
+    // start the copies of block t0 into buffer `buf`
+    auto copy = [&](int t0, int buf) {
+        bf16_t* kb = lds + (size_t)buf * 2 * TILE;
+#pragma unroll
+        for (int e = 0; e < KI; ++e) {
+            const int key = t0 + k_row[e];
+            const bf16_t* src = k_cache + (size_t)k_page[e] * page_k + head_k +
+                                (size_t)(key & (page_size - 1)) * HD + k_col[e];
+            __builtin_amdgcn_global_load_lds((const void*)src, (lds_void_t*)(kb + (e * 4 + wave) * 512), 16, 0, 0);
+        }
+        const int vkey = t0 + v_key8;
+        const bf16_t* vbase = v_cache + (size_t)v_page * page_v + head_v + (vkey & (page_size - 1));
+#pragma unroll
+        for (int e = 0; e < VI; ++e)
+            __builtin_amdgcn_global_load_lds((const void*)(vbase + v_off[e]),
+                                             (lds_void_t*)(kb + TILE + (e * 4 + wave) * 512), 16, 0, 0);
+    };
+
+    // LDS offsets (elements) of this lane's fragments inside a 32-key step of a buffer
+    int ka_row[2], ka_col[NJ], vt_col[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) ka_row[u] = (8 * (r / 4) + 4 * u + (r % 4)) * HD;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) ka_col[j] = ((c * NJ + j) ^ (CR == 16 ? r : r >> 1)) * 8;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) vt_col[sub] = ((sub * 4 + c) ^ (r >> 1)) * 8;
+    const int vt_row = r * KB;
+
+    int t0 = (wg_lo / KB) * KB;
+    const int t_last = (wg_last / KB) * KB;             // the last block; asked for again rather than branching
+    lookup(t0);
+    copy(t0, 0);
+    lookup(min(t0 + KB, t_last));
+    int buf = 0;
+    for (; t0 <= wg_last; t0 += KB, buf ^= 1) {
+        // this block has arrived (every lane waits for its own copies, then for the others),
+        // and everyone has finished reading the other buffer
+        __builtin_amdgcn_s_waitcnt(0x0F70);             // vmcnt(0)
+        __syncthreads();
+        copy(min(t0 + KB, t_last), buf ^ 1);
+        lookup(min(t0 + 2 * KB, t_last));
+        const bf16_t* ks = lds + (size_t)buf * 2 * TILE;
+        const bf16_t* vs = ks + TILE;
+#pragma unroll
+        for (int sub = 0; sub < KB / 32; ++sub) {
+            const int s0 = t0 + sub * 32;
+            if (wave_rows <= 0 || s0 > wave_last || s0 + 31 < wave_lo) continue;   // nothing this wave sees
+            Frag ka[2][NJ], vt[ND];
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int j = 0; j < NJ; ++j)
+                    ka[u][j].u = *reinterpret_cast<const uint4*>(ks + sub * 32 * HD + ka_row[u] + ka_col[j]);
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt)
+                vt[dt].u = *reinterpret_cast<const uint4*>(vs + dt * 16 * KB + vt_row + vt_col[sub]);
+            if (s0 >= full_lo && s0 + 31 <= full_hi)
+                tiles_consume<NJ, ND, CT, false>(t, ka, vt, s0 + 8 * c, 4, scale_log2);
+            else
+                tiles_consume<NJ, ND, CT, true>(t, ka, vt, s0 + 8 * c, 4, scale_log2);
+        }
+    }
+    // the copy that the last round started lands before anything else uses the buffers
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        if (!live[ct]) continue;
+        const float l = tile_sum(t[ct]);
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
         bf16_t* o = out + ((size_t)row[ct] * heads + head) * HD;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt) {
@@ -846,13 +998,14 @@ __device__ __forceinline__ void prefill_lds_block(
 }
 
 // With raw.qkv the queries are taken from the raw projections (normed and rotated here, q
-// is not read); needs head_dim == 32*NJ.
+// is not read); needs head_dim == 32*NJ.  DMA: blocks are copied straight into LDS
+// (prefill_dma_block; heads of 64 and 128).
 // grid (row blocks, kv_heads * head_tiles).  Row blocks late in a sequence walk more keys
 // than early ones; `pair` says how the work is evened out: 1: (ceil(row blocks / 2), ...)
 // workgroups that each take block (last - b) and then block b; 2: long blocks placed beside
 // short ones on a compute unit; 3: long blocks first; 0: as the grid says.
-template <int NJ, int ND, int CT, int KB>
-__global__ void __launch_bounds__(256, (CT == 2 && ND <= 8) ? 2 : 1)
+template <int NJ, int ND, int CT, int KB, bool DMA>
+__global__ void __launch_bounds__(256, (ND <= 8 && (CT == 2 || DMA)) ? 2 : 1)
 attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                              const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                              const int* __restrict__ row_start, const int* __restrict__ seq_start,
@@ -884,7 +1037,12 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
             hd_i = blockIdx.y;
         }
         (void)linear;
-        prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+        if constexpr (DMA)
+            prefill_dma_block<NJ, ND, CT>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+                                          table_width, page_size, page_shift, num_pages, heads, kv_heads,
+                                          scale_log2, window, rq, rb, hd_i, raw);
+        else
+            prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                           table_width, page_size, page_shift, num_pages, heads, kv_heads,
                                           scale_log2, window, rq, rb, hd_i, raw);
         return;
@@ -896,19 +1054,34 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
         if (blockIdx.x >= total) return;                      // the grid's slack
         const int idx = blockIdx.y * total + blockIdx.x;      // index among the real workgroups
         const int rb = total - 1 - idx / head_count, hd_i = idx % head_count;
-        prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+        if constexpr (DMA)
+            prefill_dma_block<NJ, ND, CT>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+                                          table_width, page_size, page_shift, num_pages, heads, kv_heads,
+                                          scale_log2, window, rq, rb, hd_i, raw);
+        else
+            prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                           table_width, page_size, page_shift, num_pages, heads, kv_heads,
                                           scale_log2, window, rq, rb, hd_i, raw);
         return;
     }
     const int first = blockIdx.x, second = pair ? total - 1 - first : first;
     if (first >= total || first > second) return;
-    prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+    if constexpr (DMA)
+            prefill_dma_block<NJ, ND, CT>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+                                      table_width, page_size, page_shift, num_pages, heads, kv_heads,
+                                      scale_log2, window, rq, second, blockIdx.y, raw);
+        else
+            prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                       table_width, page_size, page_shift, num_pages, heads, kv_heads,
                                       scale_log2, window, rq, second, blockIdx.y, raw);
     if (second != first) {
         __syncthreads();
-        prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+        if constexpr (DMA)
+            prefill_dma_block<NJ, ND, CT>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+                                          table_width, page_size, page_shift, num_pages, heads, kv_heads,
+                                          scale_log2, window, rq, first, blockIdx.y, raw);
+        else
+            prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                           table_width, page_size, page_shift, num_pages, heads, kv_heads,
                                           scale_log2, window, rq, first, blockIdx.y, raw);
     }
@@ -1066,17 +1239,25 @@ static int launch_prefill(
         if (direct == 8) pair = 3;                                // one tile, long blocks first
         dim3 grid((unsigned)(pair == 1 ? (blocks + 1) / 2 : blocks), kv_heads * head_tiles);
         const int kb = head_dim <= 128 ? 64 : 32;
-        const size_t lds = ((size_t)kb * (head_dim + 8) + (size_t)head_dim * (kb + 8)) * sizeof(bf16_t);
+        // heads of 64 and 128: blocks copied straight into two LDS buffers (direct 11: the
+        // staging through registers for these too)
+        const bool dma = (head_dim == 64 || head_dim == 128) && direct != 11;
+        const size_t lds = dma ? (size_t)2 * 2 * 64 * head_dim * sizeof(bf16_t)
+                               : ((size_t)kb * (head_dim + 8) + (size_t)head_dim * (kb + 8)) * sizeof(bf16_t);
 #define ARGS (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, row_start, \
              seq_start, num_seqs, tables, table_width, page_size, shift, num_pages, heads, kv_heads
 #define TAIL scale * LOG2E, window, rq
 #define TAIL_LDS scale * LOG2E, window, rq, pair, raw
+#define LDS_CALL(NJ, ND, CT, KB, DMA) attention_prefill_lds_kernel<NJ, ND, CT, KB, DMA><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS)
 #define CALL(NJ, ND)                                                                                    \
-    if (ND <= 8 && two) attention_prefill_lds_kernel<NJ, (ND <= 8 ? ND : 1), 2, 64><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS); \
-    else if (ND <= 8) attention_prefill_lds_kernel<NJ, (ND <= 8 ? ND : 1), 1, 64><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS);   \
-    else attention_prefill_lds_kernel<NJ, ND, 1, 32><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS)
+    if ((ND == 4 || ND == 8) && dma && two) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 2, 64, true); \
+    else if ((ND == 4 || ND == 8) && dma) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 1, 64, true); \
+    else if (ND <= 8 && two) LDS_CALL(NJ, (ND <= 8 ? ND : 1), 2, 64, false);                            \
+    else if (ND <= 8) LDS_CALL(NJ, (ND <= 8 ? ND : 1), 1, 64, false);                                   \
+    else LDS_CALL(NJ, ND, 1, 32, false)
         DISPATCH_HEAD_DIM(CALL)
 #undef CALL
+#undef LDS_CALL
         return tli_check_launch("attention_prefill_lds");
     }
     {
