@@ -272,6 +272,10 @@ ATT_CASES = [
     (32, 1, 32, 4, [70], [9], None),
     (6, 2, 80, 16, [200, 31], [200, 31], None),   # 3 heads a group: columns do not fill the tile
     (16, 2, 112, 64, [333], [100], 150),
+    # heads of 128 and 64 with many rows: the blocks go straight from the cache into LDS
+    (8, 2, 128, 8, [200, 75], [200, 40], None),
+    (4, 4, 128, 16, [300], [150], 70),
+    (6, 1, 64, 32, [260, 9], [131, 9], None),
 ]
 
 
@@ -279,9 +283,7 @@ PREFILL_MODES = {"bfloat16-direct": 1, "bfloat16-lds1": 2, "bfloat16-lds2": 3,
                  # the orders in which workgroups take row blocks (none, pairs in sequence, pairs that
                  # complement each other, long blocks first), which the launcher picks by the step's size
                  "bfloat16-order0": 4, "bfloat16-order1": 5, "bfloat16-order2": 6, "bfloat16-order3": 7,
-                 "bfloat16-lds1-order3": 8,
-                 # heads of 64 and 128 staged through registers as the other sizes are
-                 "bfloat16-staged": 11}
+                 "bfloat16-lds1-order3": 8}
 
 
 @pytest.mark.parametrize("dtype", DTYPES + ["bfloat16-plain"] + list(PREFILL_MODES))
@@ -424,13 +426,13 @@ RAW_CASES = [
 ]
 
 
-@pytest.mark.parametrize("mode", [0, 3, 11])
+@pytest.mark.parametrize("mode", [0, 3])
 @pytest.mark.parametrize("case", RAW_CASES)
 def test_attention_from_raw_projections(ops, case, mode):
     """The attention kernels that norm and rotate q (and for a decode step k, writing the
     row's key and value) themselves: against float64 mathematics, and the cache they
     leave against the two-kernel path's.  mode: the prefill kernel's form (0: as the
-    launcher picks, 3: two tiles a wave, 11: blocks staged through registers)."""
+    launcher picks, 3: two tiles a wave)."""
     heads, kv_heads, hd, norms, rotation, page, seq_lens, new_counts, window, writes = case
     if mode and (max(new_counts) == 1 or hd > 128):
         pytest.skip("the forms of the prefill kernel for heads up to 128")

@@ -57,7 +57,8 @@ template <int NJ, int ND>
 struct Tile {
     Frag q[NJ];               // B operand of the score MFMAs: this lane's column, dims of group c
     f32x4 acc[ND];            // O^T[dim = 16*dt + 4c + i][column]
-    f32x4 ls;                 // the column's sum of weights, four times (a row of ones times P^T)
+    f32x4 ls;                 // the column's sum of weights, four times (a row of ones times P^T),
+    float l;                  // or summed by the lanes: one of the two is used, the other stays 0
     float m, nb;              // base of the column's exponentials, -inf while nothing is seen; -base (0 then)
     int pos, lo;              // this column sees keys lo..pos (pos < lo: an idle column)
 };
@@ -67,13 +68,14 @@ __device__ __forceinline__ void tile_init(Tile<NJ, ND>& t) {
 #pragma unroll
     for (int d = 0; d < ND; ++d) t.acc[d] = (f32x4){0.f, 0.f, 0.f, 0.f};
     t.ls = (f32x4){0.f, 0.f, 0.f, 0.f};
+    t.l = 0.f;
     t.m = -INFINITY;
     t.nb = 0.f;
 }
 
 // The sum of the weights of this lane's column.
 template <int NJ, int ND>
-__device__ __forceinline__ float tile_sum(const Tile<NJ, ND>& t) { return t.ls[0]; }
+__device__ __forceinline__ float tile_sum(const Tile<NJ, ND>& t) { return t.ls[0] + t.l; }
 
 // Load the query of this lane's column: dims [c*8*NJ + 8j, +8) for j < NJ.
 template <int NJ, int ND>
@@ -97,15 +99,16 @@ __device__ __forceinline__ void tile_load_q(Tile<NJ, ND>& t, const bf16_t* q_hea
 // bfloat16 weights).  Whether it may stay is decided from each lane's own 8 scores, so
 // the usual round needs no exchange between lanes at all: only when a base has to move
 // are the columns' maxima gathered over the four lane groups and the accumulators
-// rescaled.  The sum of a column's weights is one more output MFMA, with a row of ones
-// for the values (it adds the weights as rounded to bfloat16, the ones that the
-// values meet).
+// rescaled.  MFMA_SUM: the sum of a column's weights is one more output MFMA, with a row
+// of ones for the values (it adds the weights as rounded to bfloat16, the ones that the
+// values meet); else the lanes add them (the decode kernel, which is short of registers
+// and not of vector arithmetic).
 // MASK = false skips the comparison with lo..pos when the caller knows every key is
 // seen by every live column (an idle column then computes on zeros; it is never stored).
 // The phases (all score MFMAs, all softmax arithmetic, all output MFMAs) let one tile's
 // vector arithmetic run beside another tile's matrix instructions.
 #define LAZY_BITS 8.0f
-template <int NJ, int ND, int CT, bool MASK>
+template <int NJ, int ND, int CT, bool MASK, bool MFMA_SUM = true>
 __device__ __forceinline__ void tiles_consume(Tile<NJ, ND> (&tiles)[CT], const Frag (&ka)[2][NJ],
                                               const Frag (&vt)[ND], int key_c0, int u_stride,
                                               float scale_log2) {
@@ -152,8 +155,12 @@ __device__ __forceinline__ void tiles_consume(Tile<NJ, ND> (&tiles)[CT], const F
             for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) t.acc[dt][i] *= corr;
+            if (MFMA_SUM) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) t.ls[i] *= corr;
+                for (int i = 0; i < 4; ++i) t.ls[i] *= corr;
+            } else {
+                t.l *= corr;
+            }
         }
     }
     Frag pb[CT];
@@ -167,25 +174,35 @@ __device__ __forceinline__ void tiles_consume(Tile<NJ, ND> (&tiles)[CT], const F
             for (int i = 0; i < 4; ++i) p[u][i] = __builtin_amdgcn_exp2f(fmaf(s[ct][u][i], scale_log2, nb));
         pb[ct].u = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
                               pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
+        if (!MFMA_SUM) {
+            float sum = 0.f;
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sum += p[u][i];
+            tiles[ct].l += quad_rows_sum(sum);
+        }
     }
-    Frag ones;
-    ones.u = make_uint4(0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u);
 #pragma unroll
     for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
             tiles[ct].acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt].v, pb[ct].v, tiles[ct].acc[dt], 0, 0, 0);
+    if (MFMA_SUM) {
+        Frag ones;
+        ones.u = make_uint4(0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u);
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
-        tiles[ct].ls = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pb[ct].v, tiles[ct].ls, 0, 0, 0);
+        for (int ct = 0; ct < CT; ++ct)
+            tiles[ct].ls = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pb[ct].v, tiles[ct].ls, 0, 0, 0);
+    }
 }
 
-// The same for one tile.
+// The same for one tile, the lanes adding the weights.
 template <int NJ, int ND, bool MASK>
 __device__ __forceinline__ void tile_consume(Tile<NJ, ND>& t, const Frag (&ka)[2][NJ], const Frag (&vt)[ND],
                                              int key_c0, int u_stride, float scale_log2) {
     Tile<NJ, ND> (&one)[1] = reinterpret_cast<Tile<NJ, ND>(&)[1]>(t);
-    tiles_consume<NJ, ND, 1, MASK>(one, ka, vt, key_c0, u_stride, scale_log2);
+    tiles_consume<NJ, ND, 1, MASK, false>(one, ka, vt, key_c0, u_stride, scale_log2);
 }
 
 // Process the 32 keys t0 .. t0+31 (t0 a multiple of 32) for CT column tiles that
@@ -351,7 +368,7 @@ __device__ __forceinline__ void head_from_raw(Frag (&out)[NJ], const bf16_t* src
 // own position writes that key and value into the cache first; needs head_dim == 32*NJ
 // and at most 16 heads a kv head (one workgroup per kv head and split).
 template <int NJ, int ND, bool FUSED>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, ND <= 8 ? 2 : 1)
 attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ partial,
                         bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
                         const int* __restrict__ positions, const int* __restrict__ seq_of_row,
@@ -1239,9 +1256,8 @@ static int launch_prefill(
         if (direct == 8) pair = 3;                                // one tile, long blocks first
         dim3 grid((unsigned)(pair == 1 ? (blocks + 1) / 2 : blocks), kv_heads * head_tiles);
         const int kb = head_dim <= 128 ? 64 : 32;
-        // heads of 64 and 128: blocks copied straight into two LDS buffers (direct 11: the
-        // staging through registers for these too)
-        const bool dma = (head_dim == 64 || head_dim == 128) && direct != 11;
+        // heads of 64 and 128: blocks copied straight into two LDS buffers
+        const bool dma = head_dim == 64 || head_dim == 128;
         const size_t lds = dma ? (size_t)2 * 2 * 64 * head_dim * sizeof(bf16_t)
                                : ((size_t)kb * (head_dim + 8) + (size_t)head_dim * (kb + 8)) * sizeof(bf16_t);
 #define ARGS (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, row_start, \
@@ -1250,10 +1266,10 @@ static int launch_prefill(
 #define TAIL_LDS scale * LOG2E, window, rq, pair, raw
 #define LDS_CALL(NJ, ND, CT, KB, DMA) attention_prefill_lds_kernel<NJ, ND, CT, KB, DMA><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS)
 #define CALL(NJ, ND)                                                                                    \
-    if ((ND == 4 || ND == 8) && dma && two) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 2, 64, true); \
-    else if ((ND == 4 || ND == 8) && dma) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 1, 64, true); \
-    else if (ND <= 8 && two) LDS_CALL(NJ, (ND <= 8 ? ND : 1), 2, 64, false);                            \
-    else if (ND <= 8) LDS_CALL(NJ, (ND <= 8 ? ND : 1), 1, 64, false);                                   \
+    if ((ND == 4 || ND == 8) && two) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 2, 64, true); \
+    else if (ND == 4 || ND == 8) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 1, 64, true); \
+    else if (ND <= 8 && two) LDS_CALL(NJ, ((ND <= 8 && ND != 4 && ND != 8) ? ND : 1), 2, 64, false);    \
+    else if (ND <= 8) LDS_CALL(NJ, ((ND <= 8 && ND != 4 && ND != 8) ? ND : 1), 1, 64, false);           \
     else LDS_CALL(NJ, ND, 1, 32, false)
         DISPATCH_HEAD_DIM(CALL)
 #undef CALL
