@@ -203,10 +203,10 @@ def test_recorded_decode_steps_equal_eager_ones(model_folders):
 
 
 def test_recorded_steps_of_many_rows_equal_eager_ones(tmp_path):
-    """More than 64 rows in a decode step: the matrix products of the recorded step
+    """More than 128 rows in a decode step: the matrix products of the recorded step
     are the library's.  Layer sizes of Qwen3-8B (the library picks its kernels by
-    shape), 80 to 90 live requests in steps of 96 rows; every replay is compared with
-    the same step run eagerly on a second runner, with eager prefill work and
+    shape), 140 to 150 live requests in steps of 160 rows; every replay is compared
+    with the same step run eagerly on a second runner, with eager prefill work and
     synchronisation between the replays."""
     from tiny_llm_infer_amd.config import Qwen3Config
     from tiny_llm_infer_amd.engine.loading import load_model, write_random_model
@@ -217,15 +217,15 @@ def test_recorded_steps_of_many_rows_equal_eager_ones(tmp_path):
         max_position_embeddings=4096, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False))
     folder = write_random_model(str(tmp_path / "wide"), "Qwen3ForCausalLM", cfg, seed=9)
     model, _ = load_model(folder, "bfloat16", "cuda:0")
-    make = lambda: ModelRunner(model, model.env, page_size=16, num_pages=400, max_requests=96,
-                               max_batch_tokens=2048)
+    make = lambda: ModelRunner(model, model.env, page_size=16, num_pages=700, max_requests=160,
+                               max_batch_tokens=4096)
     fast, slow = make(), make()
     slow.use_graphs = False
     rng = np.random.default_rng(4)
     live = []
     for it in range(14):
-        fresh = [f"r{it}_{j}" for j in range(80 if it == 0 else int(rng.integers(0, 4)))]
-        fresh = fresh[:90 - len(live)]
+        fresh = [f"r{it}_{j}" for j in range(140 if it == 0 else int(rng.integers(0, 4)))]
+        fresh = fresh[:150 - len(live)]
         if fresh:
             prompts = [rng.integers(0, 4096, int(rng.integers(2, 20))).tolist() for _ in fresh]
             for r in (fast, slow):
@@ -243,7 +243,7 @@ def test_recorded_steps_of_many_rows_equal_eager_ones(tmp_path):
             fast.release(k)
             slow.release(k)
             live.remove(k)
-    assert fast.graph_replays == 14 and {k[0] for k in fast.graphs} == {96}
+    assert fast.graph_replays == 14 and {k[0] for k in fast.graphs} == {160}
 
 
 def test_decode_steps_are_padded_to_few_sizes(model_folders):

@@ -1,10 +1,19 @@
-// Matrix product for 17..64 rows (a large decode batch): y[M,N] = x[M,K] . W^T with W in
+// Matrix product for 17..128 rows (a large decode batch): y[M,N] = x[M,K] . W^T with W in
 // the decode layout (see gemm_skinny.hip).  Still bound by streaming W once, but with
-// four 16-row tiles of x every W fragment meets four x fragments, and taking those
-// from L2 for every wave (as the kernel for <= 16 rows does) would cost four times
-// the traffic of W itself.  Here the waves of a workgroup own different output
-// columns and walk k together: each 128-wide slice of x (64 rows, 16 KiB) is staged
-// once in LDS and shared by all of them.
+// four or eight 16-row tiles of x every W fragment meets as many x fragments, and taking
+// those from L2 for every wave (as the kernel for <= 16 rows does) would cost that many
+// times the traffic of W itself.  Here the waves of a workgroup own different output
+// columns and walk k together: each 128-wide slice of x (16 MT rows, 4 MT KiB) is brought
+// into LDS once and shared by all of them.
+//
+// The slices of x are copied from memory straight into a ring of LDS buffers
+// (global_load_lds_dwordx4: lane l of a wave writes the 16 bytes it asked for at LDS
+// base + 16 l), DEPTH + 1 slices ahead; the W fragments go into a ring of register
+// stages, DEPTH slices ahead.  No register holds x on its way, and one barrier a slice
+// is enough.  Such a copy leaves no room for padding between rows, so the rows are
+// swizzled: the 16-byte chunk q of row r lies at chunk q ^ (r & 15), and a lane asks for
+// the chunk that belongs at its place; the 16 lanes that read one chunk column of 16
+// rows for an MFMA operand then hit 16 different bank groups.
 //
 // A workgroup owns 16*RT*WAVES output columns and one of `splits` contiguous ranges
 // of k.  With splits > 1 it writes float32 partial sums [split][M][N] and a second
@@ -17,25 +26,34 @@
 #include "common.h"
 #include <type_traits>
 
+// (the copies below set m0 in assembly and say so; nothing else in this file uses m0)
+#pragma clang diagnostic ignored "-Winline-asm"
+
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4m;
+typedef __attribute__((address_space(3))) void lds_void_m;
 
 union Pack16m {
     uint4 u;
+    u32x4m q;
     bf16x8 v;
 };
 
-#define MID_ROWS 64
-#define MID_XPITCH (128 + 8)        // elements per staged x row: 272 bytes
+#define MID_MAX_ROWS 128
 
-template <int RT, int WAVES, int DEPTH, typename TO, bool GATED>
+template <int RT, int WAVES, int DEPTH, int MT, typename TO, bool GATED>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* __restrict__ y,
                 float* __restrict__ part, int M, int N, int K, int splits, int steps_per_split) {
-    __shared__ __attribute__((aligned(16))) bf16_t xs[2][MID_ROWS][MID_XPITCH];
-    constexpr int THREADS = WAVES * 64;
-    constexpr int CHUNKS = MID_ROWS * 16 / THREADS;          // 16-byte chunks of a slice a thread stages
-    constexpr int STAGES = DEPTH + 1;                        // register stages: DEPTH fetches in flight, one in use
+    constexpr int ROWS = MT * 16;
+    constexpr int STAGES = DEPTH + 1;                        // W: DEPTH slices on their way, one in use
+    constexpr int XSLOTS = DEPTH + 2;                        // x: one slice further ahead
+    constexpr int SLICE = ROWS * 128;                        // elements of a slice of x
+    constexpr int XI = ROWS / (4 * WAVES);                   // copies a wave issues for a slice (64 x 16 bytes each)
+    static_assert(ROWS % (4 * WAVES) == 0, "a slice is a whole number of copies for every wave");
+    extern __shared__ uint4 xs_raw[];
+    bf16_t* xs = reinterpret_cast<bf16_t*>(xs_raw);          // [XSLOTS][ROWS][128], rows swizzled
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
     const int k_steps = (K + 127) / 128;
     const int tile0 = (blockIdx.x * WAVES + wave) * RT;       // this wave's first 16-column tile
@@ -43,17 +61,17 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
     const int step_begin = blockIdx.y * steps_per_split;
     const int step_end = min(k_steps, step_begin + steps_per_split);
     // Workgroups walk their k range from different starting slices, wrapping round: a
-    // slice of x is 64 rows a power of two apart, which all lie in one channel of the L2
+    // slice of x is rows a power of two apart, which all lie in one channel of the L2
     // cache, and workgroups in step would all wait for that one channel.  (Workgroups go
     // round the eight dies in turn, so neighbours on a die are blockIdx.x / 8 apart.)
     const int rot = step_begin < step_end ? (blockIdx.x / 8) % (step_end - step_begin) : 0;
     auto at = [&](int step) { return step + rot < step_end ? step + rot : step + rot - (step_end - step_begin); };
 
-    f32x4 acc[RT][4];
+    f32x4 acc[RT][MT];
 #pragma unroll
     for (int t = 0; t < RT; ++t)
 #pragma unroll
-        for (int m = 0; m < 4; ++m) acc[t][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int m = 0; m < MT; ++m) acc[t][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     // W fragments straight from the decode layout: block (tile, step) is 2048 elements,
     // fragment j of this lane at j*512 + lane*8
@@ -64,15 +82,7 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
 #pragma unroll
     for (int t = 0; t < RT; ++t)
         w_tile[t] = w + (size_t)(tile0 + t < n_tiles ? tile0 + t : 0) * k_steps * 2048 + lane * 8;
-    // W fragments and the slices of x (the first workgroup of a die to ask for a slice
-    // gets it from memory, not from L2) are fetched DEPTH slices ahead into a ring of
-    // register stages; a slice of x is written to the LDS buffer that is free one slice
-    // before its use.  Loads complete in the order of issue, so the x fetch of a slice is
-    // issued before its W fetch: the wait for an x chunk never waits for W fragments
-    // that were asked for later.
-    // x staging plan: chunk e of this thread is row (tid + e*THREADS) / 16, 16-byte column (..) % 16
     Pack16m a[STAGES][RT][4];
-    uint4 xreg[STAGES][CHUNKS];
     auto fetch_w = [&](int logical, auto STAGE) {
         constexpr int S = decltype(STAGE)::value;
         const int step = at(logical);
@@ -82,85 +92,104 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
             for (int j = 0; j < 4; ++j)
                 a[S][t][j].u = *reinterpret_cast<const uint4*>(w_tile[t] + (size_t)step * 2048 + j * 512);
     };
-    auto fetch_x = [&](int logical, auto STAGE) {
-        constexpr int S = decltype(STAGE)::value;
-        const int step = at(logical);
+    // What this lane asks for in copy e of a slice: LDS place (e WAVES + wave) 64 + lane, that
+    // is row place / 16 and the chunk that belongs at chunk place % 16 of that row.  Rows past
+    // M repeat the last row (never stored); columns past K read the row's first 8 columns
+    // instead (they meet the zeros that pad W).
+    const bf16_t* x_row[XI];
+    int x_col[XI];
 #pragma unroll
-        for (int e = 0; e < CHUNKS; ++e) {
-            // rows past M repeat the last row (never stored); columns past K read column 0 and are zeroed when staged
-            const int idx = tid + e * THREADS;
-            const int row = min(idx / 16, M - 1), k = step * 128 + (idx % 16) * 8;
-            xreg[S][e] = *reinterpret_cast<const uint4*>(x + (size_t)row * K + (k < K ? k : 0));
+    for (int e = 0; e < XI; ++e) {
+        const int place = (e * WAVES + wave) * 64 + lane, row = place / 16;
+        x_row[e] = x + (size_t)min(row, M - 1) * K;
+        x_col[e] = ((place % 16) ^ (row & 15)) * 8;
+    }
+    // (The copy is written in assembly: told of it, the compiler waits for every load in
+    // flight before the next LDS read, because the copy writes LDS.  Untold, it counts
+    // fewer loads in flight than there are when it waits for W fragments, and so waits for
+    // somewhat more than it needs: for the copies issued before the fragments it lets fly.)
+    const uint32_t xs_base = (uint32_t)(uintptr_t)(lds_void_m*)xs + (uint32_t)wave * 1024u;
+    auto fetch_x = [&](int logical) {
+        const int step = at(logical);
+        const uint32_t slot_base = xs_base + (uint32_t)((logical - step_begin) % XSLOTS) * (SLICE * 2);
+#pragma unroll
+        for (int e = 0; e < XI; ++e) {
+            const int k = step * 128 + x_col[e];
+            const bf16_t* src = x_row[e] + (k < K ? k : 0);
+            const uint32_t dst = __builtin_amdgcn_readfirstlane(slot_base + (uint32_t)(e * WAVES * 1024));
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                         :: "s"(dst), "v"(src) : "m0");
         }
     };
-    auto stage = [&](int logical, int buf, auto STAGE) {
-        constexpr int S = decltype(STAGE)::value;
-        const int step = at(logical);
-#pragma unroll
-        for (int e = 0; e < CHUNKS; ++e) {
-            const int idx = tid + e * THREADS;
-            unsigned keep = step * 128 + (idx % 16) * 8 < K ? 0xffffffffu : 0u;
-            asm volatile("" : "+v"(keep));       // opaque, or the load is moved under a branch on it
-            const uint4 v = xreg[S][e];
-            *reinterpret_cast<uint4*>(&xs[buf][idx / 16][(idx % 16) * 8]) =
-                make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
-        }
+    // Loads complete in the order of issue, and the copy of slice s+1 of x is issued before
+    // the W fragments of slice s: a wave that has multiplied slice s (it waited for those
+    // fragments) has its part of slice s+1 of x in LDS, and after the barrier that opens
+    // slice s+1 every wave has.  (The scheduling barriers keep the compiler from changing
+    // the order of issue.)
+    auto fetch = [&](int logical, auto STAGE, bool with_x) {
+        if (with_x) fetch_x(logical + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_w(logical, STAGE);
+        __builtin_amdgcn_sched_barrier(0);
     };
-    // one slice: `step` is multiplied from register stage S and LDS buffer `buf`.  FULL: every
-    // fetch of this slice exists, so none is under a branch (after a branch that may have
+    // LDS offsets of this lane's x fragments: row m*16 + r, chunk (4c + j) ^ r
+    int b_col[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) b_col[j] = r * 128 + ((4 * c + j) ^ r) * 8;
+
+    // one slice: `step` is multiplied from W stage S and the LDS slot of its x.  FULL: the
+    // fetches of this round exist, so they are under no branch (after a branch that may have
     // issued loads the compiler waits as if it had not, that is for all of them)
-    auto slice = [&](int step, int buf, auto STAGE, auto FULL_T) {
+    auto slice = [&](int step, auto STAGE, auto FULL_T) {
         constexpr int S = decltype(STAGE)::value;
         constexpr bool FULL = decltype(FULL_T)::value;
-        __syncthreads();                                   // slice `buf` is staged; the other is free
-        if (FULL || step + DEPTH < step_end) {
-            fetch_x(step + DEPTH, std::integral_constant<int, (S + DEPTH) % STAGES>{});
-            fetch_w(step + DEPTH, std::integral_constant<int, (S + DEPTH) % STAGES>{});
-        }
+        __syncthreads();        // everyone's part of this slice of x is in LDS, and everyone has finished the slice before
+        if (FULL || step + DEPTH < step_end)
+            fetch(step + DEPTH, std::integral_constant<int, (S + DEPTH) % STAGES>{}, FULL || step + DEPTH + 1 < step_end);
+        const bf16_t* xb = xs + ((step - step_begin) % XSLOTS) * SLICE;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            Pack16m b[4];
+            Pack16m b[MT];
 #pragma unroll
-            for (int m = 0; m < 4; ++m)
-                b[m].u = *reinterpret_cast<const uint4*>(&xs[buf][m * 16 + r][c * 32 + j * 8]);
+            for (int m = 0; m < MT; ++m)
+                b[m].u = *reinterpret_cast<const uint4*>(xb + m * 16 * 128 + b_col[j]);
 #pragma unroll
             for (int t = 0; t < RT; ++t)
 #pragma unroll
-                for (int m = 0; m < 4; ++m)
+                for (int m = 0; m < MT; ++m)
                     acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[S][t][j].v, b[m].v, acc[t][m], 0, 0, 0);
         }
-        // nobody reads the other buffer before the next barrier
-        if (FULL || step + 1 < step_end) stage(step + 1, buf ^ 1, std::integral_constant<int, (S + 1) % STAGES>{});
     };
-    auto slices = [&](auto self, int step, int b0, auto INDEX, auto FULL_T) -> void {
+    auto slices = [&](auto self, int step, auto INDEX, auto FULL_T) -> void {
         constexpr int I = decltype(INDEX)::value;
         if constexpr (I < STAGES) {
             if (decltype(FULL_T)::value || step + I < step_end) {
-                slice(step + I, b0 ^ (I & 1), std::integral_constant<int, I>{}, FULL_T);
-                self(self, step, b0, std::integral_constant<int, I + 1>{}, FULL_T);
+                slice(step + I, std::integral_constant<int, I>{}, FULL_T);
+                self(self, step, std::integral_constant<int, I + 1>{}, FULL_T);
             }
         }
     };
     auto prologue = [&](auto self, auto INDEX) -> void {
         constexpr int I = decltype(INDEX)::value;
         if constexpr (I < DEPTH) {
-            if (step_begin + I < step_end) {
-                fetch_x(step_begin + I, std::integral_constant<int, I>{});
-                fetch_w(step_begin + I, std::integral_constant<int, I>{});
-            }
+            if (step_begin + I < step_end)
+                fetch(step_begin + I, std::integral_constant<int, I>{}, step_begin + I + 1 < step_end);
             self(self, std::integral_constant<int, I + 1>{});
         }
     };
 
     if (step_begin < step_end) {
+        fetch_x(step_begin);
         prologue(prologue, std::integral_constant<int, 0>{});
-        stage(step_begin, 0, std::integral_constant<int, 0>{});
+        // the first slice of x has no W fragments behind it that anyone waits for before the
+        // first barrier: wait for it here
+        __builtin_amdgcn_s_waitcnt(0x0F70);             // vmcnt(0)
     }
     int step = step_begin;
-    for (; step + STAGES - 1 + DEPTH < step_end; step += STAGES)
-        slices(slices, step, (step - step_begin) & 1, std::integral_constant<int, 0>{}, std::true_type{});
+    for (; step + STAGES - 1 + DEPTH + 1 < step_end; step += STAGES)
+        slices(slices, step, std::integral_constant<int, 0>{}, std::true_type{});
     for (; step < step_end; step += STAGES)
-        slices(slices, step, (step - step_begin) & 1, std::integral_constant<int, 0>{}, std::false_type{});
+        slices(slices, step, std::integral_constant<int, 0>{}, std::false_type{});
 
     // lane holds y[m*16 + r][tile*16 + 4c + i]
     if (splits > 1) {
@@ -169,7 +198,7 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
         for (int t = 0; t < RT; ++t) {
             const int n0 = (tile0 + t) * 16 + 4 * c;
 #pragma unroll
-            for (int m = 0; m < 4; ++m) {
+            for (int m = 0; m < MT; ++m) {
                 const int row = m * 16 + r;
                 if (row >= M) continue;
 #pragma unroll
@@ -185,7 +214,7 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
         for (int t = 0; t + 1 < RT; t += 2) {
             const int n0 = ((tile0 + t) / 2) * 16 + 4 * c;
 #pragma unroll
-            for (int m = 0; m < 4; ++m) {
+            for (int m = 0; m < MT; ++m) {
                 const int row = m * 16 + r;
                 if (row >= M) continue;
 #pragma unroll
@@ -202,7 +231,7 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
     for (int t = 0; t < RT; ++t) {
         const int n0 = (tile0 + t) * 16 + 4 * c;
 #pragma unroll
-        for (int m = 0; m < 4; ++m) {
+        for (int m = 0; m < MT; ++m) {
             const int row = m * 16 + r;
             if (row >= M) continue;
 #pragma unroll
@@ -237,18 +266,30 @@ __global__ void gemm_mid_reduce_kernel(const float* __restrict__ part, TO* __res
     }
 }
 
-template <int RT, int WAVES, int DEPTH>
-static int launch_mid(const bf16_t* x, const bf16_t* w, void* y, float* part, int M, int N, int K,
-                      int y_dtype, int gated, int splits, hipStream_t s) {
+template <int RT, int WAVES, int DEPTH, int MT>
+static int launch_mid_rows(const bf16_t* x, const bf16_t* w, void* y, float* part, int M, int N, int K,
+                           int y_dtype, int gated, int splits, hipStream_t s) {
     const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
     const int steps_per_split = (k_steps + splits - 1) / splits;
     dim3 grid((n_tiles + RT * WAVES - 1) / (RT * WAVES), splits);
-    if (gated)
-        gemm_mid_kernel<RT, WAVES, DEPTH, bf16_t, true><<<grid, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, part, M, N, K, splits, steps_per_split);
-    else if (y_dtype == TLI_BF16)
-        gemm_mid_kernel<RT, WAVES, DEPTH, bf16_t, false><<<grid, WAVES * 64, 0, s>>>(x, w, (bf16_t*)y, part, M, N, K, splits, steps_per_split);
-    else
-        gemm_mid_kernel<RT, WAVES, DEPTH, float, false><<<grid, WAVES * 64, 0, s>>>(x, w, (float*)y, part, M, N, K, splits, steps_per_split);
+    const size_t lds = (size_t)(DEPTH + 2) * MT * 16 * 128 * sizeof(bf16_t);
+    // (more than 64 KiB of LDS has to be allowed for a kernel once)
+#define MID_LAUNCH(TO, G)                                                                                  \
+    {                                                                                                      \
+        auto kernel = gemm_mid_kernel<RT, WAVES, DEPTH, MT, TO, G>;                                        \
+        static bool allowed = false;                                                                       \
+        if (lds > 65536 && !allowed) {                                                                     \
+            if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,       \
+                                    (int)lds) != hipSuccess)                                               \
+                return tli_fail("gemm_mid: cannot have %zu bytes of LDS", lds);                            \
+            allowed = true;                                                                                \
+        }                                                                                                  \
+        kernel<<<grid, WAVES * 64, lds, s>>>(x, w, (TO*)y, part, M, N, K, splits, steps_per_split);        \
+    }
+    if (gated) MID_LAUNCH(bf16_t, true)
+    else if (y_dtype == TLI_BF16) MID_LAUNCH(bf16_t, false)
+    else MID_LAUNCH(float, false)
+#undef MID_LAUNCH
     if (tli_check_launch("gemm_mid")) return 1;
     if (splits > 1 && y) {
         const size_t total = (size_t)M * (gated ? N / 2 : N);
@@ -260,6 +301,17 @@ static int launch_mid(const bf16_t* x, const bf16_t* w, void* y, float* part, in
         return tli_check_launch("gemm_mid_reduce");
     }
     return 0;
+}
+
+// Four 16-row tiles of x up to 64 rows, eight beyond.
+template <int RT, int WAVES, int DEPTH>
+static int launch_mid(const bf16_t* x, const bf16_t* w, void* y, float* part, int M, int N, int K,
+                      int y_dtype, int gated, int splits, hipStream_t s) {
+    if (M <= 64) return launch_mid_rows<RT, WAVES, DEPTH, 4>(x, w, y, part, M, N, K, y_dtype, gated, splits, s);
+    if constexpr (DEPTH <= 3)       // (DEPTH + 2) slices of 32 KiB fit the 160 KiB of LDS
+        return launch_mid_rows<RT, WAVES, DEPTH, 8>(x, w, y, part, M, N, K, y_dtype, gated, splits, s);
+    else
+        return tli_fail("gemm_mid: more than 64 rows leave LDS for at most 3 slices on their way");
 }
 
 // Launch shape by measurement on MI355X (4096..151936 columns, k of 4096 and 12288): two
@@ -277,7 +329,7 @@ extern "C" int tli_gemm_mid_splits(int N, int K, int gated) {
     return splits;
 }
 
-// y[M,N] = x[M,K] . W^T for 1 <= M <= 64, W in the decode layout (`gated` as tiled = 2 of
+// y[M,N] = x[M,K] . W^T for 1 <= M <= 128, W in the decode layout (`gated` as tiled = 2 of
 // tli_gemm_skinny_bf16: y is [M, N/2] bfloat16).  `part`: splits*M*N floats when
 // splits > 1 (splits as returned by tli_gemm_mid_splits, or forced by the caller); with
 // y null the partial sums [splits][M][N] are left for the consumer to add (tli_gemm_mid_reduce,
@@ -286,7 +338,7 @@ extern "C" int tli_gemm_mid_splits(int N, int K, int gated) {
 extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* part, int M, int N, int K,
                                  int y_dtype, int gated, int splits, int cfg, void* stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > MID_ROWS) return tli_fail("gemm_mid: %d rows, at most %d", M, MID_ROWS);
+    if (M > MID_MAX_ROWS) return tli_fail("gemm_mid: %d rows, at most %d", M, MID_MAX_ROWS);
     if (K <= 0 || K % 8) return tli_fail("gemm_mid: K = %d must be a positive multiple of 8", K);
     if (y_dtype != TLI_BF16 && y_dtype != TLI_F32) return tli_fail("gemm_mid: bad output dtype %d", y_dtype);
     if (gated && (N % 32 || y_dtype != TLI_BF16))

@@ -122,7 +122,8 @@ class HipOps:
     name = "hip-gfx950"
     MAX_HEAD_DIM = 512
     SKINNY_ROWS = 64
-    MID_ROWS_FROM = 17           # from this many rows the x-sharing kernel multiplies
+    MID_ROWS_FROM = 17           # from this many rows the x-sharing kernel multiplies,
+    MID_ROWS_TO = 128            # up to this many
     DECODE_WORKGROUPS = 512      # aim of the decode attention's key splitting
     DECODE_SPLIT_KEYS = 512      # a split walks at least this many keys
 
@@ -287,11 +288,11 @@ class HipOps:
         if M == 0:
             return y
         if x.dtype == torch.bfloat16 and K % 8 == 0:
+            if tiled is not None and self.MID_ROWS_FROM <= M <= self.MID_ROWS_TO:
+                return self._linear_mid(x, tiled, y, M, N, K, 0, deferred)
             if M <= self.SKINNY_ROWS or out_dtype == torch.float32:
                 # few rows (decode), or float32 logits: the weight-streaming MFMA kernel,
                 # 64 rows at a time
-                if tiled is not None and self.MID_ROWS_FROM <= M <= self.SKINNY_ROWS:
-                    return self._linear_mid(x, tiled, y, M, N, K, 0, deferred)
                 wp = w if tiled is None else tiled
                 for m0 in range(0, M, self.SKINNY_ROWS):
                     m1 = min(M, m0 + self.SKINNY_ROWS)
@@ -339,7 +340,7 @@ class HipOps:
         return y
 
     def _linear_mid(self, x, tiled, y, M, N, K, gated, deferred=False):
-        """17..64 rows: the kernel that shares x through LDS, k cut into ranges when the
+        """17..128 rows: the kernel that shares x through LDS, k cut into ranges when the
         output alone gives too few workgroups.  ``deferred``: the partial sums of the
         ranges are left for the consumer to add, which saves the pass that adds them."""
         splits = self.mid_splits or self.lib.tli_gemm_mid_splits(N, K, gated)
@@ -371,7 +372,7 @@ class HipOps:
             return self._linear_normed(x, m, getattr(m, "gated", None), 1)
         M, K = x.shape
         gated = getattr(m, "gated", None) if not self.plain_products else None
-        if gated is not None and 0 < M <= self.SKINNY_ROWS and x.dtype == torch.bfloat16:
+        if gated is not None and 0 < M <= self.MID_ROWS_TO and x.dtype == torch.bfloat16:
             self._want(x, "linear input", torch.bfloat16, (M, m.w.shape[1]))
             y = torch.empty((M, m.inter), dtype=x.dtype, device=self.device)
             if M >= self.MID_ROWS_FROM:
