@@ -113,7 +113,7 @@ SKINNY = [(1, 4096, 4096), (8, 6144, 4096), (8, 4096, 12288), (16, 301, 80), (17
 @pytest.mark.parametrize("mnk", SKINNY)
 @pytest.mark.parametrize("out", [torch.bfloat16, torch.float32])
 def test_skinny_linear_against_plain_kernel_and_reference(ops, mnk, out):
-    """The weight-streaming MFMA kernel for up to 64 rows, beside the plain tiled kernel."""
+    """The weight-streaming MFMA kernels for up to 128 rows, beside the plain tiled kernel."""
     M, N, K = mnk
     x, w = rnd((M, K), torch.bfloat16, 7), rnd((N, K), torch.bfloat16, 8, 0.05)
     # x lies in front of NaNs: a kernel that reads past a row's end and uses it shows
@@ -550,7 +550,7 @@ def test_rotation_pairs_halves_not_neighbours(ops):
 
 
 def test_partial_sums_as_residual_delta(ops):
-    """A product of 17..64 rows whose k range is split may leave its partial sums to
+    """A product of 17..128 rows whose k range is split may leave its partial sums to
     the norm that follows: the residual and the normed rows are bit for bit what the
     product's own reduction followed by the norm gives, also for a subset of rows."""
     from tiny_llm_infer_amd.kernels.ops import DeferredSum

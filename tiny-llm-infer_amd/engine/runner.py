@@ -49,7 +49,8 @@ def _pad4(n: int) -> int:
 
 def _decode_bucket(n: int) -> int:
     """Recorded decode steps come in these numbers of rows: powers of two up to 64 (up to
-    16 rows, and from 17 to 64, the matrix products cost the same), then multiples of 32."""
+    16 rows, and from 17 to 64, the matrix products cost the same), then multiples of 32 (the
+    products cost the same from 65 to 128 rows; attention and norms do not)."""
     return _pow2_at_least(n, 1) if n <= 64 else (n + 31) // 32 * 32
 
 
