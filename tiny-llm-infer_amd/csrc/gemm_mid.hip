@@ -314,9 +314,10 @@ static int launch_mid(const bf16_t* x, const bf16_t* w, void* y, float* part, in
         return tli_fail("gemm_mid: more than 64 rows leave LDS for at most 3 slices on their way");
 }
 
-// Launch shape by measurement on MI355X (4096..151936 columns, k of 4096 and 12288): two
+// Launch shape by measurement on MI355X (4096..151936 columns, k of 4096..25600): two
 // column tiles a wave once that still leaves about 192 workgroups, else one; k is cut into
-// ranges until there are about 192 workgroups.
+// ranges until there are about 192 workgroups (tli_gemm_mid_bf16 then keeps the workgroups
+// at no more than one a compute unit where it can).
 static int mid_tiles_per_wave(int N, int gated) { return gated || (N + 15) / 16 >= 8 * 192 ? 2 : 1; }
 
 // How many ranges of k a product of this shape is cut into (the caller sizes `part` by it).
@@ -350,7 +351,16 @@ extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* p
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xp = (const bf16_t*)x;
     const bf16_t* wp = (const bf16_t*)w;
-    if (cfg == 0) cfg = 204 + 10 * mid_tiles_per_wave(N, gated);
+    if (cfg == 0) {
+        // more workgroups than compute units cost more than they bring (measured at the layer
+        // sizes of Qwen3-14B and 32B): a gated product then takes eight waves a workgroup, a
+        // plain one whose k ranges push it over takes two column tiles a wave
+        int rt = mid_tiles_per_wave(N, gated), waves = 4;
+        const int groups = ((N + 15) / 16 + 4 * rt - 1) / (4 * rt);
+        if (gated && groups > 256) waves = 8;
+        if (!gated && rt == 1 && (long)groups * splits > 256) rt = 2;
+        cfg = 200 + 10 * rt + waves;
+    }
     if (gated && (cfg / 10) % 10 < 2) return tli_fail("gemm_mid: a gated product needs pairs of row tiles");
 #define MID_CASE(D, R, W) case D * 100 + R * 10 + W: return launch_mid<R, W, D>(xp, wp, y, part, M, N, K, y_dtype, gated, splits, s);
     switch (cfg) {
