@@ -202,11 +202,13 @@ def test_recorded_decode_steps_equal_eager_ones(model_folders):
     assert compared > 30 and fast.graph_replays == compared and len(fast.graphs) >= 3
 
 
-def test_recorded_steps_of_many_rows_equal_eager_ones(tmp_path):
-    """More than 128 rows in a decode step: the matrix products of the recorded step
-    are the library's.  Layer sizes of Qwen3-8B (the library picks its kernels by
-    shape), 140 to 150 live requests in steps of 160 rows; every replay is compared
-    with the same step run eagerly on a second runner, with eager prefill work and
+@pytest.mark.parametrize("first,most,rows", [(80, 90, 96), (140, 150, 160)])
+def test_recorded_steps_of_many_rows_equal_eager_ones(tmp_path, first, most, rows):
+    """Many rows in a decode step, at the layer sizes of Qwen3-8B: up to 128 rows the
+    matrix products are the kernel with eight row tiles, beyond they are the
+    library's (which picks its kernels by shape).  80 to 90 live requests in steps
+    of 96 rows, and 140 to 150 in steps of 160; every replay is compared with the
+    same step run eagerly on a second runner, with eager prefill work and
     synchronisation between the replays."""
     from tiny_llm_infer_amd.config import Qwen3Config
     from tiny_llm_infer_amd.engine.loading import load_model, write_random_model
@@ -217,15 +219,15 @@ def test_recorded_steps_of_many_rows_equal_eager_ones(tmp_path):
         max_position_embeddings=4096, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False))
     folder = write_random_model(str(tmp_path / "wide"), "Qwen3ForCausalLM", cfg, seed=9)
     model, _ = load_model(folder, "bfloat16", "cuda:0")
-    make = lambda: ModelRunner(model, model.env, page_size=16, num_pages=700, max_requests=160,
+    make = lambda: ModelRunner(model, model.env, page_size=16, num_pages=700, max_requests=rows,
                                max_batch_tokens=4096)
     fast, slow = make(), make()
     slow.use_graphs = False
     rng = np.random.default_rng(4)
     live = []
     for it in range(14):
-        fresh = [f"r{it}_{j}" for j in range(140 if it == 0 else int(rng.integers(0, 4)))]
-        fresh = fresh[:150 - len(live)]
+        fresh = [f"r{it}_{j}" for j in range(first if it == 0 else int(rng.integers(0, 4)))]
+        fresh = fresh[:most - len(live)]
         if fresh:
             prompts = [rng.integers(0, 4096, int(rng.integers(2, 20))).tolist() for _ in fresh]
             for r in (fast, slow):
@@ -243,7 +245,7 @@ def test_recorded_steps_of_many_rows_equal_eager_ones(tmp_path):
             fast.release(k)
             slow.release(k)
             live.remove(k)
-    assert fast.graph_replays == 14 and {k[0] for k in fast.graphs} == {160}
+    assert fast.graph_replays == 14 and {k[0] for k in fast.graphs} == {rows}
 
 
 def test_decode_steps_are_padded_to_few_sizes(model_folders):
