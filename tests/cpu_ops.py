@@ -39,7 +39,7 @@ class CpuOps:
     def resolve(self, y):
         return y
 
-    def linear(self, x, w, out_dtype=None, deferred=False):
+    def linear(self, x, w, out_dtype=None, deferred=False, sums_only=False):
         w = getattr(w, "w", w)
         y = x.to(torch.float32) @ w.to(torch.float32).t()
         return y.to(out_dtype or x.dtype)

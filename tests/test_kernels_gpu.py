@@ -449,6 +449,47 @@ def test_attention_from_raw_projections(ops, case, mode):
         ops.prefill_direct = 0
 
 
+@pytest.mark.parametrize("case", [c for c in RAW_CASES if max(c[7]) == 1 and c[2] % 64 == 0])
+@pytest.mark.parametrize("parts", [1, 2, 5])
+def test_decode_attention_adds_partial_sums_of_the_projections(ops, case, parts):
+    """The decode kernel given the projections as float32 partial sums of a split k range
+    leaves the same output and the same cache, bit for bit, as given their sum rounded to
+    bfloat16 (what the product's own reduction writes)."""
+    from tiny_llm_infer_amd.kernels.ops import DeferredSum
+    heads, kv_heads, hd, norms, rotation, page, seq_lens, new_counts, window, writes = case
+    dtype = torch.bfloat16
+    num_pages = sum((n + page - 1) // page for n in seq_lens) + 3
+    step, tables, pos, seq = make_step(seq_lens, new_counts, page, num_pages, 7, kv_heads, hd, dtype, window)
+    fill_cache(step, tables, seq_lens, kv_heads, hd, dtype, 300)
+    step.cache.writes = writes
+    T = len(pos)
+    width = (heads + 2 * kv_heads) * hd
+    planes = torch.stack([rnd((T, width), torch.float32, 60 + p) for p in range(parts)]).to(DEV)
+    planes[0, 0, (heads + kv_heads) * hd + 3] = float("inf")   # a value that has diverged is made finite on its way in
+    total = planes[0].clone()
+    for p in range(1, parts):
+        total += planes[p]                                # the order of the reduction kernel
+    qkv = total.to(dtype)
+    qn = ((1 + rnd((hd,), torch.float32, 22, 0.2)).to(DEV), 1e-5) if norms else None
+    kn = ((1 + rnd((hd,), torch.float32, 23, 0.2)).to(DEV), 3e-6) if norms else None
+    rotary = None
+    if rotation:
+        half = hd // 2
+        ang = torch.arange(2048, dtype=torch.float64)[:, None] * (10000.0 ** (-2.0 * torch.arange(half, dtype=torch.float64) / hd))[None, :]
+        rotary = (torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV), hd)
+    scale = 1.0 / math.sqrt(hd)
+    k0, v0 = step.cache.k.clone(), step.cache.v.clone()
+    want = ops.qkv_attention(qkv, step, step.cache, heads, kv_heads, hd, qn, kn, rotary, scale, window)
+    k1, v1 = step.cache.k.clone(), step.cache.v.clone()
+    step.cache.k.copy_(k0)
+    step.cache.v.copy_(v0)
+    got = ops.qkv_attention(DeferredSum(planes, dtype), step, step.cache, heads, kv_heads, hd, qn, kn, rotary,
+                            scale, window)
+    assert torch.equal(got, want)
+    assert torch.equal(step.cache.k, k1) and torch.equal(step.cache.v, v1)
+    assert bool(torch.isfinite(step.cache.v.float()).all())
+
+
 def _raw_projections_case(ops, case):
     heads, kv_heads, hd, norms, rotation, page, seq_lens, new_counts, window, writes = case
     dtype = torch.bfloat16

@@ -313,24 +313,66 @@ struct RawQkv {
     const float* sin;
     float q_eps, k_eps;
     int write_cache;          // 0: the layer reads a cache that another layer writes
+    // the decode kernel only: the projections as float32 partial sums [parts][rows][columns]
+    // of a product whose k range was split (qkv is then not read); an element is their sum
+    // in part order, rounded to bfloat16 as the product's own reduction would have
+    const float* partial_sums;
+    int parts;
+    size_t part_stride;
 };
 
 // One head of the raw projections as a B operand of the score MFMAs (this lane: dims
 // [c*8*NJ, +8*NJ) of the head at `src`), after the per-head RMS norm (if nw) and the
 // half-split rotation (if cos_row).  head_dim == 32*NJ, so the first half of the head
 // lies in lane groups 0 and 1 and the rotation partner of a lane is lane ^ 32.
+// With psrc the head is taken from `parts` planes of float32 partial sums instead (the
+// head's first element in plane 0 at psrc, planes part_stride floats apart).
 template <int NJ>
 __device__ __forceinline__ void head_from_raw(Frag (&out)[NJ], const bf16_t* src, const float* nw, float eps,
-                                              const float* cos_row, const float* sin_row) {
+                                              const float* cos_row, const float* sin_row,
+                                              const float* psrc = nullptr, int parts = 0, size_t part_stride = 0) {
     const int c = (threadIdx.x % 64) / 16;
     const int d0 = c * 8 * NJ;
     float x[NJ][8];
+    if (psrc) {
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-        Frag f;
-        f.u = *reinterpret_cast<const uint4*>(src + d0 + j * 8);
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) x[j][e] = bf16_to_f32(f.e[e]);
+            for (int e = 0; e < 8; ++e) x[j][e] = 0.f;
+        // two planes a round, both asked for before either is added (the second of an odd
+        // last round is the first again, and counts as zero)
+        for (int p = 0; p < parts; p += 2) {
+            const bool pair = p + 1 < parts;
+            const float* from0 = psrc + (size_t)p * part_stride + d0;
+            const float* from1 = psrc + (size_t)(pair ? p + 1 : p) * part_stride + d0;
+            f32x4 v0[NJ][2], v1[NJ][2];
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                v0[j][0] = *reinterpret_cast<const f32x4*>(from0 + j * 8);
+                v0[j][1] = *reinterpret_cast<const f32x4*>(from0 + j * 8 + 4);
+                v1[j][0] = *reinterpret_cast<const f32x4*>(from1 + j * 8);
+                v1[j][1] = *reinterpret_cast<const f32x4*>(from1 + j * 8 + 4);
+            }
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    x[j][e] += v0[j][e / 4][e % 4];
+                    x[j][e] += pair ? v1[j][e / 4][e % 4] : 0.f;
+                }
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[j][e] = bf16_to_f32(f32_to_bf16(x[j][e]));
+    } else {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            Frag f;
+            f.u = *reinterpret_cast<const uint4*>(src + d0 + j * 8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[j][e] = bf16_to_f32(f.e[e]);
+        }
     }
     if (nw) {
         float ss = 0.f;
@@ -395,15 +437,18 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     t.pos = live ? pos : -1;
     t.lo = live ? lo : 0;
     const bf16_t* raw_row = nullptr;
+    const float* sums_row = nullptr;         // this row in the first plane of partial sums, if the projections come so
     const float *cos_row = nullptr, *sin_row = nullptr;
     if (FUSED) {
         raw_row = raw.qkv + (size_t)row * (heads + 2 * kv_heads) * head_dim;
+        if (raw.partial_sums) sums_row = raw.partial_sums + (size_t)row * (heads + 2 * kv_heads) * head_dim;
         if (raw.cos) {
             cos_row = raw.cos + (size_t)pos * (head_dim / 2);
             sin_row = raw.sin + (size_t)pos * (head_dim / 2);
         }
         // (an idle column computes on head 0; it is masked by its pos of -1)
-        head_from_raw<NJ>(t.q, raw_row + (size_t)(live ? head : 0) * head_dim, raw.q_norm_w, raw.q_eps, cos_row, sin_row);
+        head_from_raw<NJ>(t.q, raw_row + (size_t)(live ? head : 0) * head_dim, raw.q_norm_w, raw.q_eps, cos_row, sin_row,
+                          sums_row ? sums_row + (size_t)(live ? head : 0) * head_dim : nullptr, raw.parts, raw.part_stride);
     } else {
         tile_load_q(t, q + ((size_t)row * heads + (live ? head : 0)) * head_dim, head_dim, live);
     }
@@ -429,7 +474,9 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
                 if (wave == 0) {
                     Frag kf[NJ];
                     head_from_raw<NJ>(kf, raw_row + (size_t)(heads + kv_head) * head_dim, raw.k_norm_w, raw.k_eps,
-                                      cos_row, sin_row);
+                                      cos_row, sin_row,
+                                      sums_row ? sums_row + (size_t)(heads + kv_head) * head_dim : nullptr, raw.parts,
+                                      raw.part_stride);
                     bf16_t* dst = k_cache + (((size_t)page * kv_heads + kv_head) * page_size + slot) * head_dim + c * 8 * NJ;
                     if (r == 0) {
 #pragma unroll
@@ -438,7 +485,22 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
                 } else if (wave == 1) {
                     const bf16_t* src = raw_row + (size_t)(heads + kv_heads + kv_head) * head_dim;
                     bf16_t* dst = v_cache + ((size_t)page * kv_heads + kv_head) * head_dim * page_size + slot;
-                    for (int d = lane; d < head_dim; d += 64) dst[(size_t)d * page_size] = cache_value(src[d]);
+                    if (sums_row) {
+                        const float* from = sums_row + (size_t)(heads + kv_heads + kv_head) * head_dim;
+                        for (int d = lane; d < head_dim; d += 64) {
+                            float v = 0.f;
+                            for (int p = 0; p < raw.parts; p += 2) {
+                                const bool pair = p + 1 < raw.parts;
+                                const float a = from[(size_t)p * raw.part_stride + d];
+                                const float b = from[(size_t)(pair ? p + 1 : p) * raw.part_stride + d];
+                                v += a;
+                                v += pair ? b : 0.f;
+                            }
+                            dst[(size_t)d * page_size] = cache_value(f32_to_bf16(v));
+                        }
+                    } else {
+                        for (int d = lane; d < head_dim; d += 64) dst[(size_t)d * page_size] = cache_value(src[d]);
+                    }
                 }
             }
         }
@@ -1212,10 +1274,14 @@ extern "C" int tli_qkv_attention_decode_bf16(
     int num_pages, int rows, int heads, int kv_heads, int head_dim,
     const float* q_norm_w, float q_eps, const float* k_norm_w, float k_eps,
     const float* cos_table, const float* sin_table, int write_cache,
-    float scale, int window, int splits, int keys_per_split, void* stream) {
-    if (!qkv) return tli_fail("attention_decode from raw projections: no projections");
+    float scale, int window, int splits, int keys_per_split, const float* qkv_partial_sums, int qkv_parts,
+    void* stream) {
+    if (!qkv && !qkv_partial_sums) return tli_fail("attention_decode from raw projections: no projections");
+    if (qkv_partial_sums && (qkv_parts < 1 || qkv_parts > 64 || ((uintptr_t)qkv_partial_sums & 15) || head_dim % 4))
+        return tli_fail("attention_decode: %d planes of partial sums (1..64, 16-byte aligned)", qkv_parts);
     if ((cos_table == nullptr) != (sin_table == nullptr)) return tli_fail("attention_decode: cos without sin");
-    const RawQkv raw{(const bf16_t*)qkv, q_norm_w, k_norm_w, cos_table, sin_table, q_eps, k_eps, write_cache};
+    const RawQkv raw{(const bf16_t*)qkv, q_norm_w, k_norm_w, cos_table, sin_table, q_eps, k_eps, write_cache,
+                     qkv_partial_sums, qkv_parts, (size_t)rows * (heads + 2 * kv_heads) * head_dim};
     return launch_decode(nullptr, out, partial, k_cache, v_cache, positions, seq_of_row, tables, table_width,
                          page_size, num_pages, rows, heads, kv_heads, head_dim, scale, window, splits,
                          keys_per_split, &raw, stream);

@@ -85,7 +85,7 @@ def load_library():
         "tli_gemm_mid_reduce": [P, P, I, I, I, I, P],
         "tli_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
         "tli_qkv_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I,
-                                          F, I, I, I, P],
+                                          F, I, I, I, P, I, P],
         "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, I, P],
         "tli_qkv_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, P, F, P, P, F, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
@@ -262,17 +262,19 @@ class HipOps:
         t = w.view(n16 // 16, 16, k128 // 128, 4, 4, 8)          # [nb, r, kb, c, j, e]
         return t.permute(0, 2, 4, 3, 1, 5).contiguous()           # [nb, kb, j, c, r, e]
 
-    def linear(self, x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None, deferred: bool = False):
+    def linear(self, x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None, deferred: bool = False,
+               sums_only: bool = False):
         """y = x W^T.  ``w`` is a [N, K] tensor or a ``Matrix`` (row-major tensor plus
         its decode layout).  ``deferred``: the caller hands the result to ``add_rmsnorm``
-        (or to ``resolve``) and so also takes a ``DeferredSum``."""
+        (or to ``resolve``) and so also takes a ``PendingProduct`` or a ``DeferredSum``;
+        ``sums_only``: to ``qkv_attention`` (or to ``resolve``), which takes a ``DeferredSum``."""
         if isinstance(x, NormedRows):
             return self._linear_normed(x, w, getattr(w, "tiled", None), 0, out_dtype)
         if self.plain_products:
             return self.linear_plain(x, getattr(w, "w", w), out_dtype)
         tiled = getattr(w, "tiled", None)
-        if (deferred and tiled is not None and x.dtype == torch.bfloat16 and 0 < x.shape[0] <= 16
-                and out_dtype in (None, torch.bfloat16) and not self.separate_norms):
+        if (deferred and not sums_only and tiled is not None and x.dtype == torch.bfloat16
+                and 0 < x.shape[0] <= 16 and out_dtype in (None, torch.bfloat16) and not self.separate_norms):
             return PendingProduct(x, w)
         w = getattr(w, "w", w)
         M, K = x.shape
@@ -289,7 +291,7 @@ class HipOps:
             return y
         if x.dtype == torch.bfloat16 and K % 8 == 0:
             if tiled is not None and self.MID_ROWS_FROM <= M <= self.MID_ROWS_TO:
-                return self._linear_mid(x, tiled, y, M, N, K, 0, deferred)
+                return self._linear_mid(x, tiled, y, M, N, K, 0, deferred or sums_only)
             if M <= self.SKINNY_ROWS or out_dtype == torch.float32:
                 # few rows (decode), or float32 logits: the weight-streaming MFMA kernel,
                 # 64 rows at a time
@@ -469,7 +471,16 @@ class HipOps:
         """From the raw projections to the attention output: norms and rotation of q
         and k, k and v into the cache, attention over the cache.  A decode step (one
         row a sequence) does all of it in the attention kernel where the sizes allow;
-        other steps run qkv_to_cache and paged_attention."""
+        other steps run qkv_to_cache and paged_attention.  ``qkv`` may be a ``DeferredSum``:
+        the kernel of a decode step adds the partial sums itself."""
+        sums = None
+        if isinstance(qkv, DeferredSum):
+            sums = qkv
+            if not (step.max_rows_per_seq == 1 and qkv.dtype == torch.bfloat16 and cache is not None
+                    and head_dim % 64 == 0 and head_dim <= 256 and heads // kv_heads <= 16
+                    and cache.group.page_size >= 4 and not self.force_plain and not self.unfused_decode
+                    and (rotary is None or rotary[2] == head_dim)):
+                qkv, sums = self.resolve(qkv), None
         fusable = (qkv.dtype == torch.bfloat16 and cache is not None and head_dim % 64 == 0
                    and head_dim <= 256 and not self.force_plain and not self.unfused_decode
                    and (rotary is None or rotary[2] == head_dim))
@@ -483,7 +494,11 @@ class HipOps:
             q = self.qkv_to_cache(qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary)
             return self.paged_attention(q, step, cache, heads, kv_heads, head_dim, scale, window)
         T = step.num_rows
-        self._want(qkv, "qkv", None, (T, (heads + 2 * kv_heads) * head_dim))
+        if sums is not None:
+            self._want(sums.parts, "partial sums of qkv", torch.float32,
+                       (sums.parts.shape[0], T, (heads + 2 * kv_heads) * head_dim))
+        else:
+            self._want(qkv, "qkv", None, (T, (heads + 2 * kv_heads) * head_dim))
         kc, vc, g = cache.k, cache.v, cache.group
         self._check_cache(kc, vc, g, kv_heads, head_dim, qkv.dtype, step)
         qw, qe = q_norm if q_norm is not None else (None, 0.0)
@@ -501,11 +516,13 @@ class HipOps:
                 raise KernelError(f"a position reaches {step.max_seq_len}, the rotation table has {npos}")
         out = torch.empty((T, heads * head_dim), dtype=qkv.dtype, device=self.device)
         splits, per_split, partial = self._decode_splits(step, g, heads, kv_heads, head_dim, window)
-        self._call(self.lib.tli_qkv_attention_decode_bf16, qkv.data_ptr(), out.data_ptr(), _ptr(partial),
+        self._call(self.lib.tli_qkv_attention_decode_bf16, None if sums is not None else qkv.data_ptr(),
+                   out.data_ptr(), _ptr(partial),
                    kc.data_ptr(), vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
                    g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], T, heads, kv_heads,
                    head_dim, _ptr(qw), float(qe), _ptr(kw), float(ke), _ptr(cos), _ptr(sin),
                    1 if cache.writes else 0, float(scale), int(window or 0), splits, per_split,
+                   None if sums is None else sums.parts.data_ptr(), 0 if sums is None else sums.parts.shape[0],
                    self._stream())
         return out
 

@@ -74,7 +74,7 @@ class PagedAttention(Mixer):
 
     def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
         ops = self.env.ops
-        qkv = ops.linear(x, self.w_qkv)
+        qkv = ops.linear(x, self.w_qkv, sums_only=True)      # partial sums, if k was split, are the attention's to add
         rot = self.position.rotary() if self.position is not None else None
         o = ops.qkv_attention(
             qkv, step, step.cache, self.heads, self.kv_heads, self.head_dim,
