@@ -183,3 +183,49 @@ def test_real_layer_sizes(tmp_path, sizes):
             worst = _check(got, want, dtype, f"{sizes['hidden_size']} wide/{dtype}/{cut}")
             print(f"{sizes['hidden_size']} wide, {sizes['num_attention_heads']} heads, {dtype} {cut}: worst relative error {worst:.2e}")
             runner.cache.check()
+
+
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_selective_attention_through_every_cut(model_folders, tmp_path, name):
+    """With random weights every key weighs about the same, and a key that is
+    left out or counted twice changes little.  Here the head norms of q and k are
+    doubled, so scores are four times as far apart and few keys carry a row: in
+    float32 every cut still matches the plain implementation and they agree with
+    each other bit for bit; in bfloat16 (where such scores amplify the rounding
+    of q and k) the tuned kernels stay as close to it as the plain kernels do."""
+    import shutil
+    from tiny_llm_infer_amd.weights.safetensors_io import SafetensorsFile, write_safetensors
+    folder = str(tmp_path / name)
+    shutil.copytree(model_folders[name], folder)
+    path = os.path.join(folder, "model.safetensors")
+    src = SafetensorsFile(path)
+    tensors = []
+    for n in src.names():
+        t = src.read(n).clone()
+        if n.endswith("q_norm.weight") or n.endswith("k_norm.weight"):
+            t = (t.float() * 2).to(t.dtype)
+        tensors.append((n, t))
+    src.close()
+    write_safetensors(path, tensors)
+    reqs = _requests(name, [70, 45, 97, 33, 121], seed=15)
+    want = plain_logits(folder, reqs)
+    cuts = {"decode": trace_prefill_then_decode(reqs), "portions": trace_portions(reqs, seed=5),
+            "mixed": trace_mixed(reqs, max_tokens=320, seed=12)}
+    first = None
+    for cut, steps in cuts.items():
+        got = collect(steps, _replay(_runner(folder, name, "float32", 320), steps))
+        _check(got, want, "float32", f"selective {name}/float32/{cut}")
+        if first is None:
+            first = got
+        for rid in reqs:
+            assert np.array_equal(first[rid], got[rid]), (cut, rid)
+
+    def worst(got):
+        return max(max_error(got[rid], want[rid])[0] / max_error(got[rid], want[rid])[2] for rid in want)
+    for cut, steps in cuts.items():
+        tuned = worst(collect(steps, _replay(_runner(folder, name, "bfloat16", 320), steps)))
+        runner = _runner(folder, name, "bfloat16", 320)
+        runner.env.ops.use_plain_kernels()
+        plain = worst(collect(steps, _replay(runner, steps)))
+        print(f"selective {name} bfloat16 {cut}: tuned {tuned:.2e}, plain kernels {plain:.2e}")
+        assert tuned <= 1.5 * plain + 0.1 * TOL["bfloat16"], (cut, tuned, plain)
