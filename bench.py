@@ -60,6 +60,8 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiles)")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement (for profiles)")
+    ap.add_argument("--own-products", action="store_true",
+                    help="products of more than 128 rows by this library's kernel instead of the BLAS library")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -84,6 +86,7 @@ def main():
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
     t0 = time.time()
     model = random_model("Qwen3ForCausalLM", cfg, args.seed, args.dtype, "cuda:0", args.context)
+    model.env.ops.own_products = args.own_products
     torch.cuda.synchronize()
     print(f"[bench] model with {layers} layers on the device in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
 

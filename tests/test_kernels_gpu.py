@@ -170,6 +170,46 @@ def test_gated_product_writes_the_activation(ops, mki):
     close(two_pass, torch.nn.functional.silu(g) * u, torch.bfloat16, "stacked product, then activation")
 
 
+@pytest.mark.parametrize("cfg", [0, 1, 2])
+@pytest.mark.parametrize("mnk", [(129, 264, 1008), (300, 4096, 4096), (2048, 6144, 512), (513, 1000, 136), (700, 48, 8)])
+def test_product_of_many_rows_from_the_decode_layout(ops, mnk, cfg):
+    """gemm_rows (the alternative to the library for more than 128 rows) against float64, at
+    sizes that are no multiples of its tiles, with both launch shapes; rows do not depend
+    on what else is in the batch."""
+    M, N, K = mnk
+    x, w = rnd((M, K), torch.bfloat16, 1).to(DEV), rnd((N, K), torch.bfloat16, 2).to(DEV)
+    tiled = ops.tile_matrix(w)
+    y = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.rows_cfg = cfg
+    try:
+        ops._linear_rows(x, tiled, y, M, N, K, 0)
+        close(y, x.double().cpu() @ w.double().cpu().t(), torch.bfloat16, "product of many rows")
+        part = torch.empty((M // 3, N), dtype=torch.bfloat16, device=DEV)
+        ops._linear_rows(x[M // 5:M // 5 + M // 3].contiguous(), tiled, part, M // 3, N, K, 0)
+        assert torch.equal(part, y[M // 5:M // 5 + M // 3])
+    finally:
+        ops.rows_cfg = 0
+
+
+@pytest.mark.parametrize("mki", [(130, 264, 1008), (2048, 512, 1536), (300, 4096, 96)])
+def test_gated_product_of_many_rows(ops, mki):
+    """gemm_rows over the interleaved gate/up layout writes silu(x gate^T) * (x up^T)."""
+    from tiny_llm_infer_amd.parts.base import BuildEnv
+    from tiny_llm_infer_amd.parts.linear import GatedMatrix
+    M, K, inter = mki
+    x = rnd((M, K), torch.bfloat16, 3, 0.5).to(DEV)
+    gate, up = rnd((inter, K), torch.bfloat16, 4, 0.1).to(DEV), rnd((inter, K), torch.bfloat16, 5, 0.1).to(DEV)
+    m = GatedMatrix(gate, up, BuildEnv(dtype=torch.bfloat16, device=torch.device(DEV), ops=ops, max_model_len=64))
+    ops.own_products = True
+    try:
+        y = ops.linear_swiglu(x, m)
+    finally:
+        ops.own_products = False
+    g, u = x.double().cpu() @ gate.double().cpu().t(), x.double().cpu() @ up.double().cpu().t()
+    close(y, g / (1 + torch.exp(-g)) * u, torch.bfloat16, "gated product of many rows")
+    close(ops.linear_swiglu(x, m), g / (1 + torch.exp(-g)) * u, torch.bfloat16, "the library and the activation")
+
+
 def test_library_linear_for_many_rows(ops):
     x, w = rnd((300, 264), torch.bfloat16, 1), rnd((130, 264), torch.bfloat16, 2, 0.05)
     close(ops.linear(x.to(DEV), w.to(DEV)), x.double() @ w.double().t(), torch.bfloat16, "library product")

@@ -1,0 +1,280 @@
+// Matrix product for many rows (portions of prompts): y[M,N] = x[M,K] . W^T with W in the
+// decode layout (see gemm_skinny.hip), so that a model can do without a row-major copy of
+// its weights.  The library's product stays the default for more than 128 rows; this
+// kernel is the alternative (HipOps.own_products), within a few percent of it at
+// Qwen3-8B layer sizes and 2,048 rows with the SwiGLU taken into the gated product.
+//
+// A workgroup owns ROWS rows and 256 columns and walks all of k in slices of 128:
+//   x   each slice [ROWS][128] is copied from memory straight into one of two LDS slots
+//       (global_load_lds_dwordx4: lane l of a wave writes the 16 bytes it asked for at LDS
+//       base + 16 l), rows swizzled as in gemm_mid.hip (chunk q of row r at q ^ (r & 15));
+//       every wave reads all rows from there;
+//   W   a wave owns RT column tiles of 16 and takes their fragments from memory into one
+//       register stage of four k-steps of 32, each refilled for the next slice as soon as
+//       its products have been issued.
+// All loads of a wave complete in the order of issue, and every load and every wait for
+// one is written in assembly here, so the waits name exact counts: the compiler knows of no
+// load of this kernel, and a fragment's wait carries the fragment's registers through so
+// that its products come after it.
+//
+// Workgroup i runs on die i % 8 (the dies take workgroups in turn): a die is given all
+// row blocks of one column group, then of the next, so its L2 holds the W panel and the
+// rows of x that the workgroups running on it share.
+#include "common.h"
+#include <type_traits>
+
+#pragma clang diagnostic ignored "-Winline-asm"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4r;
+typedef __attribute__((address_space(3))) void lds_void_r;
+
+union Pack16r {
+    uint4 u;
+    u32x4r q;
+    bf16x8 v;
+};
+
+template <int N>
+__device__ __forceinline__ void rows_wait_loads() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Wait until at most N loads are in flight; the fragments of k-step j depend on it.
+template <int N, int RT>
+__device__ __forceinline__ void rows_wait_fragments(Pack16r (&a)[RT][4], int j) {
+    static_assert(RT == 2 || RT == 4, "two or four column tiles a wave");
+    if constexpr (RT == 4)
+        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a[0][j].q), "+v"(a[1][j].q), "+v"(a[2][j].q), "+v"(a[3][j].q) : "n"(N));
+    else
+        asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a[0][j].q), "+v"(a[1][j].q) : "n"(N));
+}
+
+// RT column tiles a wave, WAVES waves side by side, MT row tiles (ROWS = 16 MT), x fragments
+// taken MH row tiles at a time.  GATED: the column tiles alternate between a gate and an up
+// matrix (tiled = 2 of tli_gemm_skinny_bf16) and y is [M, N/2] = silu(gate) * up.
+template <int RT, int WAVES, int MT, int MH, bool GATED>
+__global__ void __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1)
+gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf16_t* __restrict__ y, int M, int N,
+                 int K) {
+    constexpr int ROWS = MT * 16;
+    constexpr int SLICE = ROWS * 128;                        // elements of a slice of x
+    constexpr int XI = ROWS / (4 * WAVES);                   // copies a wave issues for a slice (64 x 16 bytes each)
+    constexpr int HALVES = MT / MH;
+    constexpr int BATCHES = 4 * HALVES;                      // batches of x fragments in a slice
+    static_assert(ROWS % (4 * WAVES) == 0, "a slice is a whole number of copies for every wave");
+    static_assert((4 * WAVES) % 16 == 0, "the swizzle of a lane's chunk is then the same in every copy");
+    static_assert(MT % MH == 0 && 3 * RT + XI <= 63, "the wait counts fit the counter");
+    extern __shared__ uint4 xs_raw[];
+    bf16_t* xs = reinterpret_cast<bf16_t*>(xs_raw);          // [2][ROWS][128], rows swizzled
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, c = lane / 16;
+    const int k_steps = (K + 127) / 128;
+    const int n_tiles = (N + 15) / 16;
+    const int row_blocks = (M + ROWS - 1) / ROWS;
+    const int die = blockIdx.x % 8, turn = blockIdx.x / 8;
+    const int row_block = turn % row_blocks, col_group = (turn / row_blocks) * 8 + die;
+    if (col_group * RT * WAVES >= n_tiles) return;           // (the grid is rounded up to whole rounds of the dies)
+    x += (size_t)row_block * ROWS * K;
+    const int n_out = GATED ? N / 2 : N;
+    y += (size_t)row_block * ROWS * n_out;
+    M = min(ROWS, M - row_block * ROWS);
+    const int tile0 = (col_group * WAVES + wave) * RT;
+
+    f32x4 acc[RT][MT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[t][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    // W fragments: block (tile, slice) is 2048 elements, fragment j of this lane at j*512 + lane*8
+    // (a tile past the last one reads tile 0 instead: its columns are never stored)
+    const bf16_t* w_tile[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+        w_tile[t] = w + (size_t)(tile0 + t < n_tiles ? tile0 + t : 0) * k_steps * 2048 + lane * 8;
+    Pack16r a[RT][4];
+    auto load_w = [&](int slice, int j) {
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            const bf16_t* src = w_tile[t] + (size_t)slice * 2048 + j * 512;
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(a[t][j].q) : "v"(src));
+        }
+    };
+    // What this lane asks for in copy e of a slice: LDS place (e WAVES + wave) 64 + lane, that is
+    // row place / 16 and the chunk that belongs at chunk place % 16 of that row.  Rows past M
+    // repeat the last row (never stored); columns past K read the row's first 8 columns instead
+    // (they meet the zeros that pad W).
+    const int x_row0 = wave * 4 + lane / 16;
+    const int x_col = ((lane % 16) ^ (x_row0 & 15)) * 8;
+    const uint32_t xs_base = (uint32_t)(uintptr_t)(lds_void_r*)xs + (uint32_t)wave * 1024u;
+    auto copy_x = [&](int slice) {
+        const uint32_t slot_base = xs_base + (uint32_t)(slice & 1) * (SLICE * 2);
+        const int k = slice * 128 + x_col;
+#pragma unroll
+        for (int e = 0; e < XI; ++e) {
+            const bf16_t* src = x + (size_t)min(x_row0 + e * 4 * WAVES, M - 1) * K + (k < K ? k : 0);
+            const uint32_t dst = __builtin_amdgcn_readfirstlane(slot_base + (uint32_t)(e * WAVES * 1024));
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(src) : "m0", "memory");
+        }
+    };
+    // LDS offsets of this lane's x fragments: row m*16 + r, chunk (4c + j) ^ r
+    int b_col[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) b_col[j] = r * 128 + ((4 * c + j) ^ r) * 8;
+
+    // batch n of a slice: k-step j = n / HALVES, row tiles (n % HALVES) * MH ..; batch n + 1 is
+    // read from LDS before batch n is multiplied
+    Pack16r b[2][MH];
+    auto read_b = [&](int slice, int n, Pack16r (&dst)[MH]) {
+        const bf16_t* xb = xs + (slice & 1) * SLICE;
+        const int j = n / HALVES, h = n % HALVES;
+#pragma unroll
+        for (int m = 0; m < MH; ++m)
+            dst[m].u = *reinterpret_cast<const uint4*>(xb + (h * MH + m) * 16 * 128 + b_col[j]);
+    };
+    auto multiply = [&](int n, Pack16r (&src)[MH]) {
+        const int j = n / HALVES, h = n % HALVES;
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+            for (int m = 0; m < MH; ++m)
+                acc[t][h * MH + m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][j].v, src[m].v, acc[t][h * MH + m], 0, 0, 0);
+    };
+    // Loads in flight behind the fragments of k-step j when they are waited for: the k-steps
+    // after j of this slice (3 - j times RT), the copy of the next slice of x (XI) and the
+    // k-steps before j of the next slice (j times RT): 3 RT + XI for every j.  In the last slice
+    // nothing follows: (3 - j) RT.
+    auto one_slice = [&](int slice, auto LAST_T) {
+        constexpr bool LAST = decltype(LAST_T)::value;
+        read_b(slice, 0, b[0]);
+#pragma unroll
+        for (int n = 0; n < BATCHES; ++n) {
+            const int j = n / HALVES;
+            if (n % HALVES == 0) {
+                if constexpr (LAST) {
+                    if (j == 0) rows_wait_fragments<3 * RT, RT>(a, 0);
+                    if (j == 1) rows_wait_fragments<2 * RT, RT>(a, 1);
+                    if (j == 2) rows_wait_fragments<RT, RT>(a, 2);
+                    if (j == 3) rows_wait_fragments<0, RT>(a, 3);
+                } else {
+                    rows_wait_fragments<3 * RT + XI, RT>(a, j);
+                }
+            }
+            if (n + 1 < BATCHES) read_b(slice, n + 1, b[(n + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(n, b[n & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (!LAST && n % HALVES == HALVES - 1) load_w(slice + 1, j);
+        }
+    };
+
+    copy_x(0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) load_w(0, j);
+    int slice = 0;
+    for (; slice + 1 < k_steps; ++slice) {
+        rows_wait_loads<4 * RT>();         // this wave's part of the slice of x has landed (behind it: 4 RT fragments)
+        __syncthreads();                   // everyone's has, and everyone has finished the slice before
+        copy_x(slice + 1);                 // into the slot that the slice before used
+        one_slice(slice, std::false_type{});
+    }
+    rows_wait_loads<4 * RT>();
+    __syncthreads();
+    one_slice(slice, std::true_type{});
+
+    // lane holds y[m*16 + r][tile*16 + 4c + i]
+    if (GATED) {
+#pragma unroll
+        for (int t = 0; t + 1 < RT; t += 2) {
+            const int n0 = ((tile0 + t) / 2) * 16 + 4 * c;
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const int row = m * 16 + r;
+                if (row >= M) continue;
+                float o[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float g = acc[t][m][i], u = acc[t + 1][m][i];
+                    o[i] = g / (1.0f + expf(-g)) * u;
+                }
+                bf16_t* dst = y + (size_t)row * n_out + n0;
+                if (n0 + 3 < n_out && n_out % 4 == 0) {
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (n0 + i < n_out) dst[i] = f32_to_bf16(o[i]);
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        const int n0 = (tile0 + t) * 16 + 4 * c;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const int row = m * 16 + r;
+            if (row >= M) continue;
+            bf16_t* dst = y + (size_t)row * N + n0;
+            if (n0 + 3 < N && N % 4 == 0) {
+                *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(acc[t][m][0], acc[t][m][1]),
+                                                            pack_bf16x2(acc[t][m][2], acc[t][m][3]));
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n0 + i < N) dst[i] = f32_to_bf16(acc[t][m][i]);
+            }
+        }
+    }
+}
+
+template <int RT, int WAVES, int MT, int MH>
+static int launch_rows(const bf16_t* x, const bf16_t* w, bf16_t* y, int M, int N, int K, int gated, hipStream_t s) {
+    const int n_tiles = (N + 15) / 16;
+    const long col_groups = (n_tiles + RT * WAVES - 1) / (RT * WAVES), row_blocks = (M + MT * 16 - 1) / (MT * 16);
+    const long blocks = (col_groups + 7) / 8 * 8 * row_blocks;
+    if (blocks > 2147483647L) return tli_fail("gemm_rows: too many workgroups");
+    const size_t lds = (size_t)2 * MT * 16 * 128 * sizeof(bf16_t);
+    // (more than 64 KiB of LDS has to be allowed for a kernel once)
+#define ROWS_LAUNCH(G)                                                                                     \
+    {                                                                                                      \
+        auto kernel = gemm_rows_kernel<RT, WAVES, MT, MH, G>;                                              \
+        static bool allowed = false;                                                                       \
+        if (lds > 65536 && !allowed) {                                                                     \
+            if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,       \
+                                    (int)lds) != hipSuccess)                                               \
+                return tli_fail("gemm_rows: cannot have %zu bytes of LDS", lds);                           \
+            allowed = true;                                                                                \
+        }                                                                                                  \
+        kernel<<<(unsigned)blocks, WAVES * 64, lds, s>>>(x, w, y, M, N, K);                                \
+    }
+    if (gated) ROWS_LAUNCH(true)
+    else ROWS_LAUNCH(false)
+#undef ROWS_LAUNCH
+    return tli_check_launch("gemm_rows");
+}
+
+// y[M,N] = x[M,K] . W^T for any number of rows, bfloat16, W in the decode layout (`gated` as
+// tiled = 2 of tli_gemm_skinny_bf16: N counts gate and up, y is [M, N/2]).
+// cfg 0 picks the launch shape: 256 x 256 outputs a workgroup of eight waves when that gives
+// at least one and a half rounds of the 256 compute units, else 128 x 256 outputs a
+// workgroup of four waves, two workgroups a compute unit (measured on MI355X at 2,048 rows:
+// 4,096 / 6,144 / 24,576 columns); 1, 2 force one.
+extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, int M, int N, int K, int gated, int cfg,
+                                  void* stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K <= 0 || K % 8) return tli_fail("gemm_rows: K = %d must be a positive multiple of 8", K);
+    if (gated && N % 32) return tli_fail("gemm_rows: a gated product needs N %% 32 == 0");
+    if (!x || !w || !y) return tli_fail("gemm_rows: null operand");
+    if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 15) return tli_fail("gemm_rows: operands must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    if (cfg == 0) {
+        const long col_groups = ((N + 15) / 16 + 15) / 16;
+        cfg = col_groups * ((M + 255) / 256) >= 384 ? 1 : 2;
+    }
+    if (cfg == 1) return launch_rows<2, 8, 16, 4>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, M, N, K, gated, s);
+    if (cfg == 2) return launch_rows<4, 4, 8, 2>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, M, N, K, gated, s);
+    return tli_fail("gemm_rows: unknown configuration %d", cfg);
+}

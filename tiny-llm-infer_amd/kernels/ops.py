@@ -83,6 +83,7 @@ def load_library():
         "tli_gemm_mid_bf16": [P, P, P, P, I, I, I, I, I, I, I, P],
         "tli_gemm_mid_splits": [I, I, I],
         "tli_gemm_mid_reduce": [P, P, I, I, I, I, P],
+        "tli_gemm_rows_bf16": [P, P, P, I, I, I, I, I, P],
         "tli_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
         "tli_qkv_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I,
                                           F, I, I, I, P, I, P],
@@ -142,6 +143,8 @@ class HipOps:
         self.mid_cfg = 0             # measurements: launch shape and k ranges of the 17..128-row kernel
         self.mid_splits = 0
         self.skinny_cfg = 0          # measurements: force a launch shape of the weight-streaming kernel
+        self.own_products = False    # products of more than 128 rows through gemm_rows instead of the library
+        self.rows_cfg = 0            # measurements: force a launch shape of gemm_rows
 
     def use_plain_kernels(self) -> None:
         """Every product, attention and norm through the plain kernels, bfloat16 too
@@ -302,6 +305,8 @@ class HipOps:
                                y[m0:m1].data_ptr(), m1 - m0, N, K, _dtype_code(out_dtype),
                                0 if tiled is None else 1, self.skinny_cfg, self._stream())
                 return y
+            if self.own_products and tiled is not None and out_dtype == torch.bfloat16:
+                return self._linear_rows(x, tiled, y, M, N, K, 0)
             # many rows (prefill): the library's matrix product, as the reference
             # uses its library for more than one row (kernels/src/matmul_kernel_cuda.cu:84-91)
             torch.matmul(x, w.t(), out=y)
@@ -354,6 +359,13 @@ class HipOps:
                    _ptr(part), M, N, K, _dtype_code(y.dtype), gated, splits, self.mid_cfg, self._stream())
         return DeferredSum(part, y.dtype) if leave else y
 
+    def _linear_rows(self, x, tiled, y, M, N, K, gated):
+        """Any number of rows from the decode layout (``own_products``): the kernel that
+        would let a model do without the row-major copy of its weights."""
+        self._call(self.lib.tli_gemm_rows_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), M, N, K, gated,
+                   self.rows_cfg, self._stream())
+        return y
+
     def linear_plain(self, x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
         """The plain tiled kernel for any sizes and dtypes: the reference beside the tuned ones."""
         M, K = x.shape
@@ -382,6 +394,10 @@ class HipOps:
             self._call(self.lib.tli_gemm_skinny_bf16, x.data_ptr(), gated.data_ptr(), y.data_ptr(), M,
                        2 * m.inter, K, BF16, 2, self.skinny_cfg if self.skinny_cfg >= 20 else 0, self._stream())
             return y
+        if gated is not None and self.own_products and x.dtype == torch.bfloat16 and K % 8 == 0:
+            self._want(x, "linear input", torch.bfloat16, (M, m.w.shape[1]))
+            y = torch.empty((M, m.inter), dtype=x.dtype, device=self.device)
+            return self._linear_rows(x, gated, y, M, 2 * m.inter, K, 1)
         return self.swiglu(self.linear(x, m))
 
     def swiglu(self, gu: torch.Tensor) -> torch.Tensor:
