@@ -62,6 +62,7 @@ def main():
     ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement (for profiles)")
     ap.add_argument("--own-products", action="store_true",
                     help="products of more than 128 rows by this library's kernel instead of the BLAS library")
+    ap.add_argument("--rows-cfg", type=int, default=0, help="with --own-products: force a launch shape (measurements)")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -87,6 +88,7 @@ def main():
     t0 = time.time()
     model = random_model("Qwen3ForCausalLM", cfg, args.seed, args.dtype, "cuda:0", args.context)
     model.env.ops.own_products = args.own_products
+    model.env.ops.rows_cfg = args.rows_cfg
     torch.cuda.synchronize()
     print(f"[bench] model with {layers} layers on the device in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
 

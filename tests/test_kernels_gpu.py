@@ -191,8 +191,9 @@ def test_product_of_many_rows_from_the_decode_layout(ops, mnk, cfg):
         ops.rows_cfg = 0
 
 
+@pytest.mark.parametrize("cfg", [0, 1, 2])
 @pytest.mark.parametrize("mki", [(130, 264, 1008), (2048, 512, 1536), (300, 4096, 96)])
-def test_gated_product_of_many_rows(ops, mki):
+def test_gated_product_of_many_rows(ops, mki, cfg):
     """gemm_rows over the interleaved gate/up layout writes silu(x gate^T) * (x up^T)."""
     from tiny_llm_infer_amd.parts.base import BuildEnv
     from tiny_llm_infer_amd.parts.linear import GatedMatrix
@@ -200,11 +201,11 @@ def test_gated_product_of_many_rows(ops, mki):
     x = rnd((M, K), torch.bfloat16, 3, 0.5).to(DEV)
     gate, up = rnd((inter, K), torch.bfloat16, 4, 0.1).to(DEV), rnd((inter, K), torch.bfloat16, 5, 0.1).to(DEV)
     m = GatedMatrix(gate, up, BuildEnv(dtype=torch.bfloat16, device=torch.device(DEV), ops=ops, max_model_len=64))
-    ops.own_products = True
+    ops.own_products, ops.rows_cfg = True, cfg
     try:
         y = ops.linear_swiglu(x, m)
     finally:
-        ops.own_products = False
+        ops.own_products, ops.rows_cfg = False, 0
     g, u = x.double().cpu() @ gate.double().cpu().t(), x.double().cpu() @ up.double().cpu().t()
     close(y, g / (1 + torch.exp(-g)) * u, torch.bfloat16, "gated product of many rows")
     close(ops.linear_swiglu(x, m), g / (1 + torch.exp(-g)) * u, torch.bfloat16, "the library and the activation")

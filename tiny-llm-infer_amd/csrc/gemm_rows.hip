@@ -16,6 +16,8 @@
 // one is written in assembly here, so the waits name exact counts: the compiler knows of no
 // load of this kernel, and a fragment's wait carries the fragment's registers through so
 // that its products come after it.
+// (The same kernel on v_mfma_f32_32x32x16_bf16, its W operands put together from pairs of
+// these fragments by v_permlane16_swap and v_permlane32_swap, was measured 7% slower.)
 //
 // Workgroup i runs on die i % 8 (the dies take workgroups in turn): a die is given all
 // row blocks of one column group, then of the next, so its L2 holds the W panel and the
