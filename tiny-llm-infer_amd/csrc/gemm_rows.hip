@@ -1,8 +1,8 @@
 // Matrix product for many rows (portions of prompts): y[M,N] = x[M,K] . W^T with W in the
 // decode layout (see gemm_skinny.hip), so that a model can do without a row-major copy of
 // its weights.  The library's product stays the default for more than 128 rows; this
-// kernel is the alternative (HipOps.own_products), within a few percent of it at
-// Qwen3-8B layer sizes and 2,048 rows with the SwiGLU taken into the gated product.
+// kernel is the alternative (HipOps.own_products), level with it at Qwen3-8B layer sizes
+// and 2,048 rows with the SwiGLU taken into the gated product, behind it at other sizes.
 //
 // A workgroup owns ROWS rows and 256 columns and walks all of k in slices of 128:
 //   x   each slice [ROWS][128] is copied from memory straight into one of two LDS slots
@@ -19,9 +19,9 @@
 // (The same kernel on v_mfma_f32_32x32x16_bf16, its W operands put together from pairs of
 // these fragments by v_permlane16_swap and v_permlane32_swap, was measured 7% slower.)
 //
-// Workgroup i runs on die i % 8 (the dies take workgroups in turn): a die is given all
-// row blocks of one column group, then of the next, so its L2 holds the W panel and the
-// rows of x that the workgroups running on it share.
+// Workgroup i runs on die i % 8 (the dies take workgroups in turn): a die is given the row
+// blocks of 2,048 rows for one column group, then for the next, so its L2 holds the W panel
+// and the rows of x that the workgroups running on it share.
 #include "common.h"
 #include <type_traits>
 
@@ -37,6 +37,15 @@ union Pack16r {
     u32x4r q;
     bf16x8 v;
 };
+
+// f(integral_constant<int, I>) for I = FROM .. TO-1, unrolled at compile time
+template <int FROM, int TO, typename F>
+__device__ __forceinline__ void rows_static_for(F&& f) {
+    if constexpr (FROM < TO) {
+        f(std::integral_constant<int, FROM>{});
+        rows_static_for<FROM + 1, TO>(f);
+    }
+}
 
 template <int N>
 __device__ __forceinline__ void rows_wait_loads() {
@@ -73,10 +82,18 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, c = lane / 16;
     const int k_steps = (K + 127) / 128;
     const int n_tiles = (N + 15) / 16;
+    // Workgroup i runs on die i % 8.  A die takes the row blocks in chunks of 2,048 rows: all
+    // row blocks of a chunk for one column group, then for the next column group of the die, and
+    // so on; then the next chunk (the x rows of a chunk and a W panel stay in its L2 meanwhile).
+    constexpr int CHUNK = 2048 / ROWS;
     const int row_blocks = (M + ROWS - 1) / ROWS;
+    const int groups_a_die = ((n_tiles + RT * WAVES - 1) / (RT * WAVES) + 7) / 8;
     const int die = blockIdx.x % 8, turn = blockIdx.x / 8;
-    const int row_block = turn % row_blocks, col_group = (turn / row_blocks) * 8 + die;
-    if (col_group * RT * WAVES >= n_tiles) return;           // (the grid is rounded up to whole rounds of the dies)
+    const int chunk = turn / (CHUNK * groups_a_die), in_chunk = turn % (CHUNK * groups_a_die);
+    const int chunk_rows = min(CHUNK, row_blocks - chunk * CHUNK);      // row blocks of this chunk (the last may be short)
+    const int row_block = chunk * CHUNK + in_chunk % chunk_rows;
+    const int col_group = (in_chunk / chunk_rows) * 8 + die;
+    if (in_chunk >= chunk_rows * groups_a_die || col_group * RT * WAVES >= n_tiles) return;   // (the grid is rounded up)
     x += (size_t)row_block * ROWS * K;
     const int n_out = GATED ? N / 2 : N;
     y += (size_t)row_block * ROWS * n_out;
@@ -89,35 +106,54 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
 #pragma unroll
         for (int m = 0; m < MT; ++m) acc[t][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
+    // Addresses are a base in scalar registers that moves from slice to slice plus a 32-bit
+    // offset that a lane keeps for the whole kernel, so that the loads cost no vector arithmetic.
     // W fragments: block (tile, slice) is 2048 elements, fragment j of this lane at j*512 + lane*8
     // (a tile past the last one reads tile 0 instead: its columns are never stored)
-    const bf16_t* w_tile[RT];
+    uint32_t w_off[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t)
-        w_tile[t] = w + (size_t)(tile0 + t < n_tiles ? tile0 + t : 0) * k_steps * 2048 + lane * 8;
+        w_off[t] = (uint32_t)(((size_t)(tile0 + t < n_tiles ? tile0 + t : 0) * k_steps * 2048 + lane * 8) * sizeof(bf16_t));
     Pack16r a[RT][4];
-    auto load_w = [&](int slice, int j) {
+    auto load_w = [&](int slice, int j) {          // (j is a constant wherever this is called: one branch remains)
+        const uint64_t base = (uint64_t)(uintptr_t)w + (uint64_t)slice * 4096u;
 #pragma unroll
         for (int t = 0; t < RT; ++t) {
-            const bf16_t* src = w_tile[t] + (size_t)slice * 2048 + j * 512;
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(a[t][j].q) : "v"(src));
+            if (j == 0) asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(a[t][0].q) : "v"(w_off[t]), "s"(base));
+            if (j == 1) asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(a[t][1].q) : "v"(w_off[t]), "s"(base));
+            if (j == 2) asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(a[t][2].q) : "v"(w_off[t]), "s"(base));
+            if (j == 3) asm volatile("global_load_dwordx4 %0, %1, %2 offset:3072" : "=v"(a[t][3].q) : "v"(w_off[t]), "s"(base));
         }
     };
     // What this lane asks for in copy e of a slice: LDS place (e WAVES + wave) 64 + lane, that is
     // row place / 16 and the chunk that belongs at chunk place % 16 of that row.  Rows past M
-    // repeat the last row (never stored); columns past K read the row's first 8 columns instead
-    // (they meet the zeros that pad W).
+    // repeat the last row (never stored).  Where K is no multiple of 128 the columns past K of
+    // the last slice read the row's first 8 columns instead (they meet the zeros that pad W).
     const int x_row0 = wave * 4 + lane / 16;
     const int x_col = ((lane % 16) ^ (x_row0 & 15)) * 8;
+    uint32_t x_off[XI];
+#pragma unroll
+    for (int e = 0; e < XI; ++e)
+        x_off[e] = (uint32_t)(((size_t)min(x_row0 + e * 4 * WAVES, M - 1) * K + x_col) * sizeof(bf16_t));
     const uint32_t xs_base = (uint32_t)(uintptr_t)(lds_void_r*)xs + (uint32_t)wave * 1024u;
+    const bool ragged = (K & 127) != 0;
     auto copy_x = [&](int slice) {
         const uint32_t slot_base = xs_base + (uint32_t)(slice & 1) * (SLICE * 2);
-        const int k = slice * 128 + x_col;
+        if (ragged && slice == k_steps - 1) {
+            const int k = slice * 128 + x_col;
+#pragma unroll
+            for (int e = 0; e < XI; ++e) {
+                const bf16_t* src = x + (size_t)min(x_row0 + e * 4 * WAVES, M - 1) * K + (k < K ? k : 0);
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(slot_base + (uint32_t)(e * WAVES * 1024));
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(src) : "m0", "memory");
+            }
+            return;
+        }
+        const uint64_t base = (uint64_t)(uintptr_t)x + (uint64_t)slice * 256u;
 #pragma unroll
         for (int e = 0; e < XI; ++e) {
-            const bf16_t* src = x + (size_t)min(x_row0 + e * 4 * WAVES, M - 1) * K + (k < K ? k : 0);
             const uint32_t dst = __builtin_amdgcn_readfirstlane(slot_base + (uint32_t)(e * WAVES * 1024));
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(src) : "m0", "memory");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(x_off[e]), "s"(base) : "m0", "memory");
         }
     };
     // LDS offsets of this lane's x fragments: row m*16 + r, chunk (4c + j) ^ r
@@ -150,30 +186,27 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
     auto one_slice = [&](int slice, auto LAST_T) {
         constexpr bool LAST = decltype(LAST_T)::value;
         read_b(slice, 0, b[0]);
-#pragma unroll
-        for (int n = 0; n < BATCHES; ++n) {
-            const int j = n / HALVES;
-            if (n % HALVES == 0) {
-                if constexpr (LAST) {
-                    if (j == 0) rows_wait_fragments<3 * RT, RT>(a, 0);
-                    if (j == 1) rows_wait_fragments<2 * RT, RT>(a, 1);
-                    if (j == 2) rows_wait_fragments<RT, RT>(a, 2);
-                    if (j == 3) rows_wait_fragments<0, RT>(a, 3);
-                } else {
+        rows_static_for<0, BATCHES>([&](auto N_T) {
+            constexpr int n = decltype(N_T)::value, j = n / HALVES;
+            if constexpr (n % HALVES == 0) {
+                if constexpr (LAST)
+                    rows_wait_fragments<(3 - j) * RT, RT>(a, j);
+                else
                     rows_wait_fragments<3 * RT + XI, RT>(a, j);
-                }
             }
-            if (n + 1 < BATCHES) read_b(slice, n + 1, b[(n + 1) & 1]);
+            if constexpr (n + 1 < BATCHES) read_b(slice, n + 1, b[(n + 1) & 1]);
             __builtin_amdgcn_sched_barrier(0);
             multiply(n, b[n & 1]);
             __builtin_amdgcn_sched_barrier(0);
-            if (!LAST && n % HALVES == HALVES - 1) load_w(slice + 1, j);
-        }
+            if constexpr (!LAST && n % HALVES == HALVES - 1) load_w(slice + 1, j);
+        });
     };
 
     copy_x(0);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) load_w(0, j);
+    load_w(0, 0);
+    load_w(0, 1);
+    load_w(0, 2);
+    load_w(0, 3);
     int slice = 0;
     for (; slice + 1 < k_steps; ++slice) {
         rows_wait_loads<4 * RT>();         // this wave's part of the slice of x has landed (behind it: 4 RT fragments)
@@ -236,7 +269,8 @@ template <int RT, int WAVES, int MT, int MH>
 static int launch_rows(const bf16_t* x, const bf16_t* w, bf16_t* y, int M, int N, int K, int gated, hipStream_t s) {
     const int n_tiles = (N + 15) / 16;
     const long col_groups = (n_tiles + RT * WAVES - 1) / (RT * WAVES), row_blocks = (M + MT * 16 - 1) / (MT * 16);
-    const long blocks = (col_groups + 7) / 8 * 8 * row_blocks;
+    const long chunk = 2048 / (MT * 16);                     // as the kernel deals the row blocks out
+    const long blocks = (col_groups + 7) / 8 * 8 * ((row_blocks + chunk - 1) / chunk * chunk);
     if (blocks > 2147483647L) return tli_fail("gemm_rows: too many workgroups");
     const size_t lds = (size_t)2 * MT * 16 * 128 * sizeof(bf16_t);
     // (more than 64 KiB of LDS has to be allowed for a kernel once)
@@ -260,10 +294,9 @@ static int launch_rows(const bf16_t* x, const bf16_t* w, bf16_t* y, int M, int N
 
 // y[M,N] = x[M,K] . W^T for any number of rows, bfloat16, W in the decode layout (`gated` as
 // tiled = 2 of tli_gemm_skinny_bf16: N counts gate and up, y is [M, N/2]).
-// cfg 0 picks the launch shape: 256 x 256 outputs a workgroup of eight waves when that gives
-// at least one and a half rounds of the 256 compute units, else 128 x 256 outputs a
-// workgroup of four waves, two workgroups a compute unit (measured on MI355X at 2,048 rows:
-// 4,096 / 6,144 / 24,576 columns); 1, 2 force one.
+// cfg 0 or 2: 128 x 256 outputs a workgroup of four waves, two workgroups a compute unit (the
+// faster one in the model at 2,048 rows, measured on MI355X); 1: 256 x 256 outputs a workgroup
+// of eight waves.
 extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, int M, int N, int K, int gated, int cfg,
                                   void* stream) {
     if (M <= 0 || N <= 0) return 0;
@@ -272,11 +305,10 @@ extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, int M, 
     if (!x || !w || !y) return tli_fail("gemm_rows: null operand");
     if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 15) return tli_fail("gemm_rows: operands must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
-    if (cfg == 0) {
-        const long col_groups = ((N + 15) / 16 + 15) / 16;
-        cfg = col_groups * ((M + 255) / 256) >= 384 ? 1 : 2;
-    }
+    if (cfg == 0) cfg = 2;
+    if ((size_t)M * K * sizeof(bf16_t) >= (1ull << 32) || (size_t)((N + 15) / 16 * 16) * ((K + 127) / 128 * 128) * sizeof(bf16_t) >= (1ull << 32))
+        return tli_fail("gemm_rows: an operand of 4 GiB or more (offsets are 32 bits)");
     if (cfg == 1) return launch_rows<2, 8, 16, 4>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, M, N, K, gated, s);
-    if (cfg == 2) return launch_rows<4, 4, 8, 2>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, M, N, K, gated, s);
+    if (cfg == 2) return launch_rows<4, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, M, N, K, gated, s);
     return tli_fail("gemm_rows: unknown configuration %d", cfg);
 }
