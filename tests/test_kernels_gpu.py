@@ -180,15 +180,27 @@ def test_product_of_many_rows_from_the_decode_layout(ops, mnk, cfg):
     x, w = rnd((M, K), torch.bfloat16, 1).to(DEV), rnd((N, K), torch.bfloat16, 2).to(DEV)
     tiled = ops.tile_matrix(w)
     y = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
-    ops.rows_cfg = cfg
+    ops.rows_cfg, ops.rows_splits = cfg, 1
     try:
         ops._linear_rows(x, tiled, y, M, N, K, 0)
-        close(y, x.double().cpu() @ w.double().cpu().t(), torch.bfloat16, "product of many rows")
+        want = x.double().cpu() @ w.double().cpu().t()
+        close(y, want, torch.bfloat16, "product of many rows")
         part = torch.empty((M // 3, N), dtype=torch.bfloat16, device=DEV)
         ops._linear_rows(x[M // 5:M // 5 + M // 3].contiguous(), tiled, part, M // 3, N, K, 0)
         assert torch.equal(part, y[M // 5:M // 5 + M // 3])
+        # k cut into ranges (more than there are slices of 128, too): the sum of the partial products,
+        # and the partial sums left for the consumer
+        for splits in (0, 3, 16):
+            ops.rows_splits = splits
+            y2 = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+            close(ops._linear_rows(x, tiled, y2, M, N, K, 0), want, torch.bfloat16, f"{splits} ranges of k")
+            left = ops._linear_rows(x, tiled, y2, M, N, K, 0, deferred=True)
+            if splits > 1:
+                assert tuple(left.parts.shape) == (splits, M, N)
+                close(left.parts.sum(0), want, torch.float32, "partial sums")
+            close(ops.resolve(left), want, torch.bfloat16, "partial sums resolved")
     finally:
-        ops.rows_cfg = 0
+        ops.rows_cfg = ops.rows_splits = 0
 
 
 @pytest.mark.parametrize("cfg", [0, 1, 2])
@@ -201,11 +213,15 @@ def test_gated_product_of_many_rows(ops, mki, cfg):
     x = rnd((M, K), torch.bfloat16, 3, 0.5).to(DEV)
     gate, up = rnd((inter, K), torch.bfloat16, 4, 0.1).to(DEV), rnd((inter, K), torch.bfloat16, 5, 0.1).to(DEV)
     m = GatedMatrix(gate, up, BuildEnv(dtype=torch.bfloat16, device=torch.device(DEV), ops=ops, max_model_len=64))
+    g, u = x.double().cpu() @ gate.double().cpu().t(), x.double().cpu() @ up.double().cpu().t()
     ops.own_products, ops.rows_cfg = True, cfg
     try:
+        for splits in (1, 0, 4):
+            ops.rows_splits = splits
+            close(ops.linear_swiglu(x, m), g / (1 + torch.exp(-g)) * u, torch.bfloat16, f"gated product, {splits} ranges of k")
         y = ops.linear_swiglu(x, m)
     finally:
-        ops.own_products, ops.rows_cfg = False, 0
+        ops.own_products, ops.rows_cfg, ops.rows_splits = False, 0, 0
     g, u = x.double().cpu() @ gate.double().cpu().t(), x.double().cpu() @ up.double().cpu().t()
     close(y, g / (1 + torch.exp(-g)) * u, torch.bfloat16, "gated product of many rows")
     close(ops.linear_swiglu(x, m), g / (1 + torch.exp(-g)) * u, torch.bfloat16, "the library and the activation")

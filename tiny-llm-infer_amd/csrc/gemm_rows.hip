@@ -23,6 +23,7 @@
 // blocks of 2,048 rows for one column group, then for the next, so its L2 holds the W panel
 // and the rows of x that the workgroups running on it share.
 #include "common.h"
+#include "gemm_reduce.h"
 #include <type_traits>
 
 #pragma clang diagnostic ignored "-Winline-asm"
@@ -67,8 +68,8 @@ __device__ __forceinline__ void rows_wait_fragments(Pack16r (&a)[RT][4], int j) 
 // matrix (tiled = 2 of tli_gemm_skinny_bf16) and y is [M, N/2] = silu(gate) * up.
 template <int RT, int WAVES, int MT, int MH, bool GATED>
 __global__ void __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1)
-gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf16_t* __restrict__ y, int M, int N,
-                 int K) {
+gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf16_t* __restrict__ y,
+                 float* __restrict__ part, int M, int N, int K, int splits, int slices_per_split) {
     constexpr int ROWS = MT * 16;
     constexpr int SLICE = ROWS * 128;                        // elements of a slice of x
     constexpr int XI = ROWS / (4 * WAVES);                   // copies a wave issues for a slice (64 x 16 bytes each)
@@ -97,7 +98,10 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
     x += (size_t)row_block * ROWS * K;
     const int n_out = GATED ? N / 2 : N;
     y += (size_t)row_block * ROWS * n_out;
+    // with splits > 1 the workgroup walks one of `splits` ranges of k and leaves float32 partial sums
+    part += ((size_t)blockIdx.y * M + (size_t)row_block * ROWS) * N;
     M = min(ROWS, M - row_block * ROWS);
+    const int slice_begin = blockIdx.y * slices_per_split, slice_end = min(k_steps, slice_begin + slices_per_split);
     const int tile0 = (col_group * WAVES + wave) * RT;
 
     f32x4 acc[RT][MT];
@@ -139,7 +143,7 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
     const bool ragged = (K & 127) != 0;
     auto copy_x = [&](int slice) {
         const uint32_t slot_base = xs_base + (uint32_t)(slice & 1) * (SLICE * 2);
-        if (ragged && slice == k_steps - 1) {
+        if (ragged && slice == k_steps - 1) {          // (the last slice of the last range)
             const int k = slice * 128 + x_col;
 #pragma unroll
             for (int e = 0; e < XI; ++e) {
@@ -202,22 +206,45 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
         });
     };
 
-    copy_x(0);
-    load_w(0, 0);
-    load_w(0, 1);
-    load_w(0, 2);
-    load_w(0, 3);
-    int slice = 0;
-    for (; slice + 1 < k_steps; ++slice) {
-        rows_wait_loads<4 * RT>();         // this wave's part of the slice of x has landed (behind it: 4 RT fragments)
-        __syncthreads();                   // everyone's has, and everyone has finished the slice before
-        copy_x(slice + 1);                 // into the slot that the slice before used
-        one_slice(slice, std::false_type{});
+    if (slice_begin < slice_end) {
+        copy_x(slice_begin);
+        load_w(slice_begin, 0);
+        load_w(slice_begin, 1);
+        load_w(slice_begin, 2);
+        load_w(slice_begin, 3);
+        int slice = slice_begin;
+        for (; slice + 1 < slice_end; ++slice) {
+            rows_wait_loads<4 * RT>();     // this wave's part of the slice of x has landed (behind it: 4 RT fragments)
+            __syncthreads();               // everyone's has, and everyone has finished the slice before
+            copy_x(slice + 1);             // into the slot that the slice before used
+            one_slice(slice, std::false_type{});
+        }
+        rows_wait_loads<4 * RT>();
+        __syncthreads();
+        one_slice(slice, std::true_type{});
     }
-    rows_wait_loads<4 * RT>();
-    __syncthreads();
-    one_slice(slice, std::true_type{});
 
+    if (splits > 1) {
+        // partial sums [split][row][column of W as tiled]: the pass that adds them knows a gated layout
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            const int n0 = (tile0 + t) * 16 + 4 * c;
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const int row = m * 16 + r;
+                if (row >= M) continue;
+                float* dst = part + (size_t)row * N + n0;
+                if (n0 + 3 < N && N % 4 == 0) {
+                    *reinterpret_cast<f32x4*>(dst) = acc[t][m];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (n0 + i < N) dst[i] = acc[t][m][i];
+                }
+            }
+        }
+        return;
+    }
     // lane holds y[m*16 + r][tile*16 + 4c + i]
     if (GATED) {
 #pragma unroll
@@ -266,12 +293,15 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
 }
 
 template <int RT, int WAVES, int MT, int MH>
-static int launch_rows(const bf16_t* x, const bf16_t* w, bf16_t* y, int M, int N, int K, int gated, hipStream_t s) {
-    const int n_tiles = (N + 15) / 16;
+static int launch_rows(const bf16_t* x, const bf16_t* w, bf16_t* y, float* part, int M, int N, int K, int gated,
+                       int splits, hipStream_t s) {
+    const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
     const long col_groups = (n_tiles + RT * WAVES - 1) / (RT * WAVES), row_blocks = (M + MT * 16 - 1) / (MT * 16);
     const long chunk = 2048 / (MT * 16);                     // as the kernel deals the row blocks out
     const long blocks = (col_groups + 7) / 8 * 8 * ((row_blocks + chunk - 1) / chunk * chunk);
     if (blocks > 2147483647L) return tli_fail("gemm_rows: too many workgroups");
+    const int slices_per_split = (k_steps + splits - 1) / splits;
+    const dim3 grid((unsigned)blocks, (unsigned)splits);
     const size_t lds = (size_t)2 * MT * 16 * 128 * sizeof(bf16_t);
     // (more than 64 KiB of LDS has to be allowed for a kernel once)
 #define ROWS_LAUNCH(G)                                                                                     \
@@ -284,31 +314,54 @@ static int launch_rows(const bf16_t* x, const bf16_t* w, bf16_t* y, int M, int N
                 return tli_fail("gemm_rows: cannot have %zu bytes of LDS", lds);                           \
             allowed = true;                                                                                \
         }                                                                                                  \
-        kernel<<<(unsigned)blocks, WAVES * 64, lds, s>>>(x, w, y, M, N, K);                                \
+        kernel<<<grid, WAVES * 64, lds, s>>>(x, w, y, part, M, N, K, splits, slices_per_split);            \
     }
     if (gated) ROWS_LAUNCH(true)
     else ROWS_LAUNCH(false)
 #undef ROWS_LAUNCH
-    return tli_check_launch("gemm_rows");
+    if (tli_check_launch("gemm_rows")) return 1;
+    if (splits > 1 && y) {
+        const size_t total = (size_t)M * (gated ? N / 2 : N);
+        gemm_mid_reduce_kernel<bf16_t><<<(unsigned)((total + 255) / 256), 256, 0, s>>>(part, y, M, N, splits, gated);
+        return tli_check_launch("gemm_rows: sum of the partial products");
+    }
+    return 0;
+}
+
+// How many ranges of k a product of this shape is cut into (the caller sizes `part` by it):
+// until there are about three workgroups for every four compute units, a range keeping at
+// least four slices of 128.
+extern "C" int tli_gemm_rows_splits(int M, int N, int K) {
+    const long col_groups = ((N + 15) / 16 + 15) / 16, row_blocks = (M + 127) / 128;
+    const int k_steps = (K + 127) / 128;
+    int splits = 1;
+    while (col_groups * row_blocks * splits < 192 && splits * 2 * 4 <= k_steps && splits < 16) splits *= 2;
+    return splits;
 }
 
 // y[M,N] = x[M,K] . W^T for any number of rows, bfloat16, W in the decode layout (`gated` as
-// tiled = 2 of tli_gemm_skinny_bf16: N counts gate and up, y is [M, N/2]).
+// tiled = 2 of tli_gemm_skinny_bf16: N counts gate and up, y is [M, N/2]).  `part`: splits*M*N
+// floats when splits > 1 (splits as returned by tli_gemm_rows_splits, or forced by the
+// caller); with y null the partial sums [splits][M][N] are left for the consumer to add
+// (tli_gemm_mid_reduce, or tli_add_rmsnorm).
 // cfg 0 or 2: 128 x 256 outputs a workgroup of four waves, two workgroups a compute unit (the
 // faster one in the model at 2,048 rows, measured on MI355X); 1: 256 x 256 outputs a workgroup
 // of eight waves.
-extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, int M, int N, int K, int gated, int cfg,
-                                  void* stream) {
+extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, float* part, int M, int N, int K,
+                                  int gated, int splits, int cfg, void* stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K <= 0 || K % 8) return tli_fail("gemm_rows: K = %d must be a positive multiple of 8", K);
     if (gated && N % 32) return tli_fail("gemm_rows: a gated product needs N %% 32 == 0");
-    if (!x || !w || !y) return tli_fail("gemm_rows: null operand");
-    if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 15) return tli_fail("gemm_rows: operands must be 16-byte aligned");
+    if (!x || !w) return tli_fail("gemm_rows: null operand");
+    if (splits < 1 || splits > 64) return tli_fail("gemm_rows: %d splits", splits);
+    if (splits > 1 && !part) return tli_fail("gemm_rows: splits need a buffer for partial sums");
+    if (!y && (splits < 2 || gated)) return tli_fail("gemm_rows: only a plain product with split k can leave its partial sums");
+    if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y | (uintptr_t)part) & 15) return tli_fail("gemm_rows: operands must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
     if (cfg == 0) cfg = 2;
     if ((size_t)M * K * sizeof(bf16_t) >= (1ull << 32) || (size_t)((N + 15) / 16 * 16) * ((K + 127) / 128 * 128) * sizeof(bf16_t) >= (1ull << 32))
         return tli_fail("gemm_rows: an operand of 4 GiB or more (offsets are 32 bits)");
-    if (cfg == 1) return launch_rows<2, 8, 16, 4>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, M, N, K, gated, s);
-    if (cfg == 2) return launch_rows<4, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, M, N, K, gated, s);
+    if (cfg == 1) return launch_rows<2, 8, 16, 4>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
+    if (cfg == 2) return launch_rows<4, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     return tli_fail("gemm_rows: unknown configuration %d", cfg);
 }

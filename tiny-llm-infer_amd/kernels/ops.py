@@ -83,7 +83,8 @@ def load_library():
         "tli_gemm_mid_bf16": [P, P, P, P, I, I, I, I, I, I, I, P],
         "tli_gemm_mid_splits": [I, I, I],
         "tli_gemm_mid_reduce": [P, P, I, I, I, I, P],
-        "tli_gemm_rows_bf16": [P, P, P, I, I, I, I, I, P],
+        "tli_gemm_rows_bf16": [P, P, P, P, I, I, I, I, I, I, P],
+        "tli_gemm_rows_splits": [I, I, I],
         "tli_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
         "tli_qkv_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I,
                                           F, I, I, I, P, I, P],
@@ -125,6 +126,7 @@ class HipOps:
     SKINNY_ROWS = 64
     MID_ROWS_FROM = 17           # from this many rows the x-sharing kernel multiplies,
     MID_ROWS_TO = 128            # up to this many
+    ROWS_UPTO = 0                # beyond MID_ROWS_TO and up to this many rows gemm_rows multiplies, then the library
     DECODE_WORKGROUPS = 512      # aim of the decode attention's key splitting
     DECODE_SPLIT_KEYS = 512      # a split walks at least this many keys
 
@@ -143,8 +145,10 @@ class HipOps:
         self.mid_cfg = 0             # measurements: launch shape and k ranges of the 17..128-row kernel
         self.mid_splits = 0
         self.skinny_cfg = 0          # measurements: force a launch shape of the weight-streaming kernel
-        self.own_products = False    # products of more than 128 rows through gemm_rows instead of the library
-        self.rows_cfg = 0            # measurements: force a launch shape of gemm_rows
+        self.own_products = False    # every product of more than 128 rows through gemm_rows instead of the library
+        self.rows_upto = self.ROWS_UPTO   # without own_products: gemm_rows up to this many rows
+        self.rows_cfg = 0            # measurements: force a launch shape and the k ranges of gemm_rows
+        self.rows_splits = 0
 
     def use_plain_kernels(self) -> None:
         """Every product, attention and norm through the plain kernels, bfloat16 too
@@ -305,8 +309,8 @@ class HipOps:
                                y[m0:m1].data_ptr(), m1 - m0, N, K, _dtype_code(out_dtype),
                                0 if tiled is None else 1, self.skinny_cfg, self._stream())
                 return y
-            if self.own_products and tiled is not None and out_dtype == torch.bfloat16:
-                return self._linear_rows(x, tiled, y, M, N, K, 0)
+            if self._rows_kernel(M) and tiled is not None and out_dtype == torch.bfloat16:
+                return self._linear_rows(x, tiled, y, M, N, K, 0, deferred or sums_only)
             # many rows (prefill): the library's matrix product, as the reference
             # uses its library for more than one row (kernels/src/matmul_kernel_cuda.cu:84-91)
             torch.matmul(x, w.t(), out=y)
@@ -359,12 +363,22 @@ class HipOps:
                    _ptr(part), M, N, K, _dtype_code(y.dtype), gated, splits, self.mid_cfg, self._stream())
         return DeferredSum(part, y.dtype) if leave else y
 
-    def _linear_rows(self, x, tiled, y, M, N, K, gated):
-        """Any number of rows from the decode layout (``own_products``): the kernel that
-        would let a model do without the row-major copy of its weights."""
-        self._call(self.lib.tli_gemm_rows_bf16, x.data_ptr(), tiled.data_ptr(), y.data_ptr(), M, N, K, gated,
-                   self.rows_cfg, self._stream())
-        return y
+    def _rows_kernel(self, M: int) -> bool:
+        """Whether a product of M > MID_ROWS_TO rows is gemm_rows' (else the library's)."""
+        return self.own_products or M <= self.rows_upto
+
+    def _linear_rows(self, x, tiled, y, M, N, K, gated, deferred=False):
+        """Any number of rows from the decode layout; k cut into ranges when the output
+        alone gives too few workgroups.  ``deferred``: the partial sums of the ranges are
+        left for the consumer to add."""
+        splits = self.rows_splits or self.lib.tli_gemm_rows_splits(M, N, K)
+        part = None
+        if splits > 1:
+            part = torch.empty((splits, M, N), dtype=torch.float32, device=self.device)
+        leave = deferred and splits > 1 and not gated
+        self._call(self.lib.tli_gemm_rows_bf16, x.data_ptr(), tiled.data_ptr(), None if leave else y.data_ptr(),
+                   _ptr(part), M, N, K, gated, splits, self.rows_cfg, self._stream())
+        return DeferredSum(part, y.dtype) if leave else y
 
     def linear_plain(self, x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None):
         """The plain tiled kernel for any sizes and dtypes: the reference beside the tuned ones."""
@@ -394,7 +408,7 @@ class HipOps:
             self._call(self.lib.tli_gemm_skinny_bf16, x.data_ptr(), gated.data_ptr(), y.data_ptr(), M,
                        2 * m.inter, K, BF16, 2, self.skinny_cfg if self.skinny_cfg >= 20 else 0, self._stream())
             return y
-        if gated is not None and self.own_products and x.dtype == torch.bfloat16 and K % 8 == 0:
+        if gated is not None and self._rows_kernel(M) and x.dtype == torch.bfloat16 and K % 8 == 0:
             self._want(x, "linear input", torch.bfloat16, (M, m.w.shape[1]))
             y = torch.empty((M, m.inter), dtype=x.dtype, device=self.device)
             return self._linear_rows(x, gated, y, M, 2 * m.inter, K, 1)
