@@ -344,9 +344,9 @@ extern "C" int tli_gemm_rows_splits(int M, int N, int K) {
 // floats when splits > 1 (splits as returned by tli_gemm_rows_splits, or forced by the
 // caller); with y null the partial sums [splits][M][N] are left for the consumer to add
 // (tli_gemm_mid_reduce, or tli_add_rmsnorm).
-// cfg 0 or 2: 128 x 256 outputs a workgroup of four waves, two workgroups a compute unit (the
-// faster one in the model at 2,048 rows, measured on MI355X); 1: 256 x 256 outputs a workgroup
-// of eight waves.
+// cfg 0 picks the launch shape; 1: 256 x 256 outputs a workgroup of eight waves, 2: 128 x 256
+// and four waves, two workgroups a compute unit, 3: 128 x 512 and eight waves; cfg >= 10: the
+// tens for a gated product, the ones for the others (measurements).
 extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, float* part, int M, int N, int K,
                                   int gated, int splits, int cfg, void* stream) {
     if (M <= 0 || N <= 0) return 0;
@@ -358,10 +358,18 @@ extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, float* 
     if (!y && (splits < 2 || gated)) return tli_fail("gemm_rows: only a plain product with split k can leave its partial sums");
     if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y | (uintptr_t)part) & 15) return tli_fail("gemm_rows: operands must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
-    if (cfg == 0) cfg = 2;
     if ((size_t)M * K * sizeof(bf16_t) >= (1ull << 32) || (size_t)((N + 15) / 16 * 16) * ((K + 127) / 128 * 128) * sizeof(bf16_t) >= (1ull << 32))
         return tli_fail("gemm_rows: an operand of 4 GiB or more (offsets are 32 bits)");
-    if (cfg == 1) return launch_rows<2, 8, 16, 4>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
+    if (cfg >= 10) cfg = gated ? cfg / 10 : cfg % 10;       // measurements: one shape for the gated product, one for the others
+    if (cfg == 0) {
+        // 128 x 512 outputs a workgroup (one a compute unit) ask the L2 caches for a sixth less
+        // than 128 x 256 (two a compute unit): taken when its workgroups fill their last round of
+        // the 256 compute units to 85% at least
+        const long wide = (long)(((N + 15) / 16 + 31) / 32) * ((M + 127) / 128);
+        cfg = splits == 1 && wide * 100 >= (wide + 255) / 256 * 256 * 85 ? 3 : 2;
+    }
+    if (cfg == 1) return launch_rows<2, 8, 16, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     if (cfg == 2) return launch_rows<4, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
+    if (cfg == 3) return launch_rows<4, 8, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     return tli_fail("gemm_rows: unknown configuration %d", cfg);
 }
