@@ -339,6 +339,14 @@ extern "C" int tli_gemm_rows_splits(int M, int N, int K) {
     return splits;
 }
 
+// The launch shape that cfg 0 takes: 128 x 512 outputs a workgroup (one a compute unit) ask the
+// L2 caches for a sixth less than 128 x 256 (two a compute unit); taken when its workgroups
+// fill their last round of the 256 compute units to 85% at least and k is not cut.
+static int rows_pick(int M, int N, int splits) {
+    const long wide = (long)(((N + 15) / 16 + 31) / 32) * ((M + 127) / 128);
+    return splits == 1 && wide * 100 >= (wide + 255) / 256 * 256 * 85 ? 3 : 2;
+}
+
 // y[M,N] = x[M,K] . W^T for any number of rows, bfloat16, W in the decode layout (`gated` as
 // tiled = 2 of tli_gemm_skinny_bf16: N counts gate and up, y is [M, N/2]).  `part`: splits*M*N
 // floats when splits > 1 (splits as returned by tli_gemm_rows_splits, or forced by the
@@ -361,13 +369,7 @@ extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, float* 
     if ((size_t)M * K * sizeof(bf16_t) >= (1ull << 32) || (size_t)((N + 15) / 16 * 16) * ((K + 127) / 128 * 128) * sizeof(bf16_t) >= (1ull << 32))
         return tli_fail("gemm_rows: an operand of 4 GiB or more (offsets are 32 bits)");
     if (cfg >= 10) cfg = gated ? cfg / 10 : cfg % 10;       // measurements: one shape for the gated product, one for the others
-    if (cfg == 0) {
-        // 128 x 512 outputs a workgroup (one a compute unit) ask the L2 caches for a sixth less
-        // than 128 x 256 (two a compute unit): taken when its workgroups fill their last round of
-        // the 256 compute units to 85% at least
-        const long wide = (long)(((N + 15) / 16 + 31) / 32) * ((M + 127) / 128);
-        cfg = splits == 1 && wide * 100 >= (wide + 255) / 256 * 256 * 85 ? 3 : 2;
-    }
+    if (cfg == 0) cfg = rows_pick(M, N, splits);
     if (cfg == 1) return launch_rows<2, 8, 16, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     if (cfg == 2) return launch_rows<4, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     if (cfg == 3) return launch_rows<4, 8, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);

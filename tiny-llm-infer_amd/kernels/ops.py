@@ -126,7 +126,6 @@ class HipOps:
     SKINNY_ROWS = 64
     MID_ROWS_FROM = 17           # from this many rows the x-sharing kernel multiplies,
     MID_ROWS_TO = 128            # up to this many
-    ROWS_UPTO = 0                # beyond MID_ROWS_TO and up to this many rows gemm_rows multiplies, then the library
     DECODE_WORKGROUPS = 512      # aim of the decode attention's key splitting
     DECODE_SPLIT_KEYS = 512      # a split walks at least this many keys
 
@@ -146,7 +145,6 @@ class HipOps:
         self.mid_splits = 0
         self.skinny_cfg = 0          # measurements: force a launch shape of the weight-streaming kernel
         self.own_products = False    # every product of more than 128 rows through gemm_rows instead of the library
-        self.rows_upto = self.ROWS_UPTO   # without own_products: gemm_rows up to this many rows
         self.rows_cfg = 0            # measurements: force a launch shape and the k ranges of gemm_rows
         self.rows_splits = 0
 
@@ -309,7 +307,7 @@ class HipOps:
                                y[m0:m1].data_ptr(), m1 - m0, N, K, _dtype_code(out_dtype),
                                0 if tiled is None else 1, self.skinny_cfg, self._stream())
                 return y
-            if self._rows_kernel(M) and tiled is not None and out_dtype == torch.bfloat16:
+            if self.own_products and tiled is not None and out_dtype == torch.bfloat16:
                 return self._linear_rows(x, tiled, y, M, N, K, 0, deferred or sums_only)
             # many rows (prefill): the library's matrix product, as the reference
             # uses its library for more than one row (kernels/src/matmul_kernel_cuda.cu:84-91)
@@ -363,10 +361,6 @@ class HipOps:
                    _ptr(part), M, N, K, _dtype_code(y.dtype), gated, splits, self.mid_cfg, self._stream())
         return DeferredSum(part, y.dtype) if leave else y
 
-    def _rows_kernel(self, M: int) -> bool:
-        """Whether a product of M > MID_ROWS_TO rows is gemm_rows' (else the library's)."""
-        return self.own_products or M <= self.rows_upto
-
     def _linear_rows(self, x, tiled, y, M, N, K, gated, deferred=False):
         """Any number of rows from the decode layout; k cut into ranges when the output
         alone gives too few workgroups.  ``deferred``: the partial sums of the ranges are
@@ -408,7 +402,7 @@ class HipOps:
             self._call(self.lib.tli_gemm_skinny_bf16, x.data_ptr(), gated.data_ptr(), y.data_ptr(), M,
                        2 * m.inter, K, BF16, 2, self.skinny_cfg if self.skinny_cfg >= 20 else 0, self._stream())
             return y
-        if gated is not None and self._rows_kernel(M) and x.dtype == torch.bfloat16 and K % 8 == 0:
+        if gated is not None and self.own_products and x.dtype == torch.bfloat16 and K % 8 == 0:
             self._want(x, "linear input", torch.bfloat16, (M, m.w.shape[1]))
             y = torch.empty((M, m.inter), dtype=x.dtype, device=self.device)
             return self._linear_rows(x, gated, y, M, 2 * m.inter, K, 1)
