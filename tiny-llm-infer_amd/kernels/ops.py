@@ -128,7 +128,7 @@ class HipOps:
     MID_ROWS_TO = 128            # up to this many
     DECODE_WORKGROUPS = 256      # aim of the decode attention's key splitting: one workgroup a compute unit (measured
                                  # against 128, 192 and 512 at batch 1 to 64 and 128 to 30,000 keys: up to 10% over 512)
-    DECODE_SPLIT_KEYS = 512      # a split walks at least this many keys
+    DECODE_SPLIT_KEYS = 512      # a split walks at least this many keys (128, 256 and 1024 measured: no better)
 
     def __init__(self, device):
         self.device = torch.device(device)
