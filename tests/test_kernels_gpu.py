@@ -330,6 +330,10 @@ ATT_CASES = [
     # one row per sequence (decode), long enough for the keys to be split over workgroups
     (32, 8, 128, 16, [1500, 40, 129, 1, 640], [1, 1, 1, 1, 1], None),
     (8, 8, 64, 16, [130, 257], [1, 1], 19),
+    # few rows with many keys, split over few workgroups
+    (32, 8, 128, 16, [3000], [1], None),
+    (8, 2, 128, 16, [700, 2100, 513], [1, 1, 1], None),
+    (16, 4, 64, 8, [5000, 1200], [1, 1], 700),
     (5, 1, 48, 32, [300, 64], [1, 1], 100),
     (32, 1, 32, 8, [70, 3], [1, 1], None),        # 32 heads on one kv head: two head tiles
     (32, 1, 32, 4, [70], [9], None),
@@ -477,6 +481,7 @@ RAW_CASES = [
     # heads, kv_heads, head_dim, norms, rotation, page, seq_lens, new rows, window, writes
     (32, 8, 128, True, True, 16, [1500, 40, 129, 1, 640], [1] * 5, None, True),     # decode, keys split over workgroups
     (8, 8, 64, True, True, 8, [130, 257, 16, 17], [1] * 4, 19, True),
+    (32, 8, 128, True, True, 16, [2000, 600], [1, 1], None, True),                  # few rows, many keys
     (5, 1, 256, False, True, 16, [90, 33], [1, 1], None, True),
     (6, 2, 192, True, False, 4, [70, 5], [1, 1], 64, True),
     (16, 1, 64, True, True, 16, [48, 1], [1, 1], None, False),                      # reads another layer's cache
