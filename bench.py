@@ -61,7 +61,8 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiles)")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement (for profiles)")
     ap.add_argument("--own-products", action="store_true",
-                    help="products of more than 128 rows by this library's kernel instead of the BLAS library")
+                    help="every product of more than 128 rows by this library's kernel (default: the faster one for the shape)")
+    ap.add_argument("--library-products", action="store_true", help="... by the BLAS library")
     ap.add_argument("--rows-cfg", type=int, default=0, help="with --own-products: force a launch shape (measurements)")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
@@ -87,7 +88,8 @@ def main():
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
     t0 = time.time()
     model = random_model("Qwen3ForCausalLM", cfg, args.seed, args.dtype, "cuda:0", args.context)
-    model.env.ops.own_products = args.own_products
+    if args.own_products or args.library_products:
+        model.env.ops.many_rows = "own" if args.own_products else "library"
     model.env.ops.rows_cfg = args.rows_cfg
     torch.cuda.synchronize()
     print(f"[bench] model with {layers} layers on the device in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)

@@ -214,17 +214,57 @@ def test_gated_product_of_many_rows(ops, mki, cfg):
     gate, up = rnd((inter, K), torch.bfloat16, 4, 0.1).to(DEV), rnd((inter, K), torch.bfloat16, 5, 0.1).to(DEV)
     m = GatedMatrix(gate, up, BuildEnv(dtype=torch.bfloat16, device=torch.device(DEV), ops=ops, max_model_len=64))
     g, u = x.double().cpu() @ gate.double().cpu().t(), x.double().cpu() @ up.double().cpu().t()
-    ops.own_products, ops.rows_cfg = True, cfg
+    ops.many_rows, ops.rows_cfg = "own", cfg
     try:
         for splits in (1, 0, 4):
             ops.rows_splits = splits
             close(ops.linear_swiglu(x, m), g / (1 + torch.exp(-g)) * u, torch.bfloat16, f"gated product, {splits} ranges of k")
         y = ops.linear_swiglu(x, m)
     finally:
-        ops.own_products, ops.rows_cfg, ops.rows_splits = False, 0, 0
+        ops.many_rows, ops.rows_cfg, ops.rows_splits = "measure", 0, 0
     g, u = x.double().cpu() @ gate.double().cpu().t(), x.double().cpu() @ up.double().cpu().t()
     close(y, g / (1 + torch.exp(-g)) * u, torch.bfloat16, "gated product of many rows")
-    close(ops.linear_swiglu(x, m), g / (1 + torch.exp(-g)) * u, torch.bfloat16, "the library and the activation")
+    ops.many_rows = "library"
+    try:
+        close(ops.linear_swiglu(x, m), g / (1 + torch.exp(-g)) * u, torch.bfloat16, "the library and the activation")
+    finally:
+        ops.many_rows = "measure"
+
+
+def test_products_of_many_rows_take_the_faster_kernel(ops):
+    """By default a product of more than 128 rows is timed in gemm_rows and in the library when
+    its shape first comes up, and goes to the faster one from then on (the same one for every
+    number of rows in the same 128): the result is right whichever that is, nothing is timed
+    during a graph capture, and a shape met there first goes to the library."""
+    from tiny_llm_infer_amd.parts.base import BuildEnv
+    from tiny_llm_infer_amd.parts.linear import GatedMatrix, Matrix
+    env = BuildEnv(dtype=torch.bfloat16, device=torch.device(DEV), ops=ops, max_model_len=64)
+    ops.measured.clear()
+    M, N, K = 1000, 1024, 512
+    x, w = rnd((M, K), torch.bfloat16, 1).to(DEV), rnd((N, K), torch.bfloat16, 2, 0.05).to(DEV)
+    m = Matrix(w, env)
+    want = x.double().cpu() @ w.double().cpu().t()
+    close(ops.linear(x, m), want, torch.bfloat16, "product while its shape is measured")
+    assert list(ops.measured) == [(8, N, K, 0)]
+    first = ops.linear(x, m)
+    close(first, want, torch.bfloat16, "product after")
+    assert torch.equal(first, ops.linear(x, m)) and torch.equal(first[:900], ops.linear(x[:900].contiguous(), m))
+    gm = GatedMatrix(rnd((256, K), torch.bfloat16, 3, 0.1).to(DEV), rnd((256, K), torch.bfloat16, 4, 0.1).to(DEV), env)
+    g, u = x.double().cpu() @ gm.w[:256].double().cpu().t(), x.double().cpu() @ gm.w[256:].double().cpu().t()
+    close(ops.linear_swiglu(x, gm), g / (1 + torch.exp(-g)) * u, torch.bfloat16, "gated product while measured")
+    assert (8, 512, K, 1) in ops.measured
+    # a shape that first comes up under capture is not measured
+    x2 = rnd((300, K), torch.bfloat16, 5).to(DEV)
+    ops.linear(x2[:10].contiguous(), m)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = ops.linear(x2, m)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert (3, N, K, 0) not in ops.measured
+    close(y, x2.double().cpu() @ w.double().cpu().t(), torch.bfloat16, "product recorded before its shape was measured")
+    ops.measured.clear()
 
 
 def test_library_linear_for_many_rows(ops):

@@ -185,7 +185,7 @@ def test_real_layer_sizes(tmp_path, sizes):
             runner.cache.check()
     # bfloat16 once more with the products of more than 128 rows (the whole prompt of 150 tokens, and
     # the 118 + 32 of "decode" is below) through this library's own kernel instead of the BLAS library
-    model.env.ops.own_products = True
+    model.env.ops.many_rows = "own"
     steps = trace_whole(reqs)
     runner = ModelRunner(model, model.env, page_size=16, num_pages=24, max_requests=4, max_batch_tokens=512)
     worst = _check(collect(steps, _replay(runner, steps)), want, "bfloat16", f"{sizes['hidden_size']} wide/own products")

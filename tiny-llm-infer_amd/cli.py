@@ -36,9 +36,10 @@ def _common(ap: argparse.ArgumentParser) -> None:
                     help="with --config: draw seeded random weights instead of reading a checkpoint")
     ap.add_argument("--config", help="a config.json, for --random-weights")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--kernels", default="tuned", choices=["tuned", "plain", "own-products"],
-                    help="plain: the simple twins of the tuned kernels (bfloat16 too); own-products: "
-                         "matrix products of more than 128 rows by this library's kernel instead of the BLAS library")
+    ap.add_argument("--kernels", default="tuned", choices=["tuned", "plain", "own-products", "library-products"],
+                    help="plain: the simple twins of the tuned kernels (bfloat16 too); own-products / library-products: "
+                         "every matrix product of more than 128 rows by this library's kernel / by the BLAS library "
+                         "(tuned: the faster one for the shape, timed when the shape first comes up)")
 
 
 def _device(name: str) -> str:
@@ -278,9 +279,10 @@ def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
     ap.add_argument("--max-live", type=int, default=4, help="most requests live at a time")
     ap.add_argument("--max-step-tokens", type=int, default=8192, help="most tokens in one step")
     ap.add_argument("--device", default="cuda:0")
-    ap.add_argument("--kernels", default="tuned", choices=["tuned", "plain", "own-products"],
-                    help="plain: the simple twins of the tuned kernels (bfloat16 too); own-products: "
-                         "matrix products of more than 128 rows by this library's kernel instead of the BLAS library")
+    ap.add_argument("--kernels", default="tuned", choices=["tuned", "plain", "own-products", "library-products"],
+                    help="plain: the simple twins of the tuned kernels (bfloat16 too); own-products / library-products: "
+                         "every matrix product of more than 128 rows by this library's kernel / by the BLAS library "
+                         "(tuned: the faster one for the shape, timed when the shape first comes up)")
     args = ap.parse_args(argv)
     if 64 % args.page_size:
         ap.error("--page-size must divide 64")
@@ -301,11 +303,13 @@ def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
 
 def _kernels(model, which: str) -> None:
     """--kernels plain: every product, attention and norm through the plain kernels;
-    own-products: products of many rows through gemm_rows instead of the BLAS library."""
+    own-products / library-products: products of many rows always through gemm_rows / the BLAS library."""
     if which == "plain":
         model.env.ops.use_plain_kernels()
     elif which == "own-products":
-        model.env.ops.own_products = True
+        model.env.ops.many_rows = "own"
+    elif which == "library-products":
+        model.env.ops.many_rows = "library"
 
 
 USAGE = """usage: model_main --infer [options] | --bench [options] | --replay [options]

@@ -257,8 +257,11 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
                 float o[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
+                    // silu(g) * u with the hardware's exp2 and reciprocal (1 ulp each; the result is rounded to
+                    // bfloat16): the library routines would cost more vector instructions here than the
+                    // workgroup's MFMAs
                     const float g = acc[t][m][i], u = acc[t + 1][m][i];
-                    o[i] = g / (1.0f + expf(-g)) * u;
+                    o[i] = g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g)) * u;
                 }
                 bf16_t* dst = y + (size_t)row * n_out + n0;
                 if (n0 + 3 < n_out && n_out % 4 == 0) {

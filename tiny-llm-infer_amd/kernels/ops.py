@@ -145,7 +145,10 @@ class HipOps:
         self.mid_cfg = 0             # measurements: launch shape and k ranges of the 17..128-row kernel
         self.mid_splits = 0
         self.skinny_cfg = 0          # measurements: force a launch shape of the weight-streaming kernel
-        self.own_products = False    # every product of more than 128 rows through gemm_rows instead of the library
+        # Products of more than 128 rows: "measure" = the faster of gemm_rows and the BLAS library for
+        # the shape, timed once when the shape first comes up; "own" / "library" = always that one
+        self.many_rows = "measure"
+        self.measured = {}           # (rows rounded up to 128, N, K, gated) -> True where gemm_rows won
         self.rows_cfg = 0            # measurements: force a launch shape and the k ranges of gemm_rows
         self.rows_splits = 0
 
@@ -308,7 +311,7 @@ class HipOps:
                                y[m0:m1].data_ptr(), m1 - m0, N, K, _dtype_code(out_dtype),
                                0 if tiled is None else 1, self.skinny_cfg, self._stream())
                 return y
-            if self.own_products and tiled is not None and out_dtype == torch.bfloat16:
+            if tiled is not None and out_dtype == torch.bfloat16 and self._rows_kernel_wins(x, w, tiled, M, N, K, 0):
                 return self._linear_rows(x, tiled, y, M, N, K, 0, deferred or sums_only)
             # many rows (prefill): the library's matrix product, as the reference
             # uses its library for more than one row (kernels/src/matmul_kernel_cuda.cu:84-91)
@@ -362,6 +365,46 @@ class HipOps:
                    _ptr(part), M, N, K, _dtype_code(y.dtype), gated, splits, self.mid_cfg, self._stream())
         return DeferredSum(part, y.dtype) if leave else y
 
+    def _rows_kernel_wins(self, x, w, tiled, M, N, K, gated) -> bool:
+        """Whether this product of more than 128 rows goes to gemm_rows (else to the library).
+        Which one is faster changes with the shape by more than 10% either way (how well each
+        one's tiles fill the compute units), so both are timed when a shape first comes up:
+        three runs each after one to warm up, a few milliseconds, outside any graph capture."""
+        if self.many_rows != "measure":
+            return self.many_rows == "own"
+        key = ((M + 127) // 128, N, K, gated)
+        won = self.measured.get(key)
+        if won is not None:
+            return won
+        if torch.cuda.is_current_stream_capturing():
+            return False                      # (nothing can be timed now; the shape is measured when it next comes up eagerly)
+        y = torch.empty((M, N // 2 if gated else N), dtype=torch.bfloat16, device=self.device)
+        wide = torch.empty((M, N), dtype=torch.bfloat16, device=self.device) if gated else None
+
+        def library():
+            if gated:
+                torch.matmul(x, w.t(), out=wide)
+                self.swiglu(wide)
+            else:
+                torch.matmul(x, w.t(), out=y)
+
+        def own():
+            self._linear_rows(x, tiled, y, M, N, K, gated)
+
+        times = []
+        for fn in (library, own):
+            fn()
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(3):
+                fn()
+            stop.record()
+            stop.synchronize()
+            times.append(start.elapsed_time(stop))
+        won = times[1] < times[0]
+        self.measured[key] = won
+        return won
+
     def _linear_rows(self, x, tiled, y, M, N, K, gated, deferred=False):
         """Any number of rows from the decode layout; k cut into ranges when the output
         alone gives too few workgroups.  ``deferred``: the partial sums of the ranges are
@@ -403,7 +446,8 @@ class HipOps:
             self._call(self.lib.tli_gemm_skinny_bf16, x.data_ptr(), gated.data_ptr(), y.data_ptr(), M,
                        2 * m.inter, K, BF16, 2, self.skinny_cfg if self.skinny_cfg >= 20 else 0, self._stream())
             return y
-        if gated is not None and self.own_products and x.dtype == torch.bfloat16 and K % 8 == 0:
+        if (gated is not None and x.dtype == torch.bfloat16 and K % 8 == 0
+                and self._rows_kernel_wins(x, m.w, gated, M, 2 * m.inter, K, 1)):
             self._want(x, "linear input", torch.bfloat16, (M, m.w.shape[1]))
             y = torch.empty((M, m.inter), dtype=x.dtype, device=self.device)
             return self._linear_rows(x, gated, y, M, 2 * m.inter, K, 1)
