@@ -372,6 +372,8 @@ class HipOps:
         three runs each after one to warm up, a few milliseconds, outside any graph capture."""
         if self.many_rows != "measure":
             return self.many_rows == "own"
+        if max(M, N + 15) * (K + 127) * 2 >= 1 << 32:
+            return False                      # gemm_rows keeps 32-bit offsets into its operands
         key = ((M + 127) // 128, N, K, gated)
         won = self.measured.get(key)
         if won is not None:
