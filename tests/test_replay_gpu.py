@@ -236,3 +236,40 @@ def test_selective_attention_through_every_cut(model_folders, tmp_path, name):
         plain = worst(collect(steps, _replay(runner, steps)))
         print(f"selective {name} bfloat16 {cut}: tuned {tuned:.2e}, plain kernels {plain:.2e}")
         assert tuned <= 1.5 * plain + 0.1 * TOL["bfloat16"], (cut, tuned, plain)
+
+
+@pytest.mark.parametrize("batch", [40, 140])
+def test_many_rows_decoded_together_at_real_width(tmp_path, batch):
+    """40 and 140 requests at the width of Qwen3-8B (one layer): prompts in two steps of many
+    rows, then every request's last tokens one by one, all requests in one step: the products
+    for 17..128 rows with their partial sums, those for more rows, the recorded decode steps."""
+    from tiny_llm_infer_amd.config import Qwen3Config
+    from tiny_llm_infer_amd.engine.loading import load_model, write_random_model
+    from tiny_llm_infer_amd.engine.runner import ModelRunner, StepEntry
+    cfg = Qwen3Config.from_dict(dict(
+        architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=1, head_dim=128, vocab_size=1024,
+        max_position_embeddings=4096, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False, hidden_size=4096,
+        intermediate_size=12288, num_attention_heads=32, num_key_value_heads=8))
+    folder = write_random_model(str(tmp_path / "wide"), "Qwen3ForCausalLM", cfg, seed=3)
+    rng = np.random.default_rng(batch)
+    reqs = {f"r{i}": random_prompt(1024, int(n), 50 * batch + i) for i, n in enumerate(rng.integers(12, 50, batch))}
+    want = plain_logits(folder, reqs)
+    model, _ = load_model(folder, "bfloat16", "cuda:0")
+    runner = ModelRunner(model, model.env, page_size=16, num_pages=batch * 4, max_requests=batch, max_batch_tokens=8192)
+    ids, keep = list(reqs), 4
+    for rid in ids:
+        runner.admit(rid)
+    for part in (ids[:batch // 2], ids[batch // 2:]):
+        runner.step([StepEntry(r, reqs[r][:-keep], []) for r in part])
+    worst = 0.0
+    for t in range(keep):
+        out = runner.step([StepEntry(r, [reqs[r][len(reqs[r]) - keep + t]], [0]) for r in ids]).float().cpu().numpy()
+        for i, r in enumerate(ids):
+            w = want[r][len(reqs[r]) - keep + t]
+            worst = max(worst, float(np.abs(out[i] - w).max() / np.abs(w).max()))
+    print(f"{batch} rows decoded together: worst relative error {worst:.2e}")
+    assert worst <= TOL["bfloat16"]
+    assert runner.graph_replays == keep
+    for rid in ids:
+        runner.release(rid)
+    runner.cache.check()
