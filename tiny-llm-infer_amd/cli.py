@@ -248,7 +248,8 @@ def run_benchmark(argv: List[str]) -> int:
               f"median_{what}_tokens_per_second={statistics.median(rates):.2f}")
     st = engine.stats()
     print(f"engine_steps={st['steps']} preemptions={st['preemptions']} "
-          f"pages_free={min(st['pages_free'])}/{st['pages']} prefix_pages_reused={st['prefix_pages_reused']}",
+          f"pages_free={min(st['pages_free'])}/{st['pages']} prefix_pages_reused={st['prefix_pages_reused']} "
+          f"product_shapes_own_kernel={st['product_shapes_own_kernel']}/{st['product_shapes_measured']}",
           file=sys.stderr)
     return 0
 
