@@ -152,3 +152,24 @@ def test_requests_that_arrive_while_others_are_served(model_folders):
         assert [r.token_ids for r in got] == want
         assert [r.prompt_token_ids for r in got] == prompts
         eng.runner.cache.check()
+
+
+def test_step_ahead_counts_the_pages_of_the_whole_batch(model_folders):
+    """Equal-length prompts cross a page border in the same step.  With a pool two pages
+    short, the step planned ahead must see that its requests compete for the same free
+    pages, take none, and leave the decision to the ordinary path (which preempts):
+    the tokens are those of the engine without steps ahead, and no page is lost."""
+    folder = model_folders["A"]
+    cfg, w = plain_qwen3.read_model(folder)
+    prompts = [random_prompt(256, 8, 90 + i) for i in range(3)]
+    want = [plain_qwen3.greedy(cfg, w, p, 6) for p in prompts]
+    outs = []
+    for ahead in (False, True):
+        eng = _engine(folder, "A", num_kv_blocks=5)
+        eng.lookahead = ahead
+        got = eng.generate(prompts, SamplingParams(max_tokens=6, ignore_eos=True))
+        outs.append([r.token_ids for r in got])
+        assert eng.scheduler.num_preemptions > 0
+        eng.runner.cache.check()
+        assert eng.runner.cache.free_pages() == [5] and eng.is_finished()
+    assert outs[0] == outs[1] == want

@@ -90,15 +90,20 @@ class Scheduler:
         if any(not item.samples or item.sequence.status == Status.FINISHED for item in plan.sequences):
             return None
         ahead = BatchPlan()
+        need = [0] * len(self.cache.groups)
         for item in plan.sequences:
             seq = item.sequence
             if seq.completion_size + 1 >= seq.sampling.max_tokens:
                 continue                      # the running step's token is its last
             # seq.size does not count the running step's token yet: that token goes to position seq.size
-            if not self.cache.can_reserve(seq.request_id, seq.size + 1):
-                return None                   # pages run out: the ordinary path decides whom to preempt
+            for g, n in enumerate(self.cache.pages_needed(seq.request_id, seq.size + 1)):
+                need[g] += n
             ahead.sequences.append(ScheduledSequence(seq, seq.size, 1, False))
         if not ahead.sequences or len(ahead.sequences) > self.config.max_num_seqs:
+            return None
+        # the requests compete for the same pools: the whole step's pages must be free, or
+        # nothing is taken and the ordinary path decides whom to preempt
+        if any(n > g.pool.free_count for n, g in zip(need, self.cache.groups)):
             return None
         for item in ahead.sequences:
             self.cache.reserve(item.sequence.request_id, item.token_start + 1)
