@@ -7,6 +7,8 @@
 // Philox keyed by the thread index; here u_v is a hash of (seed, v) alone, so
 // the draw does not depend on the launch shape or on the batch.
 #include "common.h"
+#include "no_alloc.h"
+#include <mutex>
 
 #define SAMPLE_THREADS 1024
 
@@ -164,8 +166,56 @@ extern "C" int tli_sample(const float* logits, int rows, int vocab, const float*
     return tli_check_launch("sample");
 }
 
-// the same draw on the host, for tests and for callers that hold logits there
 extern "C" int tli_sample_scratch_bytes(int rows) { return rows * SAMPLE_CHUNKS * 8; }
+
+// ---- the same sampling for callers that cannot allocate ---------------------------------
+// The pieces' best scores and ids (what tli_sample takes as `scratch`) live in this array
+// instead: TLI_SAMPLE_NO_ALLOC_MAX_ROWS * SAMPLE_CHUNKS * 8 bytes = 256 KiB on every GPU the
+// library runs on, held until the process ends.  In host code the array's name is only a
+// stand-in for the symbol; the address of each GPU's copy is asked for once, with that GPU
+// current, and kept.  (No `used` attribute on it: that would keep the device symbol local
+// to its code object, where the runtime cannot find it by name; the use in host code below
+// is what keeps it.)
+static __device__ __align__(256) unsigned char
+    scratch[(size_t)TLI_SAMPLE_NO_ALLOC_MAX_ROWS * SAMPLE_CHUNKS * 8];
+
+#define TLI_MAX_DEVICES 64
+static void* g_scratch_of_device[TLI_MAX_DEVICES];
+static std::mutex g_scratch_lock;
+
+static int scratch_of_current_device(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return tli_fail("sample_no_alloc: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= TLI_MAX_DEVICES) return tli_fail("sample_no_alloc: device %d is beyond the %d this library keeps scratch for", dev, TLI_MAX_DEVICES);
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (!g_scratch_of_device[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return tli_fail("sample_no_alloc: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_of_device[dev] = p;
+    }
+    *ptr = g_scratch_of_device[dev];
+    return 0;
+}
+
+extern "C" int tli_sample_no_alloc(const float* logits, int rows, int vocab, const float* temperatures,
+                                   const uint32_t* seeds, const float* top_p, int* out, void* stream) {
+    if (rows <= 0) return 0;
+    if (rows > TLI_SAMPLE_NO_ALLOC_MAX_ROWS)
+        return tli_fail("sample_no_alloc: %d rows, the scratch array of this entry point holds %d",
+                        rows, TLI_SAMPLE_NO_ALLOC_MAX_ROWS);
+    void* ptr = nullptr;
+    if (scratch_of_current_device(&ptr)) return 1;
+    // nothing in the array has to start at zero: the first pass writes every (row, piece)
+    // entry that the second pass reads
+    return tli_sample(logits, rows, vocab, temperatures, seeds, top_p, out, ptr, stream);
+}
+
+extern "C" int tli_sample_no_alloc_max_rows() { return TLI_SAMPLE_NO_ALLOC_MAX_ROWS; }
+
+// the same draw on the host, for tests and for callers that hold logits there
 
 extern "C" float tli_sample_uniform(uint32_t seed_lo, uint32_t seed_hi, uint32_t token) {
     return tli_uniform(seed_lo, seed_hi, token);
