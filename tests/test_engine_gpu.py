@@ -285,3 +285,43 @@ def test_prefix_caching_on_the_gpu(model_folders):
             assert [r.token_ids for r in got] == [r.token_ids for r in plain]
         assert eng.runner.cache.prefix_hits == 14
         eng.runner.cache.check()
+
+
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_a_request_that_ends_while_its_next_step_is_on_the_device(model_folders, name):
+    """An end-of-sequence token stops one request of a batch in the middle of a run while the
+    step after it is already on the device (fed on the device, replayed from its recording in
+    bfloat16) and writes into pages that are given back meanwhile: the tokens are those of the
+    engine that launches nothing ahead, the request stops where the plain greedy run meets the
+    token, and no page is lost."""
+    from tiny_llm_infer_amd.sampling.params import SamplingParams
+    folder = model_folders[name]
+    cfg, w = plain_qwen3.read_model(folder)
+    vocab = TINY[name]["vocab_size"]
+    prompts = [random_prompt(vocab, n, 60 + n) for n in (6, 19, 11, 27)]
+    for dtype in ("float32", "bfloat16"):
+        free = _engine(folder, name, dtype, max_num_batched_tokens=64)
+        free.lookahead = False
+        runs = [r.token_ids for r in free.generate(prompts, SamplingParams(max_tokens=14, ignore_eos=True))]
+        eos = runs[1][5]                                  # request 1 meets it at its 6th token at the latest
+        outs = []
+        for ahead in (False, True):
+            eng = _engine(folder, name, dtype, max_num_batched_tokens=64)
+            eng.lookahead = ahead
+            eng.eos_token_ids = {eos}
+            outs.append([r.token_ids for r in eng.generate(prompts, SamplingParams(max_tokens=14))])
+            assert (eng.num_steps_ahead > 3) == ahead
+            if ahead and dtype == "bfloat16":
+                assert eng.runner.graph_replays > 3
+            eng.runner.cache.check()
+            assert eng.is_finished() and all(f == 64 for f in eng.runner.cache.free_pages())
+            # and the engine serves again afterwards from the pages that were given back
+            again = [r.token_ids for r in eng.generate(prompts[:2], SamplingParams(max_tokens=14))]
+            assert again == outs[-1][:2]
+        assert outs[0] == outs[1]
+        for run, got in zip(runs, outs[1]):               # each request is its free run cut after the token
+            cut = run.index(eos) + 1 if eos in run else len(run)
+            assert got == run[:cut]
+        assert len(outs[1][1]) <= 6
+        if dtype == "float32":
+            assert runs == [plain_qwen3.greedy(cfg, w, p, 14) for p in prompts]

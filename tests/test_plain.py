@@ -142,3 +142,67 @@ def test_q_and_k_norms_act_per_head_before_the_rotation():
     w3 = dict(w)
     w3["model.layers.0.self_attn.v_proj.weight"] = w["model.layers.0.self_attn.v_proj.weight"] * 7.0
     assert not torch.allclose(P.forward(cfg, w3, ids), base, atol=1e-3)
+
+
+# ---- the wiring of a layer around the residual stream ---------------------------------
+# (model/src/qwen3_paged_batch.cpp:146-148, 273-279, 297-307: n = norm(h); r = h + attn(n);
+# m = norm(r); h' = r + mlp(m); after the last layer norm(h) and the head)
+def _library_attention(n, w, p, cfg, T):
+    """The attention branch of one layer from library routines; positions 0..T-1."""
+    H, G, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    q = F.rms_norm(F.linear(n, w[p + "q_proj.weight"]).view(T, H, d), (d,), w[p + "q_norm.weight"], cfg["rms_norm_eps"])
+    k = F.rms_norm(F.linear(n, w[p + "k_proj.weight"]).view(T, G, d), (d,), w[p + "k_norm.weight"], cfg["rms_norm_eps"])
+    v = F.linear(n, w[p + "v_proj.weight"]).view(T, G, d)
+    q, k = P.rope_neox(q, list(range(T)), cfg["rope_theta"]), P.rope_neox(k, list(range(T)), cfg["rope_theta"])
+    o = F.scaled_dot_product_attention(q.transpose(0, 1), k.repeat_interleave(H // G, dim=1).transpose(0, 1),
+                                       v.repeat_interleave(H // G, dim=1).transpose(0, 1), is_causal=True)
+    return F.linear(o.transpose(0, 1).reshape(T, H * d), w[p + "o_proj.weight"])
+
+
+def test_branches_add_to_a_stream_that_is_never_normalised_itself():
+    cfg, w = _tiny(False)
+    ids = [5, 11, 2, 29, 17, 8]
+    eps = cfg["rms_norm_eps"]
+    emb = w["model.embed_tokens.weight"][ids]
+    bare = F.linear(F.rms_norm(emb, (16,), w["model.norm.weight"], eps), w["lm_head.weight"])
+    # both branches of both layers silenced: what is left is embedding -> final norm -> head, so
+    # no layer norm touches the stream itself (a post-norm arrangement would)
+    w0 = dict(w)
+    for i in range(2):
+        for name in (f"model.layers.{i}.self_attn.o_proj.weight", f"model.layers.{i}.mlp.down_proj.weight"):
+            w0[name] = torch.zeros_like(w[name])
+    assert torch.allclose(P.forward(cfg, w0, ids), bare, atol=1e-12)
+    assert not torch.allclose(P.forward(cfg, w, ids), bare, atol=1e-3)
+    # a stream a million times larger drowns the branches (their inputs are normed, so they stay as
+    # they are) and the final norm takes the factor out again
+    big = dict(w)
+    big["model.embed_tokens.weight"] = w["model.embed_tokens.weight"] * 1e6
+    assert torch.allclose(P.forward(cfg, big, ids), bare, atol=1e-3)
+
+
+def test_one_layer_equals_its_formula_in_library_routines():
+    cfg, w = _tiny(False)
+    cfg["num_hidden_layers"] = 1
+    ids = [5, 11, 2, 29, 17, 8, 8, 3]
+    T, eps, p = len(ids), cfg["rms_norm_eps"], "model.layers.0."
+    h = w["model.embed_tokens.weight"][ids]
+    r = h + _library_attention(F.rms_norm(h, (16,), w[p + "input_layernorm.weight"], eps), w, p + "self_attn.", cfg, T)
+    m = F.rms_norm(r, (16,), w[p + "post_attention_layernorm.weight"], eps)          # of r, not of h
+    out = r + F.linear(F.silu(F.linear(m, w[p + "mlp.gate_proj.weight"])) * F.linear(m, w[p + "mlp.up_proj.weight"]),
+                       w[p + "mlp.down_proj.weight"])                              # onto r, not onto h
+    want = F.linear(F.rms_norm(out, (16,), w["model.norm.weight"], eps), w["lm_head.weight"])
+    got = P.forward(cfg, w, ids)
+    assert torch.allclose(got, want, atol=1e-10)
+    # the two plausible mistakes differ by far more than that: a feed-forward that reads the stream
+    # before the attention was added, and one that is added onto it
+    m_wrong = F.rms_norm(h, (16,), w[p + "post_attention_layernorm.weight"], eps)
+    mlp = lambda t: F.linear(F.silu(F.linear(t, w[p + "mlp.gate_proj.weight"])) * F.linear(t, w[p + "mlp.up_proj.weight"]),
+                             w[p + "mlp.down_proj.weight"])
+    for wrong in (r + mlp(m_wrong), h + mlp(m)):
+        logits = F.linear(F.rms_norm(wrong, (16,), w["model.norm.weight"], eps), w["lm_head.weight"])
+        assert float((logits - got).abs().max()) > 1e-2
+    # silencing the feed-forward leaves stream + attention: the attention branch reaches the logits
+    w1 = dict(w)
+    w1[p + "mlp.down_proj.weight"] = torch.zeros_like(w[p + "mlp.down_proj.weight"])
+    assert torch.allclose(P.forward(cfg, w1, ids),
+                          F.linear(F.rms_norm(r, (16,), w["model.norm.weight"], eps), w["lm_head.weight"]), atol=1e-10)

@@ -156,7 +156,11 @@ def test_trace_run_program(model_folders, tmp_path):
     # fewer heads and a narrower feed-forward to keep the plain implementation's time down
     dict(hidden_size=5120, intermediate_size=1536, num_attention_heads=10, num_key_value_heads=2),
     dict(hidden_size=5120, intermediate_size=2560, num_attention_heads=16, num_key_value_heads=2),
-], ids=["8B", "14B-like", "32B-like"])
+    # and their true layers: 40 and 64 query heads over 8 kv heads (q as wide as, and wider than, the
+    # hidden size), intermediate 17408 and 25600; two shorter requests
+    dict(hidden_size=5120, intermediate_size=17408, num_attention_heads=40, num_key_value_heads=8),
+    dict(hidden_size=5120, intermediate_size=25600, num_attention_heads=64, num_key_value_heads=8),
+], ids=["8B", "14B-like", "32B-like", "14B", "32B"])
 def test_real_layer_sizes(tmp_path, sizes):
     """Qwen3-8B layer sizes (hidden 4096, 32 query / 8 kv heads of 128, intermediate
     12288) with random weights, one layer and a small vocabulary to keep the plain
@@ -170,7 +174,8 @@ def test_real_layer_sizes(tmp_path, sizes):
         architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=1, head_dim=128, vocab_size=2048,
         max_position_embeddings=4096, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False, **sizes))
     folder = write_random_model(str(tmp_path / "big"), "Qwen3ForCausalLM", cfg, seed=5)
-    reqs = {f"r{i}": random_prompt(2048, n, 300 + i) for i, n in enumerate([150, 97, 40])}
+    lengths = [150, 97, 40] if sizes["intermediate_size"] <= 12288 else [150, 45]
+    reqs = {f"r{i}": random_prompt(2048, n, 300 + i) for i, n in enumerate(lengths)}
     want = plain_logits(folder, reqs)
     for dtype in ("float32", "bfloat16"):
         model, _ = load_model(folder, dtype, "cuda:0")
