@@ -11,8 +11,8 @@ from tiny_llm_infer_amd.engine.scheduler import Scheduler, SchedulerConfig, Sche
 from tiny_llm_infer_amd.engine.sequence import Sequence, Status
 from tiny_llm_infer_amd.sampling.params import SamplingParams
 
-FULL = CacheNeed(2, 16, None)
-WIN = CacheNeed(2, 16, 20)
+FULL = CacheNeed.keys_and_values(2, 16, None)
+WIN = CacheNeed.keys_and_values(2, 16, 20)
 
 
 # --------------------------------------------------------------------- pages --
@@ -30,6 +30,41 @@ def test_pool_hands_out_the_lowest_free_page_and_refuses_double_release():
     with pytest.raises(PageError):
         pool.take()
     pool.check()
+
+
+def test_reviving_a_page_never_queues_it_twice():
+    """A page taken back by id and released again, many times over: the queue of free ids
+    holds every id at most once (it does not grow), the lowest free id still comes first."""
+    pool = PagePool(6)
+    assert [pool.take() for _ in range(6)] == list(range(6))
+    for p in (4, 2, 5):
+        pool.release(p)
+    for _ in range(50):
+        pool.revive(2)
+        pool.check()
+        pool.release(2)
+        pool.revive(5)
+        pool.release(5)
+    pool.check()
+    assert len(pool._heap) <= 6
+    assert [pool.take() for _ in range(3)] == [2, 4, 5]
+    with pytest.raises(PageError):
+        pool.take()
+    pool.check()
+
+
+def test_a_cache_need_names_its_records():
+    from tiny_llm_infer_amd.cache import PAGE, CacheRecord
+    kv = CacheNeed.keys_and_values(2, 16, None)
+    assert [(r.name, r.page_shape(8)) for r in kv.records] == [("k", (2, 8, 16)), ("v", (2, 16, 8))]
+    assert kv == FULL and kv != WIN and sum(r.elems_per_token() for r in kv.records) == 64
+    with pytest.raises(ValueError):
+        CacheRecord("x", (4, 4))                # no axis for the page's tokens
+    with pytest.raises(ValueError):
+        CacheNeed((CacheRecord("x", (PAGE, 4)), CacheRecord("x", (PAGE, 2))))
+    # layers whose records differ do not share a group
+    m = CacheManager([FULL, CacheNeed((CacheRecord("latent", (PAGE, 24)),), None), FULL], 8, 4, 1)
+    assert [g.cache_layers for g in m.groups] == [[0, 2], [1]]
 
 
 def test_groups_have_pages_of_their_own():

@@ -316,7 +316,7 @@ def make_step(seq_lens, new_counts, page, num_pages, seed, kv_heads, head_dim, d
     k.normal_(0, 50.0)
     v.normal_(0, 50.0)
     i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=DEV)
-    g = GroupView(k=k, v=v, tables=i32(tables), table_width=width, page_size=page, window=window)
+    g = GroupView(tensors={"k": k, "v": v}, tables=i32(tables), table_width=width, page_size=page, window=window)
     step = StepView(num_rows=len(pos), num_seqs=len(seq_lens), token_ids=i32(pos), positions=i32(pos),
                     seq_of_row=i32(seq), row_start=i32(row_start),
                     seq_start=i32([n - c for n, c in zip(seq_lens, new_counts)]), seq_len=i32(seq_lens),

@@ -437,3 +437,157 @@ def test_toy_routed_feed_forward_and_another_rotation(tmp_path, dtype):
         for k in reqs:
             assert np.abs(got[k] - want[k]).max() <= bound * max(1.0, np.abs(want[k]).max()), (dtype, k)
         runner.cache.check()
+
+
+# ------------------------------- a toy norm, and a toy mixer with a cache record of its own ---
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_norm_and_a_mixer_that_caches_one_vector_per_token(tmp_path, dtype):
+    """Defined here and registered without a change to the framework: a LayerNorm (weight and
+    bias, the plain four-argument interface) that stands before the framework's attention and
+    SwiGLU, also in bfloat16 where the stock norm hands those parts rows with a factor still
+    owed; and a mixer that keeps one float32 vector per token in pages of its own (a record it
+    declares itself, with a window, so that its pages are given back as the window passes) and
+    answers with the mean of the vectors its window holds.  All cuts against a plain version
+    written here, with so few pages that they are used again."""
+    import numpy as np
+
+    from helpers import collect, trace_mixed, trace_portions, trace_prefill_then_decode, trace_whole
+    from tiny_llm_infer_amd import register_architecture
+    from tiny_llm_infer_amd.cache import PAGE, CacheNeed, CacheRecord
+    from tiny_llm_infer_amd.config import BlockSpec, LayerCall, ModelSpec, PartSpec
+    from tiny_llm_infer_amd.engine.loading import load_model, write_random_model
+    from tiny_llm_infer_amd.engine.replay import Replayer
+    from tiny_llm_infer_amd.engine.runner import ModelRunner
+    from tiny_llm_infer_amd.engine.sizing import page_bytes, workspace_bytes
+    from tiny_llm_infer_amd.parts import Mixer, Norm, register_part
+    from tiny_llm_infer_amd.weights import TensorDecl
+
+    size, latent, window, heads, kv, hd, inter, vocab, eps = 128, 24, 13, 4, 2, 64, 96, 157, 1e-5
+
+    class ToyLayerNorm(Norm):
+        def tensors(self):
+            n = self.spec.params["size"]
+            return [TensorDecl(self.spec.names["weight"], (n,), "ones_normal"), TensorDecl(self.spec.names["bias"], (n,))]
+
+        def load(self, weights, env):
+            super().load(weights, env)
+            self.w, self.b = weights[self.spec.names["weight"]].float(), weights[self.spec.names["bias"]].float()
+
+        def forward(self, resid, delta, rows=None, num_rows=None):
+            assert delta is None or isinstance(delta, torch.Tensor)       # never an unfinished product
+            if rows is None:
+                if delta is not None:
+                    resid += delta.float()
+                h = resid
+            else:
+                pick = rows[:num_rows].long()
+                h = resid[pick] if delta is None else resid[pick] + delta[pick].float()
+            mu = h.mean(-1, keepdim=True)
+            var = ((h - mu) ** 2).mean(-1, keepdim=True)
+            return ((h - mu) / torch.sqrt(var + eps) * self.w + self.b).to(self.env.dtype)
+
+    class LatentMean(Mixer):
+        """c_t = Wc x_t is kept for every token; y_t = Wo mean(c_s, s in the last `window` tokens)."""
+        def tensors(self):
+            return [TensorDecl(self.spec.names["c"], (latent, size)), TensorDecl(self.spec.names["o"], (size, latent))]
+
+        def load(self, weights, env):
+            super().load(weights, env)
+            self.wc, self.wo = weights[self.spec.names["c"]].float(), weights[self.spec.names["o"]].float()
+
+        def cache_need(self):
+            return CacheNeed((CacheRecord("latent", (PAGE, latent), torch.float32),), window)
+
+        def workspace_elems(self, rows):
+            return rows * latent
+
+        def forward(self, x, step):
+            cache, g = step.cache.record("latent"), step.cache.group      # [pages, page, latent]
+            assert cache.dtype == torch.float32 and tuple(cache.shape[1:]) == (g.page_size, latent)
+            c = x.float() @ self.wc.t()
+            pos = step.positions[:step.num_rows].long()
+            table = g.tables[step.seq_of_row[:step.num_rows].long()]      # [rows, width]
+            cache[table.gather(1, (pos // g.page_size)[:, None])[:, 0], pos % g.page_size] = c
+            out = torch.empty((step.num_rows, latent), dtype=torch.float32, device=x.device)
+            for r in range(step.num_rows):
+                p = int(pos[r])
+                seen = torch.arange(max(0, p - window + 1), p + 1, device=x.device)
+                pages = table[r, seen // g.page_size].long()
+                assert int(pages.min()) >= 0                             # every page the window reaches is held
+                out[r] = cache[pages, seen % g.page_size].mean(0)
+            return (out @ self.wo.t()).to(x.dtype)
+
+    register_part("norm", "toy_layernorm", ToyLayerNorm, replace=True)
+    register_part("mixer", "toy_latent_mean", LatentMean, replace=True)
+
+    class ToyConfig:
+        def __init__(self, d):
+            self.d = d
+
+        def to_dict(self):
+            return self.d
+
+    def toy_spec(c):
+        ln = lambda name: PartSpec("toy_layernorm", {"size": size}, {"weight": name + ".w", "bias": name + ".b"})
+        rms = lambda n, name: PartSpec("rmsnorm", {"size": n, "eps": eps}, {"weight": name})
+        mixers = (PartSpec("toy_latent_mean", {}, {"c": "l0.c", "o": "l0.o"}),
+                  PartSpec("paged_attention", {"hidden_size": size, "num_heads": heads, "num_kv_heads": kv, "head_dim": hd,
+                                               "scale": hd ** -0.5, "window": None}, {k: f"l1.{k}" for k in "qkvo"},
+                           {"position": PartSpec("rope_neox", {"head_dim": hd, "theta": 1e4, "max_positions": 512}),
+                            "q_norm": rms(hd, "l1.qn"), "k_norm": rms(hd, "l1.kn")}))
+        blocks = tuple(BlockSpec("prenorm", mixers[i],
+                                 PartSpec("swiglu", {"hidden_size": size, "intermediate_size": inter},
+                                          {"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}),
+                                 {"mixer": ln(f"l{i}.n1"), "ffn": ln(f"l{i}.n2")}) for i in range(2))
+        return ModelSpec("ToyLatentLM", size, vocab, 512,
+                         PartSpec("token_embedding", {"vocab_size": vocab, "hidden_size": size}, {"weight": "emb"}),
+                         blocks, (LayerCall(0, 0), LayerCall(1, 1)), ln("norm"),
+                         PartSpec("linear_head", {"vocab_size": vocab, "hidden_size": size, "tied": False}, {"weight": "head"}))
+
+    register_architecture("ToyLatentLM", lambda d, origin: ToyConfig(d), toy_spec, replace=True)
+    folder = write_random_model(str(tmp_path / "toylatent"), "ToyLatentLM", ToyConfig({"architectures": ["ToyLatentLM"]}), seed=13)
+    w = {k: v for k, v in P.read_safetensors(str(tmp_path / "toylatent" / "model.safetensors")).items()}
+
+    def layernorm(h, name):
+        mu = h.mean(-1, keepdim=True)
+        return (h - mu) / torch.sqrt(((h - mu) ** 2).mean(-1, keepdim=True) + eps) * w[name + ".w"] + w[name + ".b"]
+
+    def plain(ids):
+        T = len(ids)
+        h = w["emb"][torch.tensor(ids)]
+        for i in range(2):
+            n = layernorm(h, f"l{i}.n1")
+            if i == 0:
+                c = n @ w["l0.c"].t()
+                mean = torch.stack([c[max(0, t - window + 1):t + 1].mean(0) for t in range(T)])
+                r = h + mean @ w["l0.o"].t()
+            else:
+                cfg = dict(num_attention_heads=heads, num_key_value_heads=kv, head_dim=hd, rms_norm_eps=eps, rope_theta=1e4)
+                att = {f"s.{k}_proj.weight": w[f"l1.{k}"] for k in "qkvo"}
+                att.update({"s.q_norm.weight": w["l1.qn"], "s.k_norm.weight": w["l1.kn"]})
+                r = h + P.attention_block(n, att, "s.", cfg, list(range(T)), None)
+            m = layernorm(r, f"l{i}.n2")
+            h = r + P.linear(P.swiglu(P.linear(m, w[f"l{i}.g"]), P.linear(m, w[f"l{i}.u"])), w[f"l{i}.d"])
+        return P.linear(layernorm(h, "norm"), w["head"]).numpy()
+
+    rng = np.random.default_rng(6)
+    reqs = {f"c{i}": rng.integers(0, vocab, n).tolist() for i, n in enumerate([41, 60, 10, 35])}
+    want = {k: plain(v) for k, v in reqs.items()}
+    model, _ = load_model(folder, dtype, DEV)
+    needs = model.cache_needs()
+    assert [tuple(r.name for r in n.records) for n in needs] == [("latent",), ("k", "v")]
+    # what a page costs and what a step needs aside come from what the parts declare
+    elem = 4 if dtype == "float32" else 2
+    assert page_bytes(model, 8) == 8 * (latent * 4 + 2 * kv * hd * elem)
+    assert workspace_bytes(model, 100) >= 4 * 100 * (latent + 3 * inter)
+    bound = 2e-5 if dtype == "float32" else 4e-2
+    for steps in (trace_whole(reqs), trace_prefill_then_decode(reqs), trace_portions(reqs, 3),
+                  trace_mixed(reqs, 192, seed=4)):
+        runner = ModelRunner(model, model.env, page_size=8, num_pages=24, max_requests=4, max_batch_tokens=256)
+        assert sorted(runner.group_tensors[0]) == ["latent"] and runner.group_tensors[0]["latent"].dtype == torch.float32
+        rp = Replayer(runner)
+        got = collect(steps, {s["step"]: rp.run_step(s) for s in steps})
+        for k in reqs:
+            assert np.abs(got[k] - want[k]).max() <= bound * max(1.0, np.abs(want[k]).max()), (dtype, k)
+        runner.cache.check()
+        assert runner.cache.pages_returned_total > 0 and runner.cache.free_pages() == [24, 24]

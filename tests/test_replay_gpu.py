@@ -278,3 +278,45 @@ def test_many_rows_decoded_together_at_real_width(tmp_path, batch):
     for rid in ids:
         runner.release(rid)
     runner.cache.check()
+
+
+def test_trace_run_twice_gives_the_same_bytes_and_an_index(model_folders, tmp_path):
+    """Two runs of bin/trace_run on the same bfloat16 trace (prompt portions of more than 128
+    rows among them, whose products could go to one of two kernels) write byte-identical
+    logits; index.jsonl names the request and position of every row and the block tables
+    of every step, in which no page belongs to two live requests."""
+    name = "D"
+    reqs = _requests(name, [200, 150, 70], seed=61)
+    steps = trace_mixed(reqs, max_tokens=512, seed=3)
+    first = {"step": 0, "entries": [{"id": "whole", "tokens": reqs["r0"], "want": [0, 199]}], "end": ["whole"]}
+    steps = [first] + [dict(s, step=s["step"] + 1) for s in steps]
+    runs = []
+    for run in range(2):
+        out_dir = tmp_path / f"run{run}"
+        proc = subprocess.run(
+            [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_folders[name],
+             "--dtype", "bfloat16", "--out", str(out_dir), "--max-tokens", "512"],
+            input="".join(json.dumps(s) + "\n" for s in steps), text=True,
+            stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert "kernels: own-products" in proc.stderr
+        runs.append({f: (out_dir / f).read_bytes() for f in sorted(os.listdir(out_dir))})
+    assert runs[0].keys() == runs[1].keys() and len(runs[0]) > 10
+    for f in runs[0]:
+        assert runs[0][f] == runs[1][f], f
+    index = [json.loads(line) for line in runs[0]["index.jsonl"].decode().splitlines()]
+    assert [i["step"] for i in index] == [s["step"] for s in steps]
+    vocab = TINY[name]["vocab_size"]
+    fed = {}
+    for s, i in zip(steps, index):
+        rows = []
+        for e in s["entries"]:
+            rows += [{"id": e["id"], "position": fed.get(e["id"], 0) + w} for w in e["want"]]
+            fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
+        assert i["rows"] == rows
+        if rows:
+            assert len(runs[0][i["file"]]) == 4 * vocab * len(rows)
+        assert sorted(i["block_tables"]) == sorted(e["id"] for e in s["entries"])
+        for group in range(2):                                 # D: a windowed layer and a full one
+            held = [p for t in i["block_tables"].values() for p in t[group] if p >= 0]
+            assert len(held) == len(set(held)) and all(0 <= p < 512 // 16 for p in held)

@@ -1,5 +1,6 @@
-from .manager import CacheFull, CacheManager, CacheNeed, GroupLayout, RequestCache, StateNeed
+from .manager import (PAGE, CacheFull, CacheManager, CacheNeed, CacheRecord, GroupLayout, RequestCache,
+                      StateNeed)
 from .pages import PageError, PagePool
 
-__all__ = ["CacheFull", "CacheManager", "CacheNeed", "GroupLayout", "RequestCache", "StateNeed",
-           "PageError", "PagePool"]
+__all__ = ["PAGE", "CacheFull", "CacheManager", "CacheNeed", "CacheRecord", "GroupLayout", "RequestCache",
+           "StateNeed", "PageError", "PagePool"]

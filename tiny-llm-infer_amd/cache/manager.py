@@ -22,11 +22,11 @@ of a shared prefix are not run again.  It is available only when every group kee
 all keys and no mixer keeps state, because a passed window page or a state cannot
 be taken over.
 
-Page layout on the device: keys ``[cache layer in group, page, kv head, slot,
-head_dim]``, values ``[cache layer in group, page, kv head, head_dim, slot]``, so
-that one head's part of a page is contiguous and each matrix-core operand is
-contiguous along the index it is contracted over.  The block table of a
-request maps ``position // page_size`` to a page id, -1 where no page is held.
+What a page holds is the mixer's to say (``CacheRecord``): the manager deals in
+page ids only.  The attention part keeps keys ``[cache layer in group, page, kv
+head, slot, head_dim]`` and values ``[cache layer in group, page, kv head,
+head_dim, slot]``.  The block table of a request maps ``position // page_size``
+to a page id, -1 where no page is held.
 """
 from __future__ import annotations
 
@@ -40,12 +40,56 @@ class CacheFull(RuntimeError):
     """No pages (or state slots) are left for what was asked."""
 
 
+PAGE = -1          # in a record's ``dims``: the axis that counts the tokens of a page
+
+
+@dataclass(frozen=True)
+class CacheRecord:
+    """One tensor a mixer keeps per token, given as the shape of one page of it: ``dims`` with
+    ``PAGE`` where the page's token slots are counted (exactly once).  ``dtype`` None: the run's
+    storage type, else a torch dtype.  The engine allocates, per group of layers,
+    ``[layers in group, pages, *dims]`` with ``PAGE`` replaced by the page size, zeroed."""
+    name: str
+    dims: Tuple[int, ...]
+    dtype: object = None
+
+    def __post_init__(self):
+        if list(self.dims).count(PAGE) != 1 or any(d <= 0 for d in self.dims if d != PAGE):
+            raise ValueError(f"cache record '{self.name}': dims {self.dims} must be positive sizes "
+                             f"with PAGE exactly once")
+
+    def page_shape(self, page_size: int) -> Tuple[int, ...]:
+        return tuple(page_size if d == PAGE else d for d in self.dims)
+
+    def elems_per_token(self) -> int:
+        n = 1
+        for d in self.dims:
+            if d != PAGE:
+                n *= d
+        return n
+
+
 @dataclass(frozen=True)
 class CacheNeed:
-    """What one mixer needs of the paged cache.  ``window`` None: all keys."""
-    num_kv_heads: int
-    head_dim: int
+    """What one mixer needs of the paged cache: the records it keeps for every token and
+    how far back its rows read (``window`` None: everything, else the last ``window``
+    tokens, so that pages before the window can be given back).  Cache layers whose needs
+    are equal share a group: page ids, block tables and tensors of their own."""
+    records: Tuple[CacheRecord, ...]
     window: Optional[int] = None
+
+    def __post_init__(self):
+        names = [r.name for r in self.records]
+        if not names or len(set(names)) != len(names):
+            raise ValueError("a cache need names at least one record, each once")
+
+    @staticmethod
+    def keys_and_values(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> "CacheNeed":
+        """The records of attention over keys and values: keys ``[kv head, slot, head_dim]``,
+        values transposed ``[kv head, head_dim, slot]``, so that each matrix-core operand is
+        contiguous along the index it is contracted over."""
+        return CacheNeed((CacheRecord("k", (num_kv_heads, PAGE, head_dim)),
+                          CacheRecord("v", (num_kv_heads, head_dim, PAGE))), window)
 
 
 @dataclass(frozen=True)

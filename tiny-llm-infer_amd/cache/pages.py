@@ -24,8 +24,9 @@ class PagePool:
         if num_pages < 0:
             raise ValueError("num_pages must not be negative")
         self.num_pages = num_pages
-        self._heap: List[int] = list(range(num_pages))     # may hold stale ids (lazy deletion)
-        heapq.heapify(self._heap)
+        self._heap: List[int] = list(range(num_pages))     # may hold ids that are held (lazy deletion),
+        heapq.heapify(self._heap)                           # but every id at most once
+        self._in_heap = [True] * num_pages
         self._is_free = [True] * num_pages
         self._free_count = num_pages
         self._refs = [0] * num_pages
@@ -50,6 +51,7 @@ class PagePool:
             raise PageError("the page pool is exhausted")
         while True:
             page = heapq.heappop(self._heap)
+            self._in_heap[page] = False
             if self._is_free[page]:
                 break
         assert self._refs[page] == 0
@@ -62,7 +64,7 @@ class PagePool:
         """Take a particular free page (its contents are wanted again)."""
         if not self._is_free[page]:
             raise PageError(f"page {page} is not free")
-        self._is_free[page] = False          # its heap entry goes stale and is skipped later
+        self._is_free[page] = False          # its heap entry stays: skipped by take(), used again by release()
         self._free_count -= 1
         self._refs[page] = 1
 
@@ -80,13 +82,17 @@ class PagePool:
         if self._refs[page] == 0:
             self._is_free[page] = True
             self._free_count += 1
-            heapq.heappush(self._heap, page)
+            if not self._in_heap[page]:          # (a revived page's entry is still there)
+                heapq.heappush(self._heap, page)
+                self._in_heap[page] = True
 
     def check(self) -> None:
         """Every page is either free or held, the count is right, and every free
         page can still be found: none lost, none twice."""
         if sum(self._is_free) != self._free_count:
             raise PageError("the count of free pages is wrong")
+        if len(self._heap) != sum(self._in_heap) or len(set(self._heap)) != len(self._heap):
+            raise PageError("a page id is queued twice")
         reachable = set(self._heap)
         for p in range(self.num_pages):
             if self._is_free[p] != (self._refs[p] == 0):

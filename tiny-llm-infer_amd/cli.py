@@ -262,8 +262,9 @@ the logits at the wanted places.  Nothing is sampled.
 Steps are read from standard input, one JSON object a line:
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
 For a step in which something is wanted, OUT/<step>.f32 holds the logits at the
-wanted places as little-endian float32 [wanted, vocab].  After every step a
-line "done <step>" is printed."""
+wanted places as little-endian float32 [wanted, vocab]; OUT/index.jsonl names, step by
+step, the request and position of every row and the block tables the step ran with.
+After every step a line "done <step>" is printed."""
 
 
 def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
@@ -280,10 +281,11 @@ def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
     ap.add_argument("--max-live", type=int, default=4, help="most requests live at a time")
     ap.add_argument("--max-step-tokens", type=int, default=8192, help="most tokens in one step")
     ap.add_argument("--device", default="cuda:0")
-    ap.add_argument("--kernels", default="tuned", choices=["tuned", "plain", "own-products", "library-products"],
-                    help="plain: the simple twins of the tuned kernels (bfloat16 too); own-products / library-products: "
-                         "every matrix product of more than 128 rows by this library's kernel / by the BLAS library "
-                         "(tuned: the faster one for the shape, timed when the shape first comes up)")
+    ap.add_argument("--kernels", default="own-products", choices=["own-products", "library-products", "measured", "plain"],
+                    help="which kernel multiplies more than 128 rows: this library's (the default here: the same "
+                         "trace then gives the same bytes in every run), the BLAS library's, or 'measured': the "
+                         "faster one for the shape, timed when the shape first comes up, as --infer and --bench do; "
+                         "plain: the simple twins of all tuned kernels (bfloat16 too)")
     args = ap.parse_args(argv)
     if 64 % args.page_size:
         ap.error("--page-size must divide 64")
@@ -296,8 +298,8 @@ def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
     pages = max(1, (args.max_tokens + args.page_size - 1) // args.page_size)
     runner = ModelRunner(model, model.env, page_size=args.page_size, num_pages=pages,
                          max_requests=args.max_live, max_batch_tokens=args.max_step_tokens)
-    print(f"[trace_run] ready: {type(cfg).__name__}, {args.dtype}, {pages} pages of {args.page_size}",
-          file=sys.stderr, flush=True)
+    print(f"[trace_run] ready: {type(cfg).__name__}, {args.dtype}, {pages} pages of {args.page_size}, "
+          f"kernels: {args.kernels}", file=sys.stderr, flush=True)
     Replayer(runner, args.out).run_stream(sys.stdin, ack=sys.stdout)
     return 0
 
@@ -311,6 +313,8 @@ def _kernels(model, which: str) -> None:
         model.env.ops.many_rows = "own"
     elif which == "library-products":
         model.env.ops.many_rows = "library"
+    elif which in ("measured", "tuned"):
+        model.env.ops.many_rows = "measure"
 
 
 USAGE = """usage: model_main --infer [options] | --bench [options] | --replay [options]

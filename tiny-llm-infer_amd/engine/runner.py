@@ -19,7 +19,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheFull, CacheManager
-from ..parts.base import BuildEnv, GroupView, LayerCache, StepView
+from ..parts.base import BuildEnv, GroupView, LayerCache, StepView, run_norm
 from .model import Model
 
 
@@ -115,16 +115,16 @@ class ModelRunner:
         if prefix_caching and any(n is not None for n in model.state_needs()):
             raise ValueError("prefix caching cannot take over per-request state of a mixer")
         self.cache = CacheManager(model.cache_needs(), page_size, num_pages, max_requests, prefix_caching)
-        self.group_tensors = []
+        # The pages' contents: for every group the records its mixers declared, one tensor each,
+        # [layers in group, pages, *the record's page shape], zeroed.  (One page and one state
+        # slot more than the manager hands out: what the padding rows of a recorded decode
+        # step write to.)
+        self.group_tensors: List[Dict[str, torch.Tensor]] = []
         for g in self.cache.groups:
-            n, heads, hd = len(g.cache_layers), g.need.num_kv_heads, g.need.head_dim
-            # keys [.., slot, head_dim]; values transposed [.., head_dim, slot]: both are
-            # then contiguous along the index the matrix cores contract over
-            # (one page and one state slot more than the manager hands out: what the
-            # padding rows of a recorded decode step write to)
-            k = torch.zeros((n, num_pages + 1, heads, page_size, hd), dtype=env.dtype, device=env.device)
-            v = torch.zeros((n, num_pages + 1, heads, hd, page_size), dtype=env.dtype, device=env.device)
-            self.group_tensors.append((k, v))
+            self.group_tensors.append({
+                rec.name: torch.zeros((len(g.cache_layers), num_pages + 1) + rec.page_shape(page_size),
+                                      dtype=rec.dtype or env.dtype, device=env.device)
+                for rec in g.need.records})
         self.pad_page, self.pad_slot = num_pages, max_requests
         self.states: List[Optional[torch.Tensor]] = []
         for need in model.state_needs():
@@ -152,7 +152,7 @@ class ModelRunner:
         self.cache.release(key)
 
     def cache_bytes(self) -> int:
-        return sum(k.numel() * k.element_size() * 2 for k, _ in self.group_tensors)
+        return sum(t.numel() * t.element_size() for tensors in self.group_tensors for t in tensors.values())
 
     # ---- the step -----------------------------------------------------------
     def _check(self, entries: Sequence[StepEntry]) -> None:
@@ -256,8 +256,7 @@ class ModelRunner:
             self.env.ops.feed_tokens(dev[lay["token_ids"]], dev[lay["token_from"]], feed, rows)
         groups = []
         for g, gl in enumerate(self.cache.groups):
-            k, v = self.group_tensors[g]
-            groups.append(GroupView(k=k, v=v, tables=dev[lay[f"tables{g}"]].view(seqs, width),
+            groups.append(GroupView(tensors=self.group_tensors[g], tables=dev[lay[f"tables{g}"]].view(seqs, width),
                                     table_width=width, page_size=page, window=gl.need.window))
         return StepView(
             num_rows=rows, num_seqs=seqs,
@@ -289,7 +288,7 @@ class ModelRunner:
         step.state = None
         if num_wanted == 0:
             return None
-        x = model.final_norm.forward(resid, pending, rows=step.sample_rows, num_rows=num_wanted)
+        x = run_norm(model.final_norm, resid, pending, rows=step.sample_rows, num_rows=num_wanted)
         return model.head.forward(x)
 
     def _replay(self, view: StepView, wanted: int) -> torch.Tensor:
@@ -315,7 +314,12 @@ class ModelRunner:
         """Run one batch.  Pages are reserved for every entry first; if the pool
         cannot hold the batch, CacheFull is raised and no token has been run.
         ``feed``: int32 tensor on the device that entries with ``token_from`` take
-        their token from (the tokens the previous step sampled)."""
+        their token from (the tokens the previous step sampled).
+
+        The logits that come back belong to the runner: for a recorded decode step they are
+        a view of the recording's output buffer, which the next step of the same shape
+        writes again.  Use them (sample from them, copy them) before the next call of
+        ``step``; ``clone()`` what has to outlive it."""
         self._check(entries)
         # all or nothing over the whole batch: groups are independent, requests compete
         need = [0] * len(self.cache.groups)

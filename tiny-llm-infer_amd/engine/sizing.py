@@ -8,24 +8,28 @@ from __future__ import annotations
 import torch
 
 
+def _elem_size(dtype, run_dtype) -> int:
+    return torch.empty((), dtype=dtype or run_dtype).element_size()
+
+
 def page_bytes(model, page_size: int) -> int:
-    """Bytes of one page id across all groups (each group owns as many pages)."""
-    elem = 2 if model.env.dtype == torch.bfloat16 else 4
+    """Bytes of one page id across all groups (each group owns as many pages): every record
+    that the mixers declared, for every cache layer."""
     total = 0
     for need in model.cache_needs():
         if need is not None:
-            total += 2 * need.num_kv_heads * need.head_dim * page_size * elem
+            for rec in need.records:
+                total += rec.elems_per_token() * page_size * _elem_size(rec.dtype, model.env.dtype)
     return total
 
 
 def workspace_bytes(model, max_batch_tokens: int) -> int:
-    """A bound on the activations of one step."""
-    widest = model.spec.hidden_size
-    for b in model.blocks:
-        for attr in ("inter", "q_dim"):
-            for part in (b.mixer, b.ffn):
-                widest = max(widest, 2 * int(getattr(part, attr, 0)))
-    return max_batch_tokens * (6 * widest + 4 * model.spec.hidden_size) * 4
+    """A bound on the activations of one step: the residual stream, its normed rows and two
+    deltas, and what the parts of the hungriest block say they hold (``workspace_elems``),
+    every element counted as four bytes, twice over for what the allocator keeps around."""
+    rows = max_batch_tokens
+    parts = max((b.mixer.workspace_elems(rows) + b.ffn.workspace_elems(rows) for b in model.blocks), default=0)
+    return 2 * 4 * (4 * rows * model.spec.hidden_size + parts)
 
 
 def estimate_num_pages(model, page_size: int, max_batch_tokens: int, max_num_seqs: int,

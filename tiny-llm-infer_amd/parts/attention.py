@@ -66,7 +66,11 @@ class PagedAttention(Mixer):
         env.ops.check_attention_sizes(self.heads, self.kv_heads, self.head_dim)
 
     def cache_need(self) -> Optional[CacheNeed]:
-        return CacheNeed(self.kv_heads, self.head_dim, self.window)
+        return CacheNeed.keys_and_values(self.kv_heads, self.head_dim, self.window)
+
+    def workspace_elems(self, rows: int) -> int:
+        # q, k, v rows (as float32 partial sums at worst), the rotated q, the attention's output
+        return rows * (3 * (self.q_dim + 2 * self.kv_dim) + 2 * self.q_dim)
 
     @property
     def takes_normed_rows(self) -> bool:       # x goes to the q/k/v product only

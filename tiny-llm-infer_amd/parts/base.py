@@ -31,17 +31,26 @@ class BuildEnv:
     device: torch.device
     ops: Any                      # the kernel library (kernels.ops.HipOps)
     max_model_len: int            # highest number of positions a request may reach
+    shared: Dict[Any, Any] = field(default_factory=dict)   # what parts of one model build once and share
+                                  # (a rotation table that every layer would otherwise build for itself)
 
 
 @dataclass
 class GroupView:
     """One cache group as a step sees it."""
-    k: torch.Tensor               # [layers in group, pages, kv heads, page_size, head_dim]
-    v: torch.Tensor               # [layers in group, pages, kv heads, head_dim, page_size]
+    tensors: Dict[str, torch.Tensor]   # record name -> [layers in group, pages, *page shape of the record]
     tables: torch.Tensor          # int32 [sequences in step, table width], -1 where no page
     table_width: int
     page_size: int
     window: Optional[int]
+
+    @property
+    def k(self) -> torch.Tensor:       # the attention part's records:
+        return self.tensors["k"]       # [layers in group, pages, kv heads, page_size, head_dim]
+
+    @property
+    def v(self) -> torch.Tensor:
+        return self.tensors["v"]       # [layers in group, pages, kv heads, head_dim, page_size]
 
 
 @dataclass
@@ -51,13 +60,17 @@ class LayerCache:
     layer: int                    # index inside the group's tensors
     writes: bool                  # False: keys/values were written by another call of this step
 
+    def record(self, name: str) -> torch.Tensor:
+        """This layer's tensor of the record ``name``: [pages, *page shape]."""
+        return self.group.tensors[name][self.layer]
+
     @property
     def k(self) -> torch.Tensor:
-        return self.group.k[self.layer]
+        return self.group.tensors["k"][self.layer]
 
     @property
     def v(self) -> torch.Tensor:
-        return self.group.v[self.layer]
+        return self.group.tensors["v"][self.layer]
 
 
 @dataclass
@@ -103,6 +116,13 @@ class Part:
     def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
         self.env = env
 
+    def workspace_elems(self, rows: int) -> int:
+        """How many elements of activations ``forward`` holds at its widest for a step of
+        ``rows`` rows, beyond its input and its result (the q/k/v rows of an attention, the gate
+        and up rows of a gated feed-forward).  The engine sums this over a block's parts
+        when it sets memory aside for a step before it sizes the cache."""
+        return 0
+
 
 class PositionEncoding(Part):
     """Rotary encodings expose ``rotary()``: cos and sin tables
@@ -113,12 +133,37 @@ class PositionEncoding(Part):
 
 
 class Norm(Part):
+    # A norm that sets this also takes ``lazy=True`` in ``forward``: its rows go to matrix
+    # products only (the part after it has ``takes_normed_rows``), and it may answer with
+    # whatever ``ops.linear`` / ``ops.linear_swiglu`` accept in place of a tensor (rows whose
+    # scalar factor the product applies).  A norm without it is never asked.
+    supports_lazy = False
+    # A norm that sets this takes as ``delta`` whatever ``ops.linear(..., deferred=True)``
+    # returned (a product not run yet, or partial sums).  For a norm without it the caller
+    # makes a tensor of the delta first.
+    takes_unfinished_products = False
+
     def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor],
                 rows: Optional[torch.Tensor] = None, num_rows: Optional[int] = None) -> torch.Tensor:
-        """``resid`` (float32 [T, n]) += ``delta`` if given; return the
-        normalised rows in the run dtype.  With ``rows`` only those rows are
-        computed and ``resid`` is left unchanged."""
+        """``resid`` (float32 [T, n]) += ``delta`` (run dtype [T, n]) if given; return the
+        normalised rows in the run dtype.  With ``rows`` (int32 on the device, the first
+        ``num_rows`` of them) only those rows are computed and returned, and ``resid`` is left
+        unchanged."""
         raise NotImplementedError
+
+
+def run_norm(norm: "Norm", resid: torch.Tensor, delta, consumer=None, rows=None, num_rows=None):
+    """Call a norm as blocks and the step function do: ``delta`` is what the part before still
+    owes the residual (None, a tensor, or an unfinished product), ``consumer`` the part that
+    reads the normalised rows (None: they are needed as a tensor)."""
+    if delta is not None and not isinstance(delta, torch.Tensor) and not norm.takes_unfinished_products:
+        delta = norm.env.ops.resolve(delta)
+    extra = {}
+    if rows is not None:
+        extra.update(rows=rows, num_rows=num_rows)
+    if consumer is not None and norm.supports_lazy and getattr(consumer, "takes_normed_rows", False):
+        extra["lazy"] = True
+    return norm.forward(resid, delta, **extra)
 
 
 class Mixer(Part):

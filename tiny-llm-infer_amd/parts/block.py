@@ -9,7 +9,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..weights.loader import TensorDecl
-from .base import Block, BuildEnv, StepView, register_part
+from .base import Block, BuildEnv, StepView, register_part, run_norm
 
 
 class PreNormBlock(Block):
@@ -33,10 +33,10 @@ class PreNormBlock(Block):
     def forward(self, resid: torch.Tensor, pending: Optional[torch.Tensor],
                 step: StepView) -> torch.Tensor:
         # (a part that gives its input to matrix products only lets the norm before it be
-        # taken into those products)
-        n = self.norm_mixer.forward(resid, pending, **({"lazy": True} if self.mixer.takes_normed_rows else {}))
+        # taken into those products, if the norm can do that)
+        n = run_norm(self.norm_mixer, resid, pending, consumer=self.mixer)
         a = self.mixer.forward(n, step)
-        m = self.norm_ffn.forward(resid, a, **({"lazy": True} if self.ffn.takes_normed_rows else {}))
+        m = run_norm(self.norm_ffn, resid, a, consumer=self.ffn)
         return self.ffn.forward(m, step)
 
 

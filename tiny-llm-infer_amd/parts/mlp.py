@@ -33,6 +33,9 @@ class SwiGLU(FeedForward):
         self.w_gate_up = GatedMatrix(weights[n["gate"]], weights[n["up"]], env)
         self.w_down = as_matrix(weights[n["down"]], env)
 
+    def workspace_elems(self, rows: int) -> int:
+        return rows * 3 * self.inter            # gate and up rows side by side, then the activation
+
     @property
     def takes_normed_rows(self) -> bool:       # x goes to the gate/up product only
         return getattr(self.w_gate_up, "gated", None) is not None

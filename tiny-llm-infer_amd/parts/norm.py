@@ -14,6 +14,8 @@ from .base import BuildEnv, Norm, register_part
 
 class RMSNorm(Norm):
     replayable = True
+    supports_lazy = True
+    takes_unfinished_products = True
 
     def __init__(self, spec):
         super().__init__(spec)

@@ -32,6 +32,11 @@ class NeoxRope(PositionEncoding):
     def load(self, weights, env: BuildEnv) -> None:
         super().load(weights, env)
         n = min(self.max_positions, env.max_model_len)
+        self.num_positions = n
+        key = ("rope_neox", self.theta, self.rotary_dim, n, str(env.device))
+        if key in env.shared:                 # layers with the same angles share one table
+            self.cos, self.sin = env.shared[key]
+            return
         half = self.rotary_dim // 2
         i = np.arange(half, dtype=np.float32)
         exponent = (np.float32(-2.0) * i) / np.float32(self.rotary_dim)
@@ -41,7 +46,7 @@ class NeoxRope(PositionEncoding):
         a64 = angle.astype(np.float64)
         self.cos = torch.from_numpy(np.cos(a64).astype(np.float32)).to(env.device).contiguous()
         self.sin = torch.from_numpy(np.sin(a64).astype(np.float32)).to(env.device).contiguous()
-        self.num_positions = n
+        env.shared[key] = (self.cos, self.sin)
 
     def rotary(self):
         return self.cos, self.sin, self.rotary_dim
