@@ -170,11 +170,11 @@ def _seq(i, n, max_tokens=4):
 
 def _run(sched, plan, token=1):
     """Pretend the model ran: advance the cache and post-process."""
-    for item in plan.sequences:
-        s = item.sequence
-        sched.cache.reserve(s.request_id, item.token_start + item.token_count)
-        sched.cache.advance(s.request_id, item.token_start + item.token_count)
-    return sched.postprocess(plan, [token if i.samples else None for i in plan.sequences], lambda t: False)
+    for item in plan.items:
+        s = item.seq
+        sched.cache.reserve(s.request_id, item.first + item.count)
+        sched.cache.advance(s.request_id, item.first + item.count)
+    return sched.postprocess(plan, [token if i.samples else None for i in plan.items], lambda t: False)
 
 
 def test_prompts_are_cut_to_the_token_budget_one_portion_a_step():
@@ -184,22 +184,22 @@ def test_prompts_are_cut_to_the_token_budget_one_portion_a_step():
     s.add(a)
     s.add(b)
     p = s.schedule()
-    assert [(i.sequence.request_id, i.token_start, i.token_count, i.is_prefill) for i in p.sequences] == \
+    assert [(i.seq.request_id, i.first, i.count, i.prompt_portion) for i in p.items] == \
         [(1, 0, 24, True)]
     _run(s, p)
     p = s.schedule()          # b is now first in the queue, a went to the back
-    assert [(i.sequence.request_id, i.token_start, i.token_count) for i in p.sequences] == \
+    assert [(i.seq.request_id, i.first, i.count) for i in p.items] == \
         [(2, 0, 10), (1, 24, 14)]
-    assert [i.samples for i in p.sequences] == [True, False]
+    assert [i.samples for i in p.items] == [True, False]
     _run(s, p)
     assert b.status == Status.RUNNING and b.size == 11
     p = s.schedule()          # decode first, then the rest of a's prompt
-    assert [(i.sequence.request_id, i.token_start, i.token_count, i.is_prefill) for i in p.sequences] == \
+    assert [(i.seq.request_id, i.first, i.count, i.prompt_portion) for i in p.items] == \
         [(2, 10, 1, False), (1, 38, 12, True)]
     assert p.num_tokens == 13
     _run(s, p)
     p = s.schedule()
-    assert [(i.sequence.request_id, i.is_prefill) for i in p.sequences] == [(2, False), (1, False)]
+    assert [(i.seq.request_id, i.prompt_portion) for i in p.items] == [(2, False), (1, False)]
 
 
 def test_max_num_seqs_limits_a_step_and_running_requests_take_turns():
@@ -208,10 +208,10 @@ def test_max_num_seqs_limits_a_step_and_running_requests_take_turns():
     for i in range(1, 4):
         s.add(_seq(i, 5, max_tokens=10))
     p = s.schedule()
-    assert [i.sequence.request_id for i in p.sequences] == [1, 2]
+    assert [i.seq.request_id for i in p.items] == [1, 2]
     _run(s, p)
     p = s.schedule()          # two running requests fill the step; 3 waits
-    assert [i.sequence.request_id for i in p.sequences] == [1, 2]
+    assert [i.seq.request_id for i in p.items] == [1, 2]
     _run(s, p)
 
 
@@ -225,11 +225,11 @@ def test_requests_finish_at_max_tokens_or_eos_and_give_everything_back():
     done = []
     for step in range(3):
         p = s.schedule()
-        for item in p.sequences:
-            cache.reserve(item.sequence.request_id, item.token_start + item.token_count)
-            cache.advance(item.sequence.request_id, item.token_start + item.token_count)
+        for item in p.items:
+            cache.reserve(item.seq.request_id, item.first + item.count)
+            cache.advance(item.seq.request_id, item.first + item.count)
         # b draws the end-of-sequence token 99 in the second step
-        toks = [99 if (i.sequence is b and step == 1) else 1 for i in p.sequences]
+        toks = [99 if (i.seq is b and step == 1) else 1 for i in p.items]
         done += s.postprocess(p, toks, lambda t: t == 99)
     assert [d.request_id for d in done] == [2, 1]
     assert b.completion_tokens == [1, 99] and a.completion_tokens == [1, 1, 1]
@@ -246,11 +246,11 @@ def test_when_pages_run_out_the_request_is_preempted_and_computed_again():
     _run(s, s.schedule())                       # both prompts: 2 pages each, pool full
     assert cache.free_pages() == [0]
     p = s.schedule()                            # both decode at position 7: still fits
-    assert len(p.sequences) == 2
+    assert len(p.items) == 2
     _run(s, p)
     p = s.schedule()                            # position 8 needs a third page: a is preempted,
     assert s.num_preemptions == 1               # its pages let b go on
-    assert [(i.sequence.request_id, i.is_prefill) for i in p.sequences] == [(2, False)]
+    assert [(i.seq.request_id, i.prompt_portion) for i in p.items] == [(2, False)]
     assert a.status == Status.WAITING and not a.admitted and a.preemptions == 1
     assert s.waiting[0] is a
     _run(s, p)
@@ -258,7 +258,7 @@ def test_when_pages_run_out_the_request_is_preempted_and_computed_again():
     while b.status != Status.FINISHED:
         _run(s, s.schedule())
     p = s.schedule()
-    assert [(i.sequence.request_id, i.token_start, i.token_count, i.is_prefill) for i in p.sequences] == \
+    assert [(i.seq.request_id, i.first, i.count, i.prompt_portion) for i in p.items] == \
         [(1, 0, 9, True)]
     while not s.is_finished():
         _run(s, s.schedule())
@@ -271,14 +271,14 @@ def test_a_prompt_larger_than_the_pool_is_an_error_and_a_stuck_queue_too():
     cache = CacheManager([FULL], page_size=4, num_pages=2, max_requests=2)
     s = Scheduler(SchedulerConfig(2, 64), cache)
     s.add(_seq(1, 9))
-    with pytest.raises(SchedulerError, match="more KV blocks"):
+    with pytest.raises(SchedulerError, match="more than all"):
         s.schedule()
     cache = CacheManager([FULL], page_size=4, num_pages=2, max_requests=2)
     cache.admit("someone else")
     cache.reserve("someone else", 8)
     s = Scheduler(SchedulerConfig(2, 64), cache)
     s.add(_seq(1, 5))
-    with pytest.raises(SchedulerError, match="could not make progress"):
+    with pytest.raises(SchedulerError, match="nothing can run"):
         s.schedule()
 
 

@@ -41,13 +41,13 @@ def test_greedy_generation_matches_plain(model_folders):
 
 def test_admission_checks(model_folders):
     eng = _engine(model_folders["A"], "A", max_model_len=32)
-    with pytest.raises(ValueError, match="at least one token"):
+    with pytest.raises(ValueError, match="prompt is empty"):
         eng.add_request([], SamplingParams())
-    with pytest.raises(ValueError, match="exceeds max_model_len"):
+    with pytest.raises(ValueError, match="holds at most"):
         eng.add_request([1] * 33, SamplingParams(max_tokens=1))
-    with pytest.raises(ValueError, match="completion exceeds"):
+    with pytest.raises(ValueError, match="do not fit max_model_len"):
         eng.add_request([1] * 30, SamplingParams(max_tokens=4))
-    with pytest.raises(ValueError, match="greater than zero"):
+    with pytest.raises(ValueError, match="at least one new token"):
         eng.add_request([1], SamplingParams(max_tokens=0))
     with pytest.raises(ValueError, match="top_p"):
         eng.add_request([1], SamplingParams(top_p=0.0))

@@ -121,13 +121,13 @@ def run_inference(argv: List[str]) -> int:
         gpu_memory_utilization=util, enable_prefix_caching=args.enable_prefix_caching)
     if args.eos_id is not None:
         engine.eos_token_ids = set(args.eos_id)
-    print(f"Preallocating {engine.runner.cache.num_pages} KV blocks "
-          f"({engine.runner.cache_bytes() >> 20} MiB).", file=sys.stderr)
+    print(f"cache: {engine.runner.cache.num_pages} pages of {engine.runner.page_size} tokens, "
+          f"{engine.runner.cache_bytes() >> 20} MiB", file=sys.stderr)
     sampling = SamplingParams(max_tokens=args.max_new_tokens, temperature=args.temperature,
                               top_p=args.top_p, ignore_eos=args.ignore_eos, seed=args.sampling_seed)
     results = engine.generate(prompts, sampling)
     if len(results) != len(prompts):
-        print("The engine returned an incomplete result set.", file=sys.stderr)
+        print(f"{len(results)} results came back for {len(prompts)} prompts", file=sys.stderr)
         return 1
     for r in results:
         print(" ".join(str(t) for t in r.token_ids))

@@ -15,7 +15,7 @@ import torch
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .runner import ModelRunner, StepEntry
-from .scheduler import BatchPlan, Scheduler, SchedulerConfig
+from .scheduler import StepPlan, Scheduler, SchedulerConfig
 from .sequence import Sequence, Status
 
 
@@ -23,7 +23,7 @@ from .sequence import Sequence, Status
 class _Inflight:
     """A step that is on the device: its plan, which items sample, the sampled token
     ids (int32 tensor on the device, not yet read) and each request's row in them."""
-    plan: BatchPlan
+    plan: StepPlan
     sampled_items: List[int]
     tokens: Optional[torch.Tensor]
     row_of: dict
@@ -49,7 +49,7 @@ class LLMEngine:
     def __init__(self, runner: ModelRunner, max_model_len: int, max_num_seqs: int,
                  max_num_batched_tokens: int, eos_token_ids: Seq[int] = ()):
         if max_model_len <= 0:
-            raise ValueError("Engine capacities and block size must be positive.")
+            raise ValueError(f"max_model_len is {max_model_len}; a request needs room for at least one token")
         self.runner = runner
         self.max_model_len = min(max_model_len, runner.max_model_len)
         self.scheduler = Scheduler(SchedulerConfig(max_num_seqs, max_num_batched_tokens), runner.cache)
@@ -98,17 +98,17 @@ class LLMEngine:
         """engine/src/llm_engine.cpp:41-64."""
         sampling.validate()
         if sampling.max_tokens == 0:
-            raise ValueError("max_tokens must be greater than zero.")
+            raise ValueError("max_tokens is 0: a request has to ask for at least one new token")
         if len(prompt) == 0:
-            raise ValueError("A prompt must encode to at least one token.")
+            raise ValueError("the prompt is empty: a request starts from at least one token id")
         if len(prompt) > self.max_model_len:
-            raise ValueError("The prompt exceeds max_model_len.")
+            raise ValueError(f"the prompt has {len(prompt)} tokens, this engine holds at most {self.max_model_len} a request (max_model_len)")
         if sampling.max_tokens > self.max_model_len - len(prompt) + 1:
-            raise ValueError("The requested completion exceeds max_model_len.")
+            raise ValueError(f"{len(prompt)} prompt tokens and {sampling.max_tokens} new ones do not fit max_model_len = {self.max_model_len}")
         vocab = self.runner.model.spec.vocab_size
         for t in prompt:
             if not 0 <= int(t) < vocab:
-                raise ValueError(f"Token id {t} is outside the vocabulary of {vocab}.")
+                raise ValueError(f"token id {t} in the prompt: the vocabulary has ids 0..{vocab - 1}")
 
     def add_request(self, prompt_tokens: Seq[int], sampling: Optional[SamplingParams] = None) -> int:
         sampling = sampling or SamplingParams()
@@ -150,16 +150,16 @@ class LLMEngine:
             }
 
     # ---- one step -------------------------------------------------------------------
-    def _launch(self, plan: BatchPlan, ahead_of: Optional["_Inflight"] = None) -> "_Inflight":
+    def _launch(self, plan: StepPlan, ahead_of: Optional["_Inflight"] = None) -> "_Inflight":
         """Put one planned step on the device: the batch, then the sampling.  Nothing
         is waited for.  With ``ahead_of``, every item's token is the one that step
         sampled for the same request and is taken on the device."""
         entries, sampled_items = [], []
-        for i, item in enumerate(plan.sequences):
-            seq = item.sequence
-            want = [item.token_count - 1] if item.samples else []
+        for i, item in enumerate(plan.items):
+            seq = item.seq
+            want = [item.count - 1] if item.samples else []
             if ahead_of is None:
-                toks = seq.token_ids[item.token_start:item.token_start + item.token_count]
+                toks = seq.token_ids[item.first:item.first + item.count]
                 entries.append(StepEntry(seq.request_id, toks, want))
             else:
                 entries.append(StepEntry(seq.request_id, [0], want, token_from=ahead_of.row_of[seq.request_id]))
@@ -169,7 +169,7 @@ class LLMEngine:
         tokens = None
         row_of = {}
         if sampled_items:
-            seqs = [plan.sequences[i].sequence for i in sampled_items]
+            seqs = [plan.items[i].seq for i in sampled_items]
             # a request whose previous draw is still on the device has one more sample behind it
             extra = 0 if ahead_of is None else 1
             tokens = self.sampler.launch(logits, [s.sampling for s in seqs], [s.rng_seed for s in seqs],
@@ -198,7 +198,7 @@ class LLMEngine:
         if cur is None:
             with self._lock:
                 plan = self.scheduler.schedule()
-            if not plan.sequences:
+            if not plan.items:
                 return []
             cur = self._launch(plan)
         nxt = None
@@ -208,11 +208,11 @@ class LLMEngine:
             if ahead is not None:
                 nxt = self._launch(ahead, ahead_of=cur)
                 self.num_steps_ahead += 1
-        sampled: List[Optional[int]] = [None] * len(cur.plan.sequences)
+        sampled: List[Optional[int]] = [None] * len(cur.plan.items)
         if cur.sampled_items:
             for i, tok in zip(cur.sampled_items, cur.token_list()):         # waits for this step only
                 sampled[i] = int(tok)
-        live = sum(1 for i in cur.sampled_items if cur.plan.sequences[i].sequence.status != Status.FINISHED)
+        live = sum(1 for i in cur.sampled_items if cur.plan.items[i].seq.status != Status.FINISHED)
         with self._lock:
             finished = self.scheduler.postprocess(cur.plan, sampled, self.is_eos)
         self._inflight = nxt
@@ -230,14 +230,14 @@ class LLMEngine:
         if not prompts:
             return []
         if not self.is_finished():
-            raise ValueError("Finish or step existing requests before calling generate.")
+            raise ValueError("generate() starts from an idle engine: requests added earlier are still being served (step() until is_finished())")
         if sampling is None:
             sampling = SamplingParams()
         params = [sampling] * len(prompts) if isinstance(sampling, SamplingParams) else list(sampling)
         if len(params) == 1 and len(prompts) > 1:
             params = params * len(prompts)
         if len(params) != len(prompts):
-            raise ValueError("Pass one SamplingParams object or one per prompt.")
+            raise ValueError(f"{len(params)} sampling parameter sets for {len(prompts)} prompts: give one for all or one each")
         import copy
         for prompt, p in zip(prompts, params):
             self._check_request(prompt, p)

@@ -41,21 +41,21 @@ class SchedulerConfig:
 
 
 @dataclass
-class ScheduledSequence:
-    sequence: Sequence
-    token_start: int
-    token_count: int
-    is_prefill: bool
+class PlanItem:
+    seq: Sequence
+    first: int
+    count: int
+    prompt_portion: bool
 
     @property
     def samples(self) -> bool:
         """Does this item end at the request's last token (so a token is sampled)?"""
-        return (not self.is_prefill) or self.token_start + self.token_count == self.sequence.size
+        return (not self.prompt_portion) or self.first + self.count == self.seq.size
 
 
 @dataclass
-class BatchPlan:
-    sequences: List[ScheduledSequence] = field(default_factory=list)
+class StepPlan:
+    items: List[PlanItem] = field(default_factory=list)
     num_tokens: int = 0
 
 
@@ -69,15 +69,15 @@ class Scheduler:
         self.running: Deque[Sequence] = deque()
         self.num_preemptions = 0
 
-    def add(self, sequence: Sequence) -> None:
-        if sequence.size == 0:
-            raise ValueError("A scheduled request must contain at least one token.")
-        self.waiting.append(sequence)
+    def add(self, seq: Sequence) -> None:
+        if seq.size == 0:
+            raise ValueError("a request without tokens cannot be queued")
+        self.waiting.append(seq)
 
     def is_finished(self) -> bool:
         return not self.waiting and not self.running
 
-    def plan_ahead(self, plan: BatchPlan) -> Optional[BatchPlan]:
+    def plan_ahead(self, plan: StepPlan) -> Optional[StepPlan]:
         """The plan of the step after ``plan``, made while ``plan`` is still running on
         the device, or None if it cannot be known yet.  It can when the next step is
         decode only: nothing waits, ``plan`` covers every running request and every item
@@ -85,29 +85,29 @@ class Scheduler:
         those tokens are free.  A request that reaches ``max_tokens`` with the running
         step is left out; one that will stop on an end-of-sequence token cannot be known
         and is skipped when its result comes in."""
-        if self.waiting or len(plan.sequences) != len(self.running) or not plan.sequences:
+        if self.waiting or len(plan.items) != len(self.running) or not plan.items:
             return None
-        if any(not item.samples or item.sequence.status == Status.FINISHED for item in plan.sequences):
+        if any(not item.samples or item.seq.status == Status.FINISHED for item in plan.items):
             return None
-        ahead = BatchPlan()
+        ahead = StepPlan()
         need = [0] * len(self.cache.groups)
-        for item in plan.sequences:
-            seq = item.sequence
+        for item in plan.items:
+            seq = item.seq
             if seq.completion_size + 1 >= seq.sampling.max_tokens:
                 continue                      # the running step's token is its last
             # seq.size does not count the running step's token yet: that token goes to position seq.size
             for g, n in enumerate(self.cache.pages_needed(seq.request_id, seq.size + 1)):
                 need[g] += n
-            ahead.sequences.append(ScheduledSequence(seq, seq.size, 1, False))
-        if not ahead.sequences or len(ahead.sequences) > self.config.max_num_seqs:
+            ahead.items.append(PlanItem(seq, seq.size, 1, False))
+        if not ahead.items or len(ahead.items) > self.config.max_num_seqs:
             return None
         # the requests compete for the same pools: the whole step's pages must be free, or
         # nothing is taken and the ordinary path decides whom to preempt
         if any(n > g.pool.free_count for n, g in zip(need, self.cache.groups)):
             return None
-        for item in ahead.sequences:
-            self.cache.reserve(item.sequence.request_id, item.token_start + 1)
-        ahead.num_tokens = len(ahead.sequences)
+        for item in ahead.items:
+            self.cache.reserve(item.seq.request_id, item.first + 1)
+        ahead.num_tokens = len(ahead.items)
         return ahead
 
     # ---- pages ------------------------------------------------------------
@@ -116,8 +116,7 @@ class Scheduler:
             self.cache.release(seq.request_id)
             seq.admitted = False
         seq.status = Status.WAITING
-        seq.num_cached_tokens = 0
-        seq.num_scheduled_tokens = 0
+        seq.tokens_in_cache = 0
         seq.preemptions += 1
         self.num_preemptions += 1
         self.waiting.appendleft(seq)
@@ -137,72 +136,69 @@ class Scheduler:
             return False
         self.cache.reserve(seq.request_id, seq.size)
         seq.admitted = True
-        seq.num_cached_tokens = cached
+        seq.tokens_in_cache = cached
         return True
 
     # ---- one step's plan -----------------------------------------------------
-    def schedule(self) -> BatchPlan:
-        plan = BatchPlan()
+    def schedule(self) -> StepPlan:
+        plan = StepPlan()
         budget = self.config.max_num_batched_tokens
         tokens = 0
         for _ in range(len(self.running)):
-            if len(plan.sequences) >= self.config.max_num_seqs or tokens >= budget:
+            if len(plan.items) >= self.config.max_num_seqs or tokens >= budget:
                 break
             seq = self.running.popleft()
             if not self.cache.can_reserve(seq.request_id, seq.size):
                 self._preempt(seq)
                 continue
             self.cache.reserve(seq.request_id, seq.size)
-            seq.num_scheduled_tokens = 1
-            plan.sequences.append(ScheduledSequence(seq, seq.size - 1, 1, False))
+            plan.items.append(PlanItem(seq, seq.size - 1, 1, False))
             self.running.append(seq)
             tokens += 1
 
         for _ in range(len(self.waiting)):
-            if len(plan.sequences) >= self.config.max_num_seqs or tokens >= budget:
+            if len(plan.items) >= self.config.max_num_seqs or tokens >= budget:
                 break
             seq = self.waiting.popleft()
             if not seq.admitted and not self._admit(seq):
                 if not self._pages_for_whole_pool(seq.size):
-                    raise SchedulerError("The prompt requires more KV blocks than the engine owns.")
+                    raise SchedulerError(f"request {seq.request_id} holds {seq.size} tokens, more than all {self.cache.num_pages} pages of {self.cache.page_size} can take")
                 self.waiting.append(seq)
                 continue
-            remaining = seq.size - seq.num_cached_tokens
+            remaining = seq.size - seq.tokens_in_cache
             if remaining <= 0:
-                raise SchedulerError("A waiting prompt has no uncached tokens to schedule.")
+                raise SchedulerError(f"request {seq.request_id} waits although all its {seq.size} tokens are in the cache")
             count = min(remaining, budget - tokens)
-            seq.num_scheduled_tokens = count
-            plan.sequences.append(ScheduledSequence(seq, seq.num_cached_tokens, count, True))
+            plan.items.append(PlanItem(seq, seq.tokens_in_cache, count, True))
             tokens += count
-            if seq.num_cached_tokens + count == seq.size:
+            if seq.tokens_in_cache + count == seq.size:
                 seq.status = Status.RUNNING
                 self.running.append(seq)
             else:
                 self.waiting.append(seq)
         plan.num_tokens = tokens
-        if not plan.sequences and not self.is_finished():
-            raise SchedulerError("The scheduler could not make progress with the available KV blocks.")
+        if not plan.items and not self.is_finished():
+            raise SchedulerError("nothing can run: requests remain, but neither a decode token nor a prompt portion found pages")
         return plan
 
     # ---- after the step --------------------------------------------------------
-    def postprocess(self, plan: BatchPlan, sampled: Seq[Optional[int]],
+    def postprocess(self, plan: StepPlan, sampled: Seq[Optional[int]],
                     is_eos: Callable[[int], bool]) -> List[Sequence]:
         """``sampled[i]`` is the token of plan item i, None where nothing was
         sampled.  Returns the requests that finished."""
-        if len(sampled) != len(plan.sequences):
-            raise SchedulerError("The model runner returned the wrong number of sampled tokens.")
+        if len(sampled) != len(plan.items):
+            raise SchedulerError(f"{len(sampled)} sampled tokens came back for a plan of {len(plan.items)} items")
         finished = []
-        for item, token in zip(plan.sequences, sampled):
-            seq = item.sequence
+        for item, token in zip(plan.items, sampled):
+            seq = item.seq
             if seq.status == Status.FINISHED:
                 continue            # it ended in the step before, while this one was already running
-            seq.num_cached_tokens += item.token_count
-            seq.num_scheduled_tokens = 0
+            seq.tokens_in_cache += item.count
             self.cache.register_pages(seq.request_id, seq.token_ids)     # full pages enter the prefix cache
-            if item.is_prefill and seq.num_cached_tokens < seq.size:
+            if item.prompt_portion and seq.tokens_in_cache < seq.size:
                 continue
             if token is None or token < 0:
-                raise SchedulerError("The model runner did not return a token for a completed step.")
+                raise SchedulerError(f"request {seq.request_id} reached its last token in this step but no token was sampled for it")
             seq.token_ids.append(int(token))
             seq.num_sampled += 1
             stopped = (not seq.sampling.ignore_eos) and is_eos(int(token))

@@ -23,8 +23,7 @@ class Sequence:
     prompt_size: int
     sampling: SamplingParams
     status: Status = Status.WAITING
-    num_cached_tokens: int = 0          # tokens whose keys and values are in the cache
-    num_scheduled_tokens: int = 0
+    tokens_in_cache: int = 0          # tokens whose keys and values are in the cache
     admitted: bool = False              # holds a state slot and pages
     num_sampled: int = 0                # draws used so far; survives preemption
     preemptions: int = 0

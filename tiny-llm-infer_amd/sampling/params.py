@@ -17,13 +17,13 @@ class SamplingParams:
 
     def validate(self) -> None:
         if self.max_tokens < 0:
-            raise ValueError("max_tokens cannot be negative.")
+            raise ValueError(f"max_tokens is {self.max_tokens}; it counts tokens and cannot be below zero")
         if self.temperature < 0.0:
-            raise ValueError("temperature cannot be negative.")
+            raise ValueError(f"temperature is {self.temperature}; 0 means greedy, anything above draws")
         if not 0.0 < self.top_p <= 1.0:
-            raise ValueError("top_p must be in the interval (0, 1].")
+            raise ValueError(f"top_p is {self.top_p}; it is the share of the probability mass that is kept, above 0 and at most 1")
         if self.seed < 0:
-            raise ValueError("seed cannot be negative.")
+            raise ValueError(f"seed is {self.seed}; seeds are unsigned (0: the request id seeds the draws)")
 
     @property
     def greedy(self) -> bool:
