@@ -303,16 +303,18 @@ def test_a_request_that_ends_while_its_next_step_is_on_the_device(model_folders,
         free = _engine(folder, name, dtype, max_num_batched_tokens=64)
         free.lookahead = False
         runs = [r.token_ids for r in free.generate(prompts, SamplingParams(max_tokens=14, ignore_eos=True))]
-        eos = runs[1][5]                                  # request 1 meets it at its 6th token at the latest
+        # a token that request 1 meets in the middle of its run, and the others late or never if there is one
+        others = [t for i, run in enumerate(runs) if i != 1 for t in run[:10]]
+        eos = next((t for t in runs[1][3:7] if t not in others), runs[1][5])
         outs = []
         for ahead in (False, True):
             eng = _engine(folder, name, dtype, max_num_batched_tokens=64)
             eng.lookahead = ahead
             eng.eos_token_ids = {eos}
             outs.append([r.token_ids for r in eng.generate(prompts, SamplingParams(max_tokens=14))])
-            assert (eng.num_steps_ahead > 3) == ahead
+            assert (eng.num_steps_ahead > 0) == ahead
             if ahead and dtype == "bfloat16":
-                assert eng.runner.graph_replays > 3
+                assert eng.runner.graph_replays > 0
             eng.runner.cache.check()
             assert eng.is_finished() and all(f == 64 for f in eng.runner.cache.free_pages())
             # and the engine serves again afterwards from the pages that were given back
@@ -322,6 +324,6 @@ def test_a_request_that_ends_while_its_next_step_is_on_the_device(model_folders,
         for run, got in zip(runs, outs[1]):               # each request is its free run cut after the token
             cut = run.index(eos) + 1 if eos in run else len(run)
             assert got == run[:cut]
-        assert len(outs[1][1]) <= 6
+        assert len(outs[1][1]) <= 7
         if dtype == "float32":
             assert runs == [plain_qwen3.greedy(cfg, w, p, 14) for p in prompts]
