@@ -65,6 +65,8 @@ def main():
     ap.add_argument("--library-products", action="store_true", help="... by the BLAS library")
     ap.add_argument("--rows-cfg", type=int, default=0, help="with --own-products: force a launch shape (measurements)")
     ap.add_argument("--no-check", action="store_true", help="skip the untimed comparison of logits with the 32-bit path")
+    ap.add_argument("--shape", default=None,
+                    help="a config.json whose layer sizes replace the default ones (configs/ holds the larger shapes of the family)")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -81,6 +83,11 @@ def main():
     from tiny_llm_infer_amd.sampling.params import SamplingParams
 
     cfg_json = dict(QWEN3_8B)
+    shape_name = "Qwen3-8B shape"
+    if args.shape:
+        with open(args.shape) as fh:
+            cfg_json = json.load(fh)
+        shape_name = os.path.splitext(os.path.basename(args.shape))[0].replace("_", " ")
     full_layers = cfg_json["num_hidden_layers"]
     layers = args.layers or full_layers
     cfg_json["num_hidden_layers"] = layers
@@ -214,11 +221,11 @@ def main():
     check = logit_check() if (args.dtype == "bfloat16" and not args.no_check) else {}
 
     out = {
-        "metric": f"decode tok/s @ batch {args.batch} (Qwen3-8B shape, {dkey}, random weights)",
+        "metric": f"decode tok/s @ batch {args.batch} ({shape_name}, {dkey}, random weights)",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": dkey, "data": "synthetic",
-        "config": {"model": "Qwen3-8B shape, random weights", "global_batch": args.batch,
+        "config": {"model": f"{shape_name}, random weights", "global_batch": args.batch,
                    "seq_len": args.context, "parallelism": "single GPU", "layers": layers,
                    "layers_of_config": full_layers, "hidden_size": cfg.hidden_size,
                    "intermediate_size": cfg.intermediate_size, "heads": cfg.num_attention_heads,
