@@ -61,8 +61,9 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiles)")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement (for profiles)")
     ap.add_argument("--own-products", action="store_true",
-                    help="every product of more than 128 rows by this library's kernel (default: the faster one for the shape)")
-    ap.add_argument("--library-products", action="store_true", help="... by the BLAS library")
+                    help="every product of more than 128 rows by this library's kernel (the default)")
+    ap.add_argument("--library-products", action="store_true", help="... by the BLAS library (every matrix is then held twice)")
+    ap.add_argument("--measured-products", action="store_true", help="... by whichever was timed faster for the shape")
     ap.add_argument("--rows-cfg", type=int, default=0, help="with --own-products: force a launch shape (measurements)")
     ap.add_argument("--no-check", action="store_true", help="skip the untimed comparison of logits with the 32-bit path")
     ap.add_argument("--shape", default=None,
@@ -95,10 +96,15 @@ def main():
     elem = 2 if args.dtype == "bfloat16" else 4
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
     t0 = time.time()
-    model = random_model("Qwen3ForCausalLM", cfg, args.seed, args.dtype, "cuda:0", args.context)
-    if args.own_products or args.library_products:
-        model.env.ops.many_rows = "own" if args.own_products else "library"
-    model.env.ops.rows_cfg = args.rows_cfg
+    from tiny_llm_infer_amd.kernels.ops import HipOps
+    ops = HipOps("cuda:0")
+    # which kernel multiplies more than 128 rows is settled before the weights are loaded: a matrix
+    # keeps its row-major form only where the library (or the plain kernels of the untimed check) reads it
+    ops.many_rows = "library" if args.library_products else ("measure" if args.measured_products else "own")
+    ops.rows_cfg = args.rows_cfg
+    before = torch.cuda.memory_allocated()
+    model = random_model("Qwen3ForCausalLM", cfg, args.seed, args.dtype, "cuda:0", args.context, ops=ops)
+    weight_gb = (torch.cuda.memory_allocated() - before) / 1e9
     torch.cuda.synchronize()
     print(f"[bench] model with {layers} layers on the device in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
 
@@ -231,7 +237,7 @@ def main():
                    "intermediate_size": cfg.intermediate_size, "heads": cfg.num_attention_heads,
                    "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "vocab_size": cfg.vocab_size, "prompt_len": args.prompt_len,
-                   "page_size": page, "prefill_tokens": T},
+                   "page_size": page, "prefill_tokens": T, "weights_gb_on_device": round(weight_gb, 2)},
         "prefill": {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
                     "frac": round(pre_flops / pre / MFMA_PEAK[dkey], 4), "of": "median of 5",
                     "best_ms": round(pre_best * 1e3, 3)},

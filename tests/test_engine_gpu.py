@@ -202,13 +202,15 @@ def test_recorded_decode_steps_equal_eager_ones(model_folders):
     assert compared > 30 and fast.graph_replays == compared and len(fast.graphs) >= 3
 
 
-@pytest.mark.parametrize("first,most,rows", [(80, 90, 96), (140, 150, 160)])
-def test_recorded_steps_of_many_rows_equal_eager_ones(tmp_path, first, most, rows):
+@pytest.mark.parametrize("first,most,rows,products", [(80, 90, 96, "own"), (140, 150, 160, "own"),
+                                                       (140, 150, 160, "library")])
+def test_recorded_steps_of_many_rows_equal_eager_ones(tmp_path, first, most, rows, products):
     """Many rows in a decode step, at the layer sizes of Qwen3-8B: up to 128 rows the
-    matrix products are the kernel with eight row tiles, beyond they are the
-    library's (which picks its kernels by shape).  80 to 90 live requests in steps
-    of 96 rows, and 140 to 150 in steps of 160; every replay is compared with the
-    same step run eagerly on a second runner, with eager prefill work and
+    matrix products are the kernel with eight row tiles, beyond they are the kernel for
+    any number of rows, or the library's where that was asked for before the weights were
+    loaded (it picks its kernels by shape, and its calls are recorded too).  80 to 90 live
+    requests in steps of 96 rows, and 140 to 150 in steps of 160; every replay is compared
+    with the same step run eagerly on a second runner, with eager prefill work and
     synchronisation between the replays."""
     from tiny_llm_infer_amd.config import Qwen3Config
     from tiny_llm_infer_amd.engine.loading import load_model, write_random_model
@@ -218,7 +220,12 @@ def test_recorded_steps_of_many_rows_equal_eager_ones(tmp_path, first, most, row
         hidden_size=4096, intermediate_size=12288, num_attention_heads=32, num_key_value_heads=8,
         max_position_embeddings=4096, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False))
     folder = write_random_model(str(tmp_path / "wide"), "Qwen3ForCausalLM", cfg, seed=9)
-    model, _ = load_model(folder, "bfloat16", "cuda:0")
+    from tiny_llm_infer_amd.kernels.ops import HipOps
+    ops = HipOps("cuda:0")
+    ops.many_rows = products
+    model, _ = load_model(folder, "bfloat16", "cuda:0", ops=ops)
+    held = model.blocks[0].ffn.w_down
+    assert (held._w is not None) == (products == "library") and held.tiled is not None     # one form, or both
     make = lambda: ModelRunner(model, model.env, page_size=16, num_pages=700, max_requests=rows,
                                max_batch_tokens=4096)
     fast, slow = make(), make()

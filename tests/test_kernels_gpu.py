@@ -221,24 +221,51 @@ def test_gated_product_of_many_rows(ops, mki, cfg):
             close(ops.linear_swiglu(x, m), g / (1 + torch.exp(-g)) * u, torch.bfloat16, f"gated product, {splits} ranges of k")
         y = ops.linear_swiglu(x, m)
     finally:
-        ops.many_rows, ops.rows_cfg, ops.rows_splits = "measure", 0, 0
+        ops.many_rows, ops.rows_cfg, ops.rows_splits = "own", 0, 0
     g, u = x.double().cpu() @ gate.double().cpu().t(), x.double().cpu() @ up.double().cpu().t()
     close(y, g / (1 + torch.exp(-g)) * u, torch.bfloat16, "gated product of many rows")
+    # the library reads the stacked row-major form, which this matrix does not hold: it is put
+    # together from the interleaved decode layout
+    assert m._w is None and torch.equal(m.w, torch.cat([gate, up]))
     ops.many_rows = "library"
     try:
         close(ops.linear_swiglu(x, m), g / (1 + torch.exp(-g)) * u, torch.bfloat16, "the library and the activation")
     finally:
-        ops.many_rows = "measure"
+        ops.many_rows = "own"
 
 
-def test_products_of_many_rows_take_the_faster_kernel(ops):
-    """By default a product of more than 128 rows is timed in gemm_rows and in the library when
-    its shape first comes up, and goes to the faster one from then on (the same one for every
-    number of rows in the same 128): the result is right whichever that is, nothing is timed
-    during a graph capture, and a shape met there first goes to the library."""
+def test_a_matrix_is_held_once_unless_the_library_reads_it(ops):
     from tiny_llm_infer_amd.parts.base import BuildEnv
     from tiny_llm_infer_amd.parts.linear import GatedMatrix, Matrix
     env = BuildEnv(dtype=torch.bfloat16, device=torch.device(DEV), ops=ops, max_model_len=64)
+    w = rnd((1000, 264), torch.bfloat16, 2, 0.05).to(DEV)            # sizes that the decode layout pads
+    m = Matrix(w, env)
+    assert m._w is None and m.tiled is not None and m.shape == (1000, 264)
+    assert m.nbytes() == m.tiled.numel() * 2 and torch.equal(m.w, w)
+    gate, up = rnd((48, 136), torch.bfloat16, 3).to(DEV), rnd((48, 136), torch.bfloat16, 4).to(DEV)
+    g = GatedMatrix(gate, up, env)
+    assert g._w is None and g.tiled is None and g.gated is not None and torch.equal(g.w, torch.cat([gate, up]))
+    odd = GatedMatrix(gate[:40], up[:40], env)                         # 40 rows do not pair up in blocks of 16
+    assert odd.gated is None and odd.tiled is not None and torch.equal(odd.w, torch.cat([gate[:40], up[:40]]))
+    ops.many_rows = "library"
+    try:
+        both = Matrix(w, env)
+        assert both._w is not None and both.tiled is not None and both.nbytes() > 2 * w.numel() * 2 - 1
+    finally:
+        ops.many_rows = "own"
+    exact = Matrix(w.float(), BuildEnv(dtype=torch.float32, device=torch.device(DEV), ops=ops, max_model_len=64))
+    assert exact.tiled is None and exact._w is not None
+
+
+def test_products_of_many_rows_take_the_faster_kernel(ops):
+    """With ``many_rows`` = "measure" a product of more than 128 rows is timed in gemm_rows and in
+    the library when its shape first comes up, and goes to the faster one from then on (the same
+    one for every number of rows in the same 128): the result is right whichever that is, nothing
+    is timed during a graph capture, and a shape met there first goes to the library."""
+    from tiny_llm_infer_amd.parts.base import BuildEnv
+    from tiny_llm_infer_amd.parts.linear import GatedMatrix, Matrix
+    env = BuildEnv(dtype=torch.bfloat16, device=torch.device(DEV), ops=ops, max_model_len=64)
+    ops.many_rows = "measure"
     ops.measured.clear()
     M, N, K = 1000, 1024, 512
     x, w = rnd((M, K), torch.bfloat16, 1).to(DEV), rnd((N, K), torch.bfloat16, 2, 0.05).to(DEV)
@@ -265,6 +292,7 @@ def test_products_of_many_rows_take_the_faster_kernel(ops):
     assert (3, N, K, 0) not in ops.measured
     close(y, x2.double().cpu() @ w.double().cpu().t(), torch.bfloat16, "product recorded before its shape was measured")
     ops.measured.clear()
+    ops.many_rows = "own"
 
 
 def test_library_linear_for_many_rows(ops):

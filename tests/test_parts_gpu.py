@@ -79,8 +79,10 @@ def test_embedding_and_head_parts(envs, dtype, tied):
     assert logits.dtype == torch.float32 and tuple(logits.shape) == (3, vocab)
     matrix = w["emb" if tied else "head"].cpu().double()
     close(logits, P.linear(x.double(), matrix), torch.float32 if dtype == torch.float32 else dtype, "head")
-    if tied:
+    if tied and dtype == torch.float32:
         assert head.weight.w.data_ptr() == emb.table.data_ptr()       # one copy of the matrix
+    elif tied:                      # the row-major matrix once (rows are gathered from it), its decode layout once
+        assert head.weight._w is None and head.weight.tiled is not None and torch.equal(head.weight.w, emb.table)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

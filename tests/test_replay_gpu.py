@@ -189,12 +189,13 @@ def test_real_layer_sizes(tmp_path, sizes):
             print(f"{sizes['hidden_size']} wide, {sizes['num_attention_heads']} heads, {dtype} {cut}: worst relative error {worst:.2e}")
             runner.cache.check()
     # bfloat16 once more with the products of more than 128 rows (the whole prompt of 150 tokens, and
-    # the 118 + 32 of "decode" is below) through this library's own kernel instead of the BLAS library
-    model.env.ops.many_rows = "own"
+    # the 118 + 32 of "decode" is below) through the BLAS library instead of this library's own kernel
+    # (the row-major matrices it reads are put together from the decode layout at every call)
+    model.env.ops.many_rows = "library"
     steps = trace_whole(reqs)
     runner = ModelRunner(model, model.env, page_size=16, num_pages=24, max_requests=4, max_batch_tokens=512)
-    worst = _check(collect(steps, _replay(runner, steps)), want, "bfloat16", f"{sizes['hidden_size']} wide/own products")
-    print(f"{sizes['hidden_size']} wide, own products of many rows: worst relative error {worst:.2e}")
+    worst = _check(collect(steps, _replay(runner, steps)), want, "bfloat16", f"{sizes['hidden_size']} wide/library products")
+    print(f"{sizes['hidden_size']} wide, library products of many rows: worst relative error {worst:.2e}")
 
 
 @pytest.mark.parametrize("name", ["B", "D"])

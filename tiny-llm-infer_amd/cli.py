@@ -36,10 +36,11 @@ def _common(ap: argparse.ArgumentParser) -> None:
                     help="with --config: draw seeded random weights instead of reading a checkpoint")
     ap.add_argument("--config", help="a config.json, for --random-weights")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--kernels", default="tuned", choices=["tuned", "plain", "own-products", "library-products"],
-                    help="plain: the simple twins of the tuned kernels (bfloat16 too); own-products / library-products: "
-                         "every matrix product of more than 128 rows by this library's kernel / by the BLAS library "
-                         "(tuned: the faster one for the shape, timed when the shape first comes up)")
+    ap.add_argument("--kernels", default="tuned", choices=["tuned", "plain", "own-products", "library-products", "measured"],
+                    help="tuned (= own-products): every matrix product by this library's kernels, each matrix held "
+                         "once; library-products: products of more than 128 rows by the BLAS library (each matrix is "
+                         "then held twice); measured: by whichever was timed faster for the shape when it first came "
+                         "up; plain: the simple twins of the tuned kernels (bfloat16 too)")
 
 
 def _device(name: str) -> str:
@@ -67,13 +68,10 @@ def _load(args, max_seq_len: int):
             data = json.load(fh)
         arch = architecture_of(data, args.config)
         cfg = arch.read_config(data, args.config)
-        model = random_model(arch.name, cfg, args.seed, args.dtype, device, max_seq_len)
-        _kernels(model, args.kernels)
-        return model
+        return random_model(arch.name, cfg, args.seed, args.dtype, device, max_seq_len, ops=_ops(device, args.kernels))
     if not args.model:
         raise SystemExit2("--model is required (or --config with --random-weights)")
-    model, _ = load_model(args.model, args.dtype, device, max_seq_len)
-    _kernels(model, args.kernels)
+    model, _ = load_model(args.model, args.dtype, device, max_seq_len, ops=_ops(device, args.kernels))
     return model
 
 
@@ -282,9 +280,9 @@ def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
     ap.add_argument("--max-step-tokens", type=int, default=8192, help="most tokens in one step")
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--kernels", default="own-products", choices=["own-products", "library-products", "measured", "plain"],
-                    help="which kernel multiplies more than 128 rows: this library's (the default here: the same "
+                    help="which kernel multiplies more than 128 rows: this library's (the default: the same "
                          "trace then gives the same bytes in every run), the BLAS library's, or 'measured': the "
-                         "faster one for the shape, timed when the shape first comes up, as --infer and --bench do; "
+                         "faster one for the shape, timed when the shape first comes up; "
                          "plain: the simple twins of all tuned kernels (bfloat16 too)")
     args = ap.parse_args(argv)
     if 64 % args.page_size:
@@ -293,8 +291,7 @@ def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
     from .engine.loading import load_model
     from .engine.replay import Replayer
     from .engine.runner import ModelRunner
-    model, cfg = load_model(args.model, args.dtype, _device(args.device))
-    _kernels(model, args.kernels)
+    model, cfg = load_model(args.model, args.dtype, _device(args.device), ops=_ops(_device(args.device), args.kernels))
     pages = max(1, (args.max_tokens + args.page_size - 1) // args.page_size)
     runner = ModelRunner(model, model.env, page_size=args.page_size, num_pages=pages,
                          max_requests=args.max_live, max_batch_tokens=args.max_step_tokens)
@@ -304,17 +301,23 @@ def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
     return 0
 
 
-def _kernels(model, which: str) -> None:
-    """--kernels plain: every product, attention and norm through the plain kernels;
-    own-products / library-products: products of many rows always through gemm_rows / the BLAS library."""
+def _ops(device: str, which: str):
+    """The kernel library set up as --kernels says, before any weight is loaded (which form of a
+    matrix is kept depends on who multiplies with it).  plain: every product, attention and norm
+    through the plain kernels; own-products / library-products / measured: products of more than
+    128 rows through gemm_rows / the BLAS library / whichever was timed faster for the shape."""
+    from .kernels.ops import HipOps
+    ops = HipOps(device)
     if which == "plain":
-        model.env.ops.use_plain_kernels()
-    elif which == "own-products":
-        model.env.ops.many_rows = "own"
+        ops.many_rows = "library"            # the plain kernels read the row-major form
+        ops.use_plain_kernels()
     elif which == "library-products":
-        model.env.ops.many_rows = "library"
-    elif which in ("measured", "tuned"):
-        model.env.ops.many_rows = "measure"
+        ops.many_rows = "library"
+    elif which == "measured":
+        ops.many_rows = "measure"
+    else:                                    # "tuned", "own-products"
+        ops.many_rows = "own"
+    return ops
 
 
 USAGE = """usage: model_main --infer [options] | --bench [options] | --replay [options]

@@ -144,6 +144,8 @@ class LLMEngine:
                 "pages_taken_total": cache.pages_taken_total,
                 "prefix_pages_reused": cache.prefix_hits,
                 "recorded_decode_shapes": len(self.runner.graphs),
+                "weight_bytes": self.runner.model.weight_bytes(),
+                "cache_bytes": self.runner.cache_bytes(),
                 # shapes of products of more than 128 rows measured so far, and how many went to this library's kernel
                 "product_shapes_measured": len(getattr(self.runner.env.ops, "measured", {})),
                 "product_shapes_own_kernel": sum(getattr(self.runner.env.ops, "measured", {}).values()),

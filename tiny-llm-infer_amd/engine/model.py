@@ -74,6 +74,30 @@ class Model:
         self.final_norm.load(weights, env)
         self.head.load(weights, env, share_with=self.embedding)
 
+    def weight_bytes(self) -> int:
+        """Bytes of device memory the loaded weights take: every tensor that a part holds (in
+        whatever forms it holds a matrix), each storage counted once."""
+        from ..parts.base import Part
+        seen, total, stack = set(), 0, [self.embedding, self.final_norm, self.head, *self.blocks]
+        visited = set()
+        while stack:
+            obj = stack.pop()
+            if id(obj) in visited:
+                continue
+            visited.add(id(obj))
+            if isinstance(obj, torch.Tensor):
+                key = obj.untyped_storage().data_ptr()
+                if key not in seen:
+                    seen.add(key)
+                    total += obj.untyped_storage().nbytes()
+            elif isinstance(obj, (list, tuple)):
+                stack.extend(obj)
+            elif isinstance(obj, dict):
+                stack.extend(obj.values())
+            elif isinstance(obj, Part) or type(obj).__module__.endswith("parts.linear"):
+                stack.extend(v for k, v in vars(obj).items() if k not in ("env", "ops", "spec"))
+        return total
+
     # ---- convenience ------------------------------------------------------
     def load_from(self, model_path: str, env: BuildEnv) -> None:
         self._load_stream(load_tensors(model_path, self.tensors(), env.dtype, env.device), env)

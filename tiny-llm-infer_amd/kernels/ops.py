@@ -29,7 +29,7 @@ class PendingProduct:
 
     def __init__(self, x: torch.Tensor, matrix):
         self.x, self.matrix = x, matrix
-        self.shape = (x.shape[0], matrix.w.shape[0])
+        self.shape = (x.shape[0], _shape_of(matrix)[0])
         self.dtype = x.dtype
 
 
@@ -103,6 +103,13 @@ def load_library():
     return lib
 
 
+def _shape_of(w) -> Tuple[int, int]:
+    """(out, in) of a [out, in] tensor or of a matrix as the parts hold it, without asking for its
+    row-major form (which such a matrix may have to put together first)."""
+    shape = getattr(w, "shape", None)
+    return tuple(shape) if shape is not None else tuple(w.w.shape)
+
+
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
@@ -145,13 +152,20 @@ class HipOps:
         self.mid_cfg = 0             # measurements: launch shape and k ranges of the 17..128-row kernel
         self.mid_splits = 0
         self.skinny_cfg = 0          # measurements: force a launch shape of the weight-streaming kernel
-        # Products of more than 128 rows: "measure" = the faster of gemm_rows and the BLAS library for
-        # the shape, timed once when the shape first comes up; "own" / "library" = always that one
-        self.many_rows = "measure"
+        # Products of more than 128 rows: "own" = gemm_rows; "library" = the BLAS library; "measure" = the
+        # faster of the two for the shape, timed once when the shape first comes up.  The latter two
+        # multiply with the row-major form of a matrix, which is then held beside its decode layout
+        # (see keep_row_major): set this before the weights are loaded.
+        self.many_rows = "own"
         self.measured = {}           # (rows rounded up to 128, N, K, gated) -> True where gemm_rows won
         self._cold = None            # what is written between two timed runs
         self.rows_cfg = 0            # measurements: force a launch shape and the k ranges of gemm_rows
         self.rows_splits = 0
+
+    @property
+    def keep_row_major(self) -> bool:
+        """Whether a bfloat16 matrix is to keep its row-major form beside its decode layout."""
+        return self.many_rows != "own"
 
     def use_plain_kernels(self) -> None:
         """Every product, attention and norm through the plain kernels, bfloat16 too
@@ -272,6 +286,13 @@ class HipOps:
         t = w.view(n16 // 16, 16, k128 // 128, 4, 4, 8)          # [nb, r, kb, c, j, e]
         return t.permute(0, 2, 4, 3, 1, 5).contiguous()           # [nb, kb, j, c, r, e]
 
+    def untile_matrix(self, tiled: torch.Tensor, shape) -> torch.Tensor:
+        """The row-major matrix [N, K] again from its decode layout (a new tensor)."""
+        N, K = shape
+        nb, kb = tiled.shape[0], tiled.shape[1]
+        w = tiled.permute(0, 4, 1, 3, 2, 5).reshape(nb * 16, kb * 128)        # [nb, r, kb, c, j, e]
+        return w[:N, :K].contiguous()
+
     def linear(self, x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None, deferred: bool = False,
                sums_only: bool = False):
         """y = x W^T.  ``w`` is a [N, K] tensor or a ``Matrix`` (row-major tensor plus
@@ -286,15 +307,15 @@ class HipOps:
         if (deferred and not sums_only and tiled is not None and x.dtype == torch.bfloat16
                 and 0 < x.shape[0] <= 16 and out_dtype in (None, torch.bfloat16) and not self.separate_norms):
             return PendingProduct(x, w)
-        w = getattr(w, "w", w)
+        matrix = w
         M, K = x.shape
-        N, K2 = w.shape
+        N, K2 = _shape_of(matrix)
         if K != K2:
             raise KernelError(f"linear: input has {K} columns, the matrix {K2}")
         self._want(x, "linear input")
-        self._want(w, "linear matrix")
-        if x.dtype != w.dtype:
-            raise KernelError(f"linear: input is {x.dtype}, the matrix {w.dtype}")
+        w_dtype = getattr(matrix, "dtype", None) or matrix.w.dtype
+        if x.dtype != w_dtype:
+            raise KernelError(f"linear: input is {x.dtype}, the matrix {w_dtype}")
         out_dtype = out_dtype or x.dtype
         y = torch.empty((M, N), dtype=out_dtype, device=self.device)
         if M == 0:
@@ -305,19 +326,26 @@ class HipOps:
             if M <= self.SKINNY_ROWS or out_dtype == torch.float32:
                 # few rows (decode), or float32 logits: the weight-streaming MFMA kernel,
                 # 64 rows at a time
-                wp = w if tiled is None else tiled
+                wp = tiled
+                if wp is None:
+                    wp = getattr(matrix, "w", matrix)
+                    self._want(wp, "linear matrix")
                 for m0 in range(0, M, self.SKINNY_ROWS):
                     m1 = min(M, m0 + self.SKINNY_ROWS)
                     self._call(self.lib.tli_gemm_skinny_bf16, x[m0:m1].data_ptr(), wp.data_ptr(),
                                y[m0:m1].data_ptr(), m1 - m0, N, K, _dtype_code(out_dtype),
                                0 if tiled is None else 1, self.skinny_cfg, self._stream())
                 return y
-            if tiled is not None and out_dtype == torch.bfloat16 and self._rows_kernel_wins(x, w, tiled, M, N, K, 0):
+            if tiled is not None and out_dtype == torch.bfloat16 and self._rows_kernel_wins(x, matrix, tiled, M, N, K, 0):
                 return self._linear_rows(x, tiled, y, M, N, K, 0, deferred or sums_only)
-            # many rows (prefill): the library's matrix product, as the reference
-            # uses its library for more than one row (kernels/src/matmul_kernel_cuda.cu:84-91)
+            # many rows (prefill) where the library was asked for: its matrix product, as the
+            # reference uses its library for more than one row (kernels/src/matmul_kernel_cuda.cu:84-91)
+            w = getattr(matrix, "w", matrix)
+            self._want(w, "linear matrix")
             torch.matmul(x, w.t(), out=y)
             return y
+        w = getattr(matrix, "w", matrix)
+        self._want(w, "linear matrix")
         self._call(self.lib.tli_gemm_plain, x.data_ptr(), w.data_ptr(), y.data_ptr(), M, N, K,
                    _dtype_code(x.dtype), _dtype_code(w.dtype), _dtype_code(out_dtype), self._stream())
         return y
@@ -326,8 +354,8 @@ class HipOps:
         """resid += x W^T, and the rows of the norm that follows, its factor still owed."""
         x, m = p.x, p.matrix
         M, K = x.shape
-        N = m.w.shape[0]
-        self._want(x, "linear input", torch.bfloat16, (M, m.w.shape[1]))
+        N = _shape_of(m)[0]
+        self._want(x, "linear input", torch.bfloat16, (M, _shape_of(m)[1]))
         if tuple(resid.shape) != (M, N):
             raise KernelError(f"the product gives {(M, N)}, the residual is {tuple(resid.shape)}")
         xw = torch.empty((M, N), dtype=torch.bfloat16, device=self.device)
@@ -344,9 +372,9 @@ class HipOps:
             raise KernelError("normed rows that still owe their factor need a matrix in the decode layout")
         if out_dtype not in (None, torch.bfloat16):
             raise KernelError("normed rows that still owe their factor give bfloat16 products")
-        rows_out = m.w.shape[0]
-        if m.w.shape[1] != K:
-            raise KernelError(f"linear: input has {K} columns, the matrix {m.w.shape[1]}")
+        rows_out = _shape_of(m)[0]
+        if _shape_of(m)[1] != K:
+            raise KernelError(f"linear: input has {K} columns, the matrix {_shape_of(m)[1]}")
         N = 2 * m.inter if gated else rows_out
         y = torch.empty((M, m.inter if gated else N), dtype=torch.bfloat16, device=self.device)
         self._call(self.lib.tli_gemm_skinny_fused_bf16, x.xw.data_ptr(), tiled.data_ptr(), y.data_ptr(), M, N, K,
@@ -366,15 +394,16 @@ class HipOps:
                    _ptr(part), M, N, K, _dtype_code(y.dtype), gated, splits, self.mid_cfg, self._stream())
         return DeferredSum(part, y.dtype) if leave else y
 
-    def _rows_kernel_wins(self, x, w, tiled, M, N, K, gated) -> bool:
+    def _rows_kernel_wins(self, x, matrix, tiled, M, N, K, gated) -> bool:
         """Whether this product of more than 128 rows goes to gemm_rows (else to the library).
-        Which one is faster changes with the shape by more than 10% either way (how well each
-        one's tiles fill the compute units), so both are timed when a shape first comes up:
-        three runs each after one to warm up, a few milliseconds, outside any graph capture."""
-        if self.many_rows != "measure":
-            return self.many_rows == "own"
+        With ``many_rows`` = "measure": which one is faster changes with the shape by up to 10%
+        either way (how well each one's tiles fill the compute units), so both are timed when a
+        shape first comes up: three runs each after one to warm up, a few milliseconds, outside
+        any graph capture."""
         if max(M, N + 15) * (K + 127) * 2 >= 1 << 32:
             return False                      # gemm_rows keeps 32-bit offsets into its operands
+        if self.many_rows != "measure":
+            return self.many_rows == "own"
         key = ((M + 127) // 128, N, K, gated)
         won = self.measured.get(key)
         if won is not None:
@@ -383,6 +412,7 @@ class HipOps:
             return False                      # (nothing can be timed now; the shape is measured when it next comes up eagerly)
         y = torch.empty((M, N // 2 if gated else N), dtype=torch.bfloat16, device=self.device)
         wide = torch.empty((M, N), dtype=torch.bfloat16, device=self.device) if gated else None
+        w = getattr(matrix, "w", matrix)
 
         def library():
             if gated:
@@ -449,7 +479,7 @@ class HipOps:
         M, K = x.shape
         gated = getattr(m, "gated", None) if not self.plain_products else None
         if gated is not None and 0 < M <= self.MID_ROWS_TO and x.dtype == torch.bfloat16:
-            self._want(x, "linear input", torch.bfloat16, (M, m.w.shape[1]))
+            self._want(x, "linear input", torch.bfloat16, (M, _shape_of(m)[1]))
             y = torch.empty((M, m.inter), dtype=x.dtype, device=self.device)
             if M >= self.MID_ROWS_FROM:
                 return self._linear_mid(x, gated, y, M, 2 * m.inter, K, 1)
@@ -457,8 +487,8 @@ class HipOps:
                        2 * m.inter, K, BF16, 2, self.skinny_cfg if self.skinny_cfg >= 20 else 0, self._stream())
             return y
         if (gated is not None and x.dtype == torch.bfloat16 and K % 8 == 0
-                and self._rows_kernel_wins(x, m.w, gated, M, 2 * m.inter, K, 1)):
-            self._want(x, "linear input", torch.bfloat16, (M, m.w.shape[1]))
+                and self._rows_kernel_wins(x, m, gated, M, 2 * m.inter, K, 1)):
+            self._want(x, "linear input", torch.bfloat16, (M, _shape_of(m)[1]))
             y = torch.empty((M, m.inter), dtype=x.dtype, device=self.device)
             return self._linear_rows(x, gated, y, M, 2 * m.inter, K, 1)
         return self.swiglu(self.linear(x, m))
