@@ -4,7 +4,7 @@
 // library's product, whichever it measured faster for the shape: at the layer sizes of
 // Qwen3-8B to 32B and 512 to 4,096 rows either is ahead by up to 15% somewhere.
 //
-// A workgroup owns ROWS rows and 256 columns and walks all of k in slices of 128:
+// A workgroup owns ROWS rows and 192, 256 or 512 columns and walks all of k in slices of 128:
 //   x   each slice [ROWS][128] is copied from memory straight into one of two LDS slots
 //       (global_load_lds_dwordx4: lane l of a wave writes the 16 bytes it asked for at LDS
 //       base + 16 l), rows swizzled as in gemm_mid.hip (chunk q of row r at q ^ (r & 15));
@@ -56,9 +56,11 @@ __device__ __forceinline__ void rows_wait_loads() {
 // Wait until at most N loads are in flight; the fragments of k-step j depend on it.
 template <int N, int RT>
 __device__ __forceinline__ void rows_wait_fragments(Pack16r (&a)[RT][4], int j) {
-    static_assert(RT == 2 || RT == 4, "two or four column tiles a wave");
+    static_assert(RT == 2 || RT == 3 || RT == 4, "two, three or four column tiles a wave");
     if constexpr (RT == 4)
         asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a[0][j].q), "+v"(a[1][j].q), "+v"(a[2][j].q), "+v"(a[3][j].q) : "n"(N));
+    else if constexpr (RT == 3)
+        asm volatile("s_waitcnt vmcnt(%3)" : "+v"(a[0][j].q), "+v"(a[1][j].q), "+v"(a[2][j].q) : "n"(N));
     else
         asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a[0][j].q), "+v"(a[1][j].q) : "n"(N));
 }
@@ -342,12 +344,31 @@ extern "C" int tli_gemm_rows_splits(int M, int N, int K) {
     return splits;
 }
 
-// The launch shape that cfg 0 takes: 128 x 512 outputs a workgroup (one a compute unit) ask the
-// L2 caches for a sixth less than 128 x 256 (two a compute unit); taken when its workgroups
-// fill their last round of the 256 compute units to 85% at least and k is not cut.
-static int rows_pick(int M, int N, int splits) {
-    const long wide = (long)(((N + 15) / 16 + 31) / 32) * ((M + 127) / 128);
-    return splits == 1 && wide * 100 >= (wide + 255) / 256 * 256 * 85 ? 3 : 2;
+// The launch shape that cfg 0 takes: the one whose workgroups fill the 256 compute units best.
+// What a shape costs is counted in rounds of workgroups, from measurements at the layer sizes of
+// Qwen3-8B to 32B and 256 to 4,096 rows.  With four waves a workgroup two workgroups share a
+// compute unit and each then takes 1.75 times as long as alone, so up to 256 workgroups cost one
+// unit, up to 512 cost 1.75, and every further 512 as much again (a remainder of up to 256 one
+// unit); 128 x 192 outputs cost 6% more a column than 128 x 256 but divide 6,144 or 5,120
+// columns over the chip where 256 leave a quarter of it idle.  128 x 512 outputs in eight
+// waves, one workgroup a compute unit, ask the L2 caches for a sixth less: 0.84 a column, in
+// rounds of 256 workgroups.
+static int rows_pick(int M, int N, int splits, int gated) {
+    const long n_tiles = (N + 15) / 16, row_blocks = (M + 127) / 128;
+    auto shared = [&](long tiles_a_group) {
+        const long wgs = (n_tiles + tiles_a_group - 1) / tiles_a_group * row_blocks * splits;
+        if (wgs <= 256) return 1.0;
+        const long full = wgs / 512, rem = wgs % 512;
+        return 1.75 * (double)full + (rem == 0 ? 0.0 : rem <= 256 ? 1.0 : 1.75);
+    };
+    const long wgs3 = (n_tiles + 31) / 32 * row_blocks * splits;
+    const double cost2 = shared(16) * 256.0, cost4 = shared(12) * 192.0 * 1.06;
+    const double cost3 = (double)((wgs3 + 255) / 256) * 512.0 * 0.84;
+    int best = 2;
+    double cost = cost2;
+    if (cost3 < cost) { best = 3; cost = cost3; }
+    if (!gated && cost4 < cost) best = 4;
+    return best;
 }
 
 // y[M,N] = x[M,K] . W^T for any number of rows, bfloat16, W in the decode layout (`gated` as
@@ -356,8 +377,9 @@ static int rows_pick(int M, int N, int splits) {
 // caller); with y null the partial sums [splits][M][N] are left for the consumer to add
 // (tli_gemm_mid_reduce, or tli_add_rmsnorm).
 // cfg 0 picks the launch shape; 1: 256 x 256 outputs a workgroup of eight waves, 2: 128 x 256
-// and four waves, two workgroups a compute unit, 3: 128 x 512 and eight waves; cfg >= 10: the
-// tens for a gated product, the ones for the others (measurements).
+// and four waves, two workgroups a compute unit, 3: 128 x 512 and eight waves, 4: 128 x 192 and
+// four waves (not for a gated product); cfg >= 10: the tens for a gated product, the ones for
+// the others (measurements).
 extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, float* part, int M, int N, int K,
                                   int gated, int splits, int cfg, void* stream) {
     if (M <= 0 || N <= 0) return 0;
@@ -372,9 +394,13 @@ extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, float* 
     if ((size_t)M * K * sizeof(bf16_t) >= (1ull << 32) || (size_t)((N + 15) / 16 * 16) * ((K + 127) / 128 * 128) * sizeof(bf16_t) >= (1ull << 32))
         return tli_fail("gemm_rows: an operand of 4 GiB or more (offsets are 32 bits)");
     if (cfg >= 10) cfg = gated ? cfg / 10 : cfg % 10;       // measurements: one shape for the gated product, one for the others
-    if (cfg == 0) cfg = rows_pick(M, N, splits);
+    if (cfg == 0) cfg = rows_pick(M, N, splits, gated);
     if (cfg == 1) return launch_rows<2, 8, 16, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     if (cfg == 2) return launch_rows<4, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     if (cfg == 3) return launch_rows<4, 8, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
+    if (cfg == 4) {
+        if (gated) return tli_fail("gemm_rows: three column tiles a wave do not pair up for a gated product");
+        return launch_rows<3, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
+    }
     return tli_fail("gemm_rows: unknown configuration %d", cfg);
 }
