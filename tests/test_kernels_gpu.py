@@ -170,7 +170,7 @@ def test_gated_product_writes_the_activation(ops, mki):
     close(two_pass, torch.nn.functional.silu(g) * u, torch.bfloat16, "stacked product, then activation")
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 6])
 @pytest.mark.parametrize("mnk", [(129, 264, 1008), (300, 4096, 4096), (2048, 6144, 512), (513, 1000, 136), (700, 48, 8), (4500, 520, 256),
                                  (1024, 5120, 384)])
 def test_product_of_many_rows_from_the_decode_layout(ops, mnk, cfg):

@@ -68,8 +68,13 @@ __device__ __forceinline__ void rows_wait_fragments(Pack16r (&a)[RT][4], int j) 
 // RT column tiles a wave, WAVES waves side by side, MT row tiles (ROWS = 16 MT), x fragments
 // taken MH row tiles at a time.  GATED: the column tiles alternate between a gate and an up
 // matrix (tiled = 2 of tli_gemm_skinny_bf16) and y is [M, N/2] = silu(gate) * up.
-template <int RT, int WAVES, int MT, int MH, bool GATED>
-__global__ void __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1)
+// KG = 2: the workgroup has two such sets of WAVES waves; they take the slices of k in turn (each
+// set with LDS slots of its own) and the second set's sums are added to the first's through
+// LDS at the end.  Where the outputs alone give one workgroup a compute unit, that puts two
+// waves on every SIMD without partial sums in memory.  (The slices of a k range must then be
+// even in number.)
+template <int RT, int WAVES, int MT, int MH, bool GATED, int KG = 1>
+__global__ void __launch_bounds__(WAVES * KG * 64, WAVES * KG == 4 ? 2 : 1)
 gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf16_t* __restrict__ y,
                  float* __restrict__ part, int M, int N, int K, int splits, int slices_per_split) {
     constexpr int ROWS = MT * 16;
@@ -81,8 +86,12 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
     static_assert((4 * WAVES) % 16 == 0, "the swizzle of a lane's chunk is then the same in every copy");
     static_assert(MT % MH == 0 && 3 * RT + XI <= 63, "the wait counts fit the counter");
     extern __shared__ uint4 xs_raw[];
-    bf16_t* xs = reinterpret_cast<bf16_t*>(xs_raw);          // [2][ROWS][128], rows swizzled
-    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, c = lane / 16;
+    const int lane = threadIdx.x % 64, r = lane % 16, c = lane / 16;
+    // set of waves (the same for a whole wave, and said so: slice numbers follow from it and go into scalar
+    // registers), wave in the set
+    const int kg = KG == 1 ? 0 : __builtin_amdgcn_readfirstlane((int)(threadIdx.x / 64) / WAVES);
+    const int wave = (int)(threadIdx.x / 64) % WAVES;
+    bf16_t* xs = reinterpret_cast<bf16_t*>(xs_raw) + (size_t)kg * 2 * SLICE;     // [2][ROWS][128] for this set, rows swizzled
     const int k_steps = (K + 127) / 128;
     const int n_tiles = (N + 15) / 16;
     // Workgroup i runs on die i % 8.  A die takes the row blocks in chunks of 2,048 rows: all
@@ -143,8 +152,10 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
         x_off[e] = (uint32_t)(((size_t)min(x_row0 + e * 4 * WAVES, M - 1) * K + x_col) * sizeof(bf16_t));
     const uint32_t xs_base = (uint32_t)(uintptr_t)(lds_void_r*)xs + (uint32_t)wave * 1024u;
     const bool ragged = (K & 127) != 0;
+    // the slot of a slice: the sets of waves take slices in turn, a set's slices alternate between its two slots
+    auto slot_of = [&](int slice) { return ((slice - slice_begin) / KG) & 1; };
     auto copy_x = [&](int slice) {
-        const uint32_t slot_base = xs_base + (uint32_t)(slice & 1) * (SLICE * 2);
+        const uint32_t slot_base = xs_base + (uint32_t)slot_of(slice) * (SLICE * 2);
         if (ragged && slice == k_steps - 1) {          // (the last slice of the last range)
             const int k = slice * 128 + x_col;
 #pragma unroll
@@ -171,7 +182,7 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
     // read from LDS before batch n is multiplied
     Pack16r b[2][MH];
     auto read_b = [&](int slice, int n, Pack16r (&dst)[MH]) {
-        const bf16_t* xb = xs + (slice & 1) * SLICE;
+        const bf16_t* xb = xs + slot_of(slice) * SLICE;
         const int j = n / HALVES, h = n % HALVES;
 #pragma unroll
         for (int m = 0; m < MH; ++m)
@@ -204,26 +215,49 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
             __builtin_amdgcn_sched_barrier(0);
             multiply(n, b[n & 1]);
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (!LAST && n % HALVES == HALVES - 1) load_w(slice + 1, j);
+            if constexpr (!LAST && n % HALVES == HALVES - 1) load_w(slice + KG, j);
         });
     };
 
     if (slice_begin < slice_end) {
-        copy_x(slice_begin);
-        load_w(slice_begin, 0);
-        load_w(slice_begin, 1);
-        load_w(slice_begin, 2);
-        load_w(slice_begin, 3);
-        int slice = slice_begin;
-        for (; slice + 1 < slice_end; ++slice) {
+        int slice = slice_begin + kg;
+        copy_x(slice);
+        load_w(slice, 0);
+        load_w(slice, 1);
+        load_w(slice, 2);
+        load_w(slice, 3);
+        for (; slice + KG < slice_end; slice += KG) {
             rows_wait_loads<4 * RT>();     // this wave's part of the slice of x has landed (behind it: 4 RT fragments)
             __syncthreads();               // everyone's has, and everyone has finished the slice before
-            copy_x(slice + 1);             // into the slot that the slice before used
+            copy_x(slice + KG);            // into the slot that the slice before used
             one_slice(slice, std::false_type{});
         }
         rows_wait_loads<4 * RT>();
         __syncthreads();
         one_slice(slice, std::true_type{});
+    }
+    if constexpr (KG == 2) {
+        // the second set hands its sums over: [wave][accumulator][lane] of 16 bytes, as much as
+        // the four slots of x together
+        static_assert(KG == 1 || RT * MT * 64 * 16 * WAVES <= 2 * 2 * SLICE * 2, "the sums fit the slots of x");
+        __syncthreads();                   // nobody reads x any more
+        f32x4* sums = reinterpret_cast<f32x4*>(xs_raw) + (size_t)wave * RT * MT * 64 + lane;
+        if (kg == 1) {
+#pragma unroll
+            for (int t = 0; t < RT; ++t)
+#pragma unroll
+                for (int m = 0; m < MT; ++m) sums[(t * MT + m) * 64] = acc[t][m];
+        }
+        __syncthreads();
+        if (kg == 1) return;
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const f32x4 other = sums[(t * MT + m) * 64];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[t][m][i] += other[i];
+            }
     }
 
     if (splits > 1) {
@@ -297,7 +331,7 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
     }
 }
 
-template <int RT, int WAVES, int MT, int MH>
+template <int RT, int WAVES, int MT, int MH, int KG = 1>
 static int launch_rows(const bf16_t* x, const bf16_t* w, bf16_t* y, float* part, int M, int N, int K, int gated,
                        int splits, hipStream_t s) {
     const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
@@ -306,12 +340,15 @@ static int launch_rows(const bf16_t* x, const bf16_t* w, bf16_t* y, float* part,
     const long blocks = (col_groups + 7) / 8 * 8 * ((row_blocks + chunk - 1) / chunk * chunk);
     if (blocks > 2147483647L) return tli_fail("gemm_rows: too many workgroups");
     const int slices_per_split = (k_steps + splits - 1) / splits;
+    if (KG == 2 && (slices_per_split % 2 || k_steps % slices_per_split))
+        return tli_fail("gemm_rows: two sets of waves need an even number of slices in every range of k (%d of %d)",
+                        slices_per_split, k_steps);
     const dim3 grid((unsigned)blocks, (unsigned)splits);
-    const size_t lds = (size_t)2 * MT * 16 * 128 * sizeof(bf16_t);
+    const size_t lds = (size_t)KG * 2 * MT * 16 * 128 * sizeof(bf16_t);
     // (more than 64 KiB of LDS has to be allowed for a kernel once)
 #define ROWS_LAUNCH(G)                                                                                     \
     {                                                                                                      \
-        auto kernel = gemm_rows_kernel<RT, WAVES, MT, MH, G>;                                              \
+        auto kernel = gemm_rows_kernel<RT, WAVES, MT, MH, G, KG>;                                          \
         static bool allowed = false;                                                                       \
         if (lds > 65536 && !allowed) {                                                                     \
             if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,       \
@@ -319,7 +356,7 @@ static int launch_rows(const bf16_t* x, const bf16_t* w, bf16_t* y, float* part,
                 return tli_fail("gemm_rows: cannot have %zu bytes of LDS", lds);                           \
             allowed = true;                                                                                \
         }                                                                                                  \
-        kernel<<<grid, WAVES * 64, lds, s>>>(x, w, y, part, M, N, K, splits, slices_per_split);            \
+        kernel<<<grid, WAVES * KG * 64, lds, s>>>(x, w, y, part, M, N, K, splits, slices_per_split);       \
     }
     if (gated) ROWS_LAUNCH(true)
     else ROWS_LAUNCH(false)
@@ -352,8 +389,10 @@ extern "C" int tli_gemm_rows_splits(int M, int N, int K) {
 // unit); 128 x 192 outputs cost 6% more a column than 128 x 256 but divide 6,144 or 5,120
 // columns over the chip where 256 leave a quarter of it idle.  128 x 512 outputs in eight
 // waves, one workgroup a compute unit, ask the L2 caches for a sixth less: 0.84 a column, in
-// rounds of 256 workgroups.
-static int rows_pick(int M, int N, int splits, int gated) {
+// rounds of 256 workgroups.  128 x 256 outputs by two sets of four waves that share out the
+// slices of k (one workgroup a compute unit again) cost 0.88 of what four waves alone do, and a
+// good deal less where k is cut into ranges as well; only for an even number of slices.
+static int rows_pick(int M, int N, int K, int splits, int gated) {
     const long n_tiles = (N + 15) / 16, row_blocks = (M + 127) / 128;
     auto shared = [&](long tiles_a_group) {
         const long wgs = (n_tiles + tiles_a_group - 1) / tiles_a_group * row_blocks * splits;
@@ -364,10 +403,14 @@ static int rows_pick(int M, int N, int splits, int gated) {
     const long wgs3 = (n_tiles + 31) / 32 * row_blocks * splits;
     const double cost2 = shared(16) * 256.0, cost4 = shared(12) * 192.0 * 1.06;
     const double cost3 = (double)((wgs3 + 255) / 256) * 512.0 * 0.84;
+    const long k_steps = (K + 127) / 128, per = (k_steps + splits - 1) / splits;
+    const long wgs2 = (n_tiles + 15) / 16 * row_blocks * splits;
+    const double cost6 = (double)((wgs2 + 255) / 256) * 256.0 * 0.88;
     int best = 2;
     double cost = cost2;
     if (cost3 < cost) { best = 3; cost = cost3; }
-    if (!gated && cost4 < cost) best = 4;
+    if (!gated && cost4 < cost) { best = 4; cost = cost4; }
+    if (!gated && per % 2 == 0 && k_steps % per == 0 && cost6 < cost) best = 6;
     return best;
 }
 
@@ -378,8 +421,9 @@ static int rows_pick(int M, int N, int splits, int gated) {
 // (tli_gemm_mid_reduce, or tli_add_rmsnorm).
 // cfg 0 picks the launch shape; 1: 256 x 256 outputs a workgroup of eight waves, 2: 128 x 256
 // and four waves, two workgroups a compute unit, 3: 128 x 512 and eight waves, 4: 128 x 192 and
-// four waves (not for a gated product); cfg >= 10: the tens for a gated product, the ones for
-// the others (measurements).
+// four waves (not for a gated product), 6: 128 x 256 by two sets of four waves that take the
+// slices of k in turn; cfg >= 10: the tens for a gated product, the ones for the others
+// (measurements).
 extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, float* part, int M, int N, int K,
                                   int gated, int splits, int cfg, void* stream) {
     if (M <= 0 || N <= 0) return 0;
@@ -394,10 +438,16 @@ extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, float* 
     if ((size_t)M * K * sizeof(bf16_t) >= (1ull << 32) || (size_t)((N + 15) / 16 * 16) * ((K + 127) / 128 * 128) * sizeof(bf16_t) >= (1ull << 32))
         return tli_fail("gemm_rows: an operand of 4 GiB or more (offsets are 32 bits)");
     if (cfg >= 10) cfg = gated ? cfg / 10 : cfg % 10;       // measurements: one shape for the gated product, one for the others
-    if (cfg == 0) cfg = rows_pick(M, N, splits, gated);
+    if (cfg == 0) cfg = rows_pick(M, N, K, splits, gated);
     if (cfg == 1) return launch_rows<2, 8, 16, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     if (cfg == 2) return launch_rows<4, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     if (cfg == 3) return launch_rows<4, 8, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
+    if (cfg == 6) {
+        const int k_steps = (K + 127) / 128, per = (k_steps + splits - 1) / splits;
+        if (per % 2 || k_steps % per) cfg = 2;       // (an odd number of slices somewhere: one set of waves)
+        else return launch_rows<4, 4, 8, 1, 2>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
+    }
+    if (cfg == 2) return launch_rows<4, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     if (cfg == 4) {
         if (gated) return tli_fail("gemm_rows: three column tiles a wave do not pair up for a gated product");
         return launch_rows<3, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
