@@ -99,13 +99,28 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
     // so on; then the next chunk (the x rows of a chunk and a W panel stay in its L2 meanwhile).
     constexpr int CHUNK = 2048 / ROWS;
     const int row_blocks = (M + ROWS - 1) / ROWS;
-    const int groups_a_die = ((n_tiles + RT * WAVES - 1) / (RT * WAVES) + 7) / 8;
+    const int col_groups = (n_tiles + RT * WAVES - 1) / (RT * WAVES);
+    const int groups_a_die = (col_groups + 7) / 8;
     const int die = blockIdx.x % 8, turn = blockIdx.x / 8;
     const int chunk = turn / (CHUNK * groups_a_die), in_chunk = turn % (CHUNK * groups_a_die);
     const int chunk_rows = min(CHUNK, row_blocks - chunk * CHUNK);      // row blocks of this chunk (the last may be short)
-    const int row_block = chunk * CHUNK + in_chunk % chunk_rows;
-    const int col_group = (in_chunk / chunk_rows) * 8 + die;
-    if (in_chunk >= chunk_rows * groups_a_die || col_group * RT * WAVES >= n_tiles) return;   // (the grid is rounded up)
+    // The column groups that do not make a whole round of the eight dies are dealt out by row
+    // blocks instead, so that every die gets as many workgroups as the others (5,120 columns are
+    // 20 groups of 256: two for every die, and of the other four each die takes half the row
+    // blocks of one).
+    const int whole = col_groups / 8, left = col_groups % 8;
+    int row_block, col_group;
+    if (in_chunk < whole * chunk_rows) {
+        row_block = chunk * CHUNK + in_chunk % chunk_rows;
+        col_group = (in_chunk / chunk_rows) * 8 + die;
+    } else {
+        const int share = (left * chunk_rows + 7) / 8;                   // workgroups of the left-over groups a die takes
+        const int j = in_chunk - whole * chunk_rows;
+        const int at = die * share + j;                                   // index among the left-over groups' workgroups
+        if (j >= share || at >= left * chunk_rows) return;                // (the grid is rounded up)
+        row_block = chunk * CHUNK + at % chunk_rows;
+        col_group = whole * 8 + at / chunk_rows;
+    }
     x += (size_t)row_block * ROWS * K;
     const int n_out = GATED ? N / 2 : N;
     y += (size_t)row_block * ROWS * n_out;
@@ -382,30 +397,31 @@ extern "C" int tli_gemm_rows_splits(int M, int N, int K) {
 }
 
 // The launch shape that cfg 0 takes: the one whose workgroups fill the 256 compute units best.
-// What a shape costs is counted in rounds of workgroups, from measurements at the layer sizes of
-// Qwen3-8B to 32B and 256 to 4,096 rows.  With four waves a workgroup two workgroups share a
-// compute unit and each then takes 1.75 times as long as alone, so up to 256 workgroups cost one
-// unit, up to 512 cost 1.75, and every further 512 as much again (a remainder of up to 256 one
-// unit); 128 x 192 outputs cost 6% more a column than 128 x 256 but divide 6,144 or 5,120
+// What a shape costs is counted in rounds of workgroups on a die (the kernel deals the
+// workgroups out evenly over the eight dies of 32 compute units), from measurements at the
+// layer sizes of Qwen3-8B to 32B and 256 to 8,192 rows.  With four waves a workgroup two
+// workgroups share a compute unit and each then takes 1.75 times as long as alone, so up to 32
+// workgroups a die cost one unit, up to 64 cost 1.75, and every further 64 as much again (a
+// remainder of up to 32 one unit); 128 x 192 outputs cost 6% more a column than 128 x 256 but divide 6,144 or 5,120
 // columns over the chip where 256 leave a quarter of it idle.  128 x 512 outputs in eight
 // waves, one workgroup a compute unit, ask the L2 caches for a sixth less: 0.84 a column, in
-// rounds of 256 workgroups.  128 x 256 outputs by two sets of four waves that share out the
+// rounds of 32 workgroups a die.  128 x 256 outputs by two sets of four waves that share out the
 // slices of k (one workgroup a compute unit again) cost 0.88 of what four waves alone do, and a
 // good deal less where k is cut into ranges as well; only for an even number of slices.
 static int rows_pick(int M, int N, int K, int splits, int gated) {
     const long n_tiles = (N + 15) / 16, row_blocks = (M + 127) / 128;
-    auto shared = [&](long tiles_a_group) {
-        const long wgs = (n_tiles + tiles_a_group - 1) / tiles_a_group * row_blocks * splits;
-        if (wgs <= 256) return 1.0;
-        const long full = wgs / 512, rem = wgs % 512;
-        return 1.75 * (double)full + (rem == 0 ? 0.0 : rem <= 256 ? 1.0 : 1.75);
+    // workgroups of the busiest of the eight dies (each has 32 compute units), in units of one
+    // workgroup alone on its compute unit
+    auto a_die = [&](long tiles_a_group) { return ((n_tiles + tiles_a_group - 1) / tiles_a_group * row_blocks * splits + 7) / 8; };
+    auto shared = [&](long wgs) {                  // four waves a workgroup: two workgroups share a compute unit
+        if (wgs <= 32) return 1.0;
+        const long full = wgs / 64, rem = wgs % 64;
+        return 1.75 * (double)full + (rem == 0 ? 0.0 : rem <= 32 ? 1.0 : 1.75);
     };
-    const long wgs3 = (n_tiles + 31) / 32 * row_blocks * splits;
-    const double cost2 = shared(16) * 256.0, cost4 = shared(12) * 192.0 * 1.06;
-    const double cost3 = (double)((wgs3 + 255) / 256) * 512.0 * 0.84;
+    auto alone = [&](long wgs) { return (double)((wgs + 31) / 32); };     // eight waves: one workgroup a compute unit
     const long k_steps = (K + 127) / 128, per = (k_steps + splits - 1) / splits;
-    const long wgs2 = (n_tiles + 15) / 16 * row_blocks * splits;
-    const double cost6 = (double)((wgs2 + 255) / 256) * 256.0 * 0.88;
+    const double cost2 = shared(a_die(16)) * 256.0, cost4 = shared(a_die(12)) * 192.0 * 1.06;
+    const double cost3 = alone(a_die(32)) * 512.0 * 0.84, cost6 = alone(a_die(16)) * 256.0 * 0.88;
     int best = 2;
     double cost = cost2;
     if (cost3 < cost) { best = 3; cost = cost3; }
