@@ -895,7 +895,8 @@ __device__ __forceinline__ void prefill_lds_block(
 // its place.  Keys: row = key, 16-byte chunk q of the row lies at chunk q ^ f(key) with
 // f(key) = (key & 3) | ((key >> 3) & 3) << 2 (halved for rows of 8 chunks): the 16 lanes
 // that read one chunk column for an MFMA operand (keys 8 (r/4) + 4 u + r%4) then hit 16
-// different bank groups.  Values: row = dim, 64 keys = 8 chunks, chunk q at q ^ (dim >> 1 & 7).
+// different bank groups.  Values: eight planes of 8 keys, a plane [dim][8 keys]: the 16 lanes
+// that read one plane for an MFMA operand take 256 bytes in a row.
 typedef __attribute__((address_space(3))) void lds_void_t;
 
 template <int NJ, int ND, int CT>
@@ -966,62 +967,69 @@ __device__ __forceinline__ void prefill_dma_block(
     const int wave_lo = window > 0 ? max(0, wave_first - window + 1) : 0;
     const int full_lo = window > 0 ? max(0, wave_last - window + 1) : 0, full_hi = wave_first;
 
-    // what this lane asks for in copy e of a block: for keys the row k_row[e] and the
-    // elements from k_col[e]; for values the dim row v_dim[e] and always the same 8 keys
+    const int wave_u = __builtin_amdgcn_readfirstlane(tid / 64);     // the wave, in a scalar register (for the copies' addresses)
+    // Copy w = 4 e + wave of a block (the waves take the copies in turn) moves 64 x 16 bytes: for
+    // keys the KPC rows from w KPC of the block (lane l: row l / CR, the chunk that belongs at
+    // chunk l % CR of that row); for values 64 dims of the plane w / WPP (lane l: dim
+    // (w % WPP) 64 + l, the plane's 8 keys).  A page holds at least 8 keys, so what copy e moves of
+    // the keys and what it moves of the values lies in one and the same page.  The copy's address
+    // is a base in scalar registers (the block's place in a page of more than 64 keys, the head,
+    // the page) plus an offset that a lane keeps for the whole kernel; the (at most 8) pages of a
+    // block are looked up by lanes 0..7 with one load and handed out with v_readlane.
+    constexpr int KPC = 64 / CR;                      // key rows a copy moves (4 or 8)
+    constexpr int WPP = HD / 64;                      // copies that make up a plane of values
+    static_assert(KI == VI && KPC * WPP == 8, "copy e of the keys and of the values share a page");
     auto swz_key = [](int key) {
         const int f = (key & 3) | (((key >> 3) & 3) << 2);
         return CR == 16 ? f : f >> 1;
     };
-    int k_row[KI], k_col[KI];
-    size_t v_off[VI];
+    uint32_t k_loff[KI], v_loff[VI];
+    int page_at[KI];                                  // which of the block's pages copy e wants
 #pragma unroll
     for (int e = 0; e < KI; ++e) {
-        const int slot = (e * 4 + wave) * 64 + lane;
-        k_row[e] = slot / CR;
-        k_col[e] = ((slot % CR) ^ swz_key(k_row[e])) * 8;
+        const int w = e * 4 + wave_u, first = w * KPC;  // the copy's first key in the block
+        const int k_row = first + lane / CR;
+        k_loff[e] = (uint32_t)((((first & (page_size - 1)) + lane / CR) * HD + ((lane % CR) ^ swz_key(k_row)) * 8) *
+                               sizeof(bf16_t));
+        v_loff[e] = (uint32_t)(((size_t)((w % WPP) * 64 + lane) * page_size + ((first & ~7) & (page_size - 1))) *
+                               sizeof(bf16_t));
+        page_at[e] = __builtin_amdgcn_readfirstlane(first >> page_shift);
     }
-    const int v_key8 = ((lane % CV) ^ ((((wave * 64 + lane) / CV) >> 1) & 7)) * 8;     // the same for every e
-#pragma unroll
-    for (int e = 0; e < VI; ++e) v_off[e] = (size_t)(((e * 4 + wave) * 64 + lane) / CV) * page_size;
-    const size_t head_k = (size_t)kv_head * page_size * HD, page_k = (size_t)kv_heads * page_size * HD;
-    const size_t head_v = (size_t)kv_head * HD * page_size, page_v = (size_t)kv_heads * HD * page_size;
-    int k_page[KI], v_page;
-    auto page_of = [&](int key) {
-        const int page = table[min(key >> page_shift, table_width - 1)];
-        return (unsigned)page < (unsigned)num_pages ? page : 0;      // no page: page 0, masked below
-    };
+    const uint64_t page_bytes = (uint64_t)kv_heads * page_size * HD * sizeof(bf16_t);     // of the keys, and of the values
+    const uint64_t head_bytes = (uint64_t)kv_head * page_size * HD * sizeof(bf16_t);
+    int lane_page = 0;                                // lane l < 8: page l of the block looked up last
     auto lookup = [&](int t0) {
-#pragma unroll
-        for (int e = 0; e < KI; ++e) k_page[e] = page_of(t0 + k_row[e]);
-        v_page = page_of(t0 + v_key8);
+        const int page = table[min((t0 >> page_shift) + (lane & 7), table_width - 1)];
+        lane_page = (unsigned)page < (unsigned)num_pages ? page : 0;      // no page: page 0, masked below
     };
-    // start the copies of block t0 into buffer `buf`
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)lds;
+    auto dma = [&](uint32_t lds_byte, uint32_t lane_off, uint64_t base) {
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + lds_byte);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off), "s"(base)
+                     : "m0", "memory");
+    };
+    // start the copies of block t0 (whose pages were looked up last) into buffer `buf`
     auto copy = [&](int t0, int buf) {
-        bf16_t* kb = lds + (size_t)buf * 2 * TILE;
+        const uint32_t kb = (uint32_t)buf * (uint32_t)(2 * TILE * sizeof(bf16_t));
+        const uint64_t in_page = (uint64_t)(t0 & (page_size - 1) & ~63);     // pages of more than 64 keys
+        const uint64_t k_base = (uint64_t)(uintptr_t)k_cache + head_bytes + in_page * (HD * sizeof(bf16_t));
+        const uint64_t v_base = (uint64_t)(uintptr_t)v_cache + head_bytes + in_page * sizeof(bf16_t);
 #pragma unroll
         for (int e = 0; e < KI; ++e) {
-            const int key = t0 + k_row[e];
-            const bf16_t* src = k_cache + (size_t)k_page[e] * page_k + head_k +
-                                (size_t)(key & (page_size - 1)) * HD + k_col[e];
-            __builtin_amdgcn_global_load_lds((const void*)src, (lds_void_t*)(kb + (e * 4 + wave) * 512), 16, 0, 0);
+            const uint64_t page_off = (uint64_t)(uint32_t)__builtin_amdgcn_readlane(lane_page, page_at[e]) * page_bytes;
+            dma(kb + (e * 4 + wave_u) * 1024, k_loff[e], k_base + page_off);
+            dma(kb + (uint32_t)(TILE * sizeof(bf16_t)) + (e * 4 + wave_u) * 1024, v_loff[e], v_base + page_off);
         }
-        const int vkey = t0 + v_key8;
-        const bf16_t* vbase = v_cache + (size_t)v_page * page_v + head_v + (vkey & (page_size - 1));
-#pragma unroll
-        for (int e = 0; e < VI; ++e)
-            __builtin_amdgcn_global_load_lds((const void*)(vbase + v_off[e]),
-                                             (lds_void_t*)(kb + TILE + (e * 4 + wave) * 512), 16, 0, 0);
     };
 
     // LDS offsets (elements) of this lane's fragments inside a 32-key step of a buffer
-    int ka_row[2], ka_col[NJ], vt_col[2];
+    // (values: plane 4 sub + c of the buffer, dim 16 dt + r: 16 lanes read 256 bytes in a row)
+    int ka_row[2], ka_col[NJ];
 #pragma unroll
     for (int u = 0; u < 2; ++u) ka_row[u] = (8 * (r / 4) + 4 * u + (r % 4)) * HD;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) ka_col[j] = ((c * NJ + j) ^ (CR == 16 ? r : r >> 1)) * 8;
-#pragma unroll
-    for (int sub = 0; sub < 2; ++sub) vt_col[sub] = ((sub * 4 + c) ^ (r >> 1)) * 8;
-    const int vt_row = r * KB;
+    const int vt_at = (c * HD + r) * 8;
 
     int t0 = (wg_lo / KB) * KB;
     const int t_last = (wg_last / KB) * KB;             // the last block; asked for again rather than branching
@@ -1050,7 +1058,7 @@ __device__ __forceinline__ void prefill_dma_block(
                     ka[u][j].u = *reinterpret_cast<const uint4*>(ks + sub * 32 * HD + ka_row[u] + ka_col[j]);
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt)
-                vt[dt].u = *reinterpret_cast<const uint4*>(vs + dt * 16 * KB + vt_row + vt_col[sub]);
+                vt[dt].u = *reinterpret_cast<const uint4*>(vs + (sub * 4 * HD + dt * 16) * 8 + vt_at);
             if (s0 >= full_lo && s0 + 31 <= full_hi)
                 tiles_consume<NJ, ND, CT, false>(t, ka, vt, s0 + 8 * c, 4, scale_log2);
             else
