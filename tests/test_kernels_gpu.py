@@ -412,6 +412,16 @@ ATT_CASES = [
     (8, 2, 128, 8, [200, 75], [200, 40], None),
     (4, 4, 128, 16, [300], [150], 70),
     (6, 1, 64, 32, [260, 9], [131, 9], None),
+    # long portions: many steps of 32 keys through the four LDS buffers, the block table's entries
+    # taken from a register that is filled again on the way; windows whose edges lie inside a
+    # portion (steps that need the comparison with the row's range before and after steps that do not);
+    # pages of more keys than a step
+    (8, 2, 128, 16, [2500], [2200], None),
+    (32, 8, 128, 16, [1100, 300], [1000, 37], 200),
+    (8, 4, 64, 8, [900, 40], [640, 40], 96),
+    (8, 2, 128, 64, [700], [650], None),
+    (4, 2, 128, 128, [700, 130], [333, 2], 100),
+    (4, 1, 64, 256, [600], [600], None),
 ]
 
 
@@ -419,7 +429,9 @@ PREFILL_MODES = {"bfloat16-direct": 1, "bfloat16-lds1": 2, "bfloat16-lds2": 3,
                  # the orders in which workgroups take row blocks (none, pairs in sequence, pairs that
                  # complement each other, long blocks first), which the launcher picks by the step's size
                  "bfloat16-order0": 4, "bfloat16-order1": 5, "bfloat16-order2": 6, "bfloat16-order3": 7,
-                 "bfloat16-lds1-order3": 8}
+                 "bfloat16-lds1-order3": 8,
+                 # the kernel for heads of 64 and 128 that does not overlap the phases of a step
+                 "bfloat16-unpipelined": 9}
 
 
 @pytest.mark.parametrize("dtype", DTYPES + ["bfloat16-plain"] + list(PREFILL_MODES))

@@ -27,6 +27,9 @@
 // never leave the lane's registers.  Softmax statistics are per column and
 // thus per lane (replicated over the 4 lane groups).
 #include "common.h"
+#include <type_traits>
+
+#pragma clang diagnostic ignored "-Winline-asm"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -203,6 +206,107 @@ __device__ __forceinline__ void tile_consume(Tile<NJ, ND>& t, const Frag (&ka)[2
                                              int key_c0, int u_stride, float scale_log2) {
     Tile<NJ, ND> (&one)[1] = reinterpret_cast<Tile<NJ, ND>(&)[1]>(t);
     tiles_consume<NJ, ND, 1, MASK, false>(one, ka, vt, key_c0, u_stride, scale_log2);
+}
+
+// The phases of tiles_consume as functions of their own, for a caller that overlaps them: the
+// score MFMAs of the next 32 keys run beside the vector arithmetic of these.
+template <int NJ, int ND, int CT>
+__device__ __forceinline__ void tiles_scores(const Tile<NJ, ND> (&tiles)[CT], const Frag (&ka)[2][NJ], f32x4 (&s)[CT][2]) {
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) s[ct][u] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    // (the 2 CT sums take turns, so that no MFMA waits for the one before it)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                s[ct][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[u][j].v, tiles[ct].q[j].v, s[ct][u], 0, 0, 0);
+}
+
+// Scores -> exponents of the weights, score * scale - base, in place; the bases move (and the
+// sums are rescaled) where an exponent would pass LAZY_BITS.  The maxima are taken of the
+// exponents, the results of a multiply-add, not of the MFMA's output, which the compiler would
+// first pass through a second instruction that quiets signalling NaNs.
+template <int NJ, int ND, int CT, bool MASK>
+__device__ __forceinline__ void tiles_exponents(Tile<NJ, ND> (&tiles)[CT], f32x4 (&s)[CT][2], int key_c0, int u_stride,
+                                                float scale_log2) {
+    float top[CT];
+    bool move = false;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        Tile<NJ, ND>& t = tiles[ct];
+        top[ct] = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (MASK) {
+                    const int key = key_c0 + u * u_stride + i;
+                    s[ct][u][i] = (key >= t.lo && key <= t.pos) ? s[ct][u][i] : -INFINITY;
+                }
+                s[ct][u][i] = fmaf(s[ct][u][i], scale_log2, t.nb);
+                top[ct] = fmaxf(top[ct], s[ct][u][i]);
+            }
+        // (nothing seen before: the base is -inf and nb is 0, so the first key that is seen moves the
+        // base; nothing seen now either: -inf > -inf is false)
+        move = move || top[ct] > (t.m == -INFINITY ? -INFINITY : LAZY_BITS);
+    }
+    if (__builtin_amdgcn_ballot_w64(move) != 0) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            Tile<NJ, ND>& t = tiles[ct];
+            // top is relative to the old base (-nb, 0 while nothing was seen)
+            const float m_new = fmaxf(t.m, quad_rows_max(top[ct]) - t.nb);
+            const float base = (m_new == -INFINITY) ? 0.f : m_new;
+            const float corr = __builtin_amdgcn_exp2f(t.m - base);       // exp2(-inf) = 0 the first time
+            const float shift = -base - t.nb;                            // the exponents follow the base
+            t.m = m_new;
+            t.nb = -base;
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) t.acc[dt][i] *= corr;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) t.ls[i] *= corr;
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) s[ct][u][i] += shift;
+        }
+    }
+}
+
+// Exponents -> weights, as the B operands of the output MFMAs.
+template <int CT>
+__device__ __forceinline__ void tiles_pack(const f32x4 (&s)[CT][2], Frag (&pb)[CT]) {
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        float p[2][4];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) p[u][i] = __builtin_amdgcn_exp2f(s[ct][u][i]);
+        pb[ct].u = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
+                              pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
+    }
+}
+
+// The weighted sums of the values, and the sums of the weights (a row of ones for the values).
+template <int NJ, int ND, int CT>
+__device__ __forceinline__ void tiles_output(Tile<NJ, ND> (&tiles)[CT], const Frag (&vt)[ND], const Frag (&pb)[CT]) {
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+            tiles[ct].acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt[dt].v, pb[ct].v, tiles[ct].acc[dt], 0, 0, 0);
+    Frag ones;
+    ones.u = make_uint4(0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u);
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+        tiles[ct].ls = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pb[ct].v, tiles[ct].ls, 0, 0, 0);
 }
 
 // Process the 32 keys t0 .. t0+31 (t0 a multiple of 32) for CT column tiles that
@@ -1084,6 +1188,259 @@ __device__ __forceinline__ void prefill_dma_block(
     }
 }
 
+// -------------------------- prefill, copied straight into LDS, phases overlapped --
+// The same work once more for heads of 64 and 128, in steps of 32 keys through four LDS
+// buffers, with the phases of a wave's step overlapped: while the matrix pipeline works on the
+// scores of step i+1 the vector units turn the exponents of step i into weights, and while it
+// adds up the values of step i they turn the scores of step i+1 into exponents.  A wave
+// issues one instruction at a time, and an MFMA that waits for the pipeline holds up what
+// follows it, so the two kinds stand interleaved in the program.
+//   top of iteration i:  block i+1 has landed (the copies of block i+2 may still be under way),
+//                        barrier, start the copy of block i+3 into the buffer that block i-1 left
+//   then:                key fragments of step i+1 and value fragments of step i from LDS,
+//                        weights of step i, scores of step i+1, output of step i, exponents of
+//                        step i+1 (its bases may move: the sums are rescaled after the output)
+// A wave sees the steps a..b of the workgroup's 0..n-1 (late rows see more keys than early
+// ones); before and after them it only takes part in the barriers and the copies.
+// (WAVES = 8, one workgroup a compute unit that asks the L2 caches for every key half as
+// often, was measured 3 to 6% slower than two workgroups of four.)
+template <int NJ, int ND, int CT, int WAVES>
+__device__ __forceinline__ void prefill_pipe_block(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int* __restrict__ row_start,
+    const int* __restrict__ seq_start, int num_seqs, const int* __restrict__ tables, int table_width,
+    int page_size, int page_shift, int num_pages, int heads, int kv_heads, float scale_log2, int window,
+    int rq, int block, int head_index, const RawQkv& raw) {
+    static_assert(ND == 2 * NJ && (ND == 4 || ND == 8), "heads of 64 or 128");
+    constexpr int KB = 32;
+    constexpr int HD = ND * 16;
+    constexpr int CR = HD / 8;                        // 16-byte chunks of a key row
+    constexpr int KI = KB * CR / (64 * WAVES), VI = HD * 4 / (64 * WAVES);     // copies a wave issues for a block: keys, values
+    static_assert(KI >= 1 && VI >= 1, "every wave takes part in the copies");
+    constexpr int PER = KI + VI;
+    constexpr int TILE = KB * HD;                     // elements of a block's keys (and of its values)
+    extern __shared__ uint4 lds_raw[];
+    bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw); // buffer b: keys at b * 2 TILE, values TILE further
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
+    const int group = heads / kv_heads;
+    const int head_tiles = (group + 15) / 16;
+    const int kv_head = head_index / head_tiles, head_tile = head_index % head_tiles;
+    const int heads_here = min(16, group - head_tile * 16);
+    const int rows_per_wave = CT * rq, rows_per_block = WAVES * rows_per_wave;
+    int seq = 0, first_row = 0, n_rows = 0;
+    for (; seq < num_seqs; ++seq) {
+        first_row = row_start[seq];
+        n_rows = row_start[seq + 1] - first_row;
+        const int blocks = (n_rows + rows_per_block - 1) / rows_per_block;
+        if (block < blocks) break;
+        block -= blocks;
+    }
+    if (seq >= num_seqs) return;                      // the whole workgroup leaves together
+    const int start = seq_start[seq];
+    const int block0 = block * rows_per_block;        // first row of the workgroup in the portion
+    const int block_rows = min(rows_per_block, n_rows - block0);
+    const int local0 = block0 + wave * rows_per_wave;
+    const int wave_rows = max(0, min(rows_per_wave, n_rows - local0));
+    const int col_row = r / heads_here, col_head = head_tile * 16 + r % heads_here;
+    const int head = kv_head * group + col_head;
+    const int* table = tables + (size_t)seq * table_width;
+
+    Tile<NJ, ND> t[CT];
+    bool live[CT];
+    int row[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int local = ct * rq + col_row;
+        live[ct] = col_row < rq && local < wave_rows;
+        row[ct] = first_row + (live[ct] ? local0 + local : 0);
+        const int pos = start + local0 + local;
+        tile_init(t[ct]);
+        t[ct].pos = live[ct] ? pos : -1;
+        t[ct].lo = live[ct] ? (window > 0 ? max(0, pos - window + 1) : 0) : 0;
+        if (raw.qkv) {
+            const int at = live[ct] ? pos : start;
+            const float* cos_row = raw.cos ? raw.cos + (size_t)at * (HD / 2) : nullptr;
+            const float* sin_row = raw.cos ? raw.sin + (size_t)at * (HD / 2) : nullptr;
+            head_from_raw<NJ>(t[ct].q, raw.qkv + ((size_t)row[ct] * (heads + 2 * kv_heads) + head) * HD,
+                              raw.q_norm_w, raw.q_eps, cos_row, sin_row);
+        } else {
+            tile_load_q(t[ct], q + ((size_t)row[ct] * heads + head) * HD, HD, live[ct]);
+        }
+    }
+    const int wg_first = start + block0, wg_last = wg_first + block_rows - 1;
+    const int wg_lo = window > 0 ? max(0, wg_first - window + 1) : 0;
+    const int wave_first = start + local0, wave_last = wave_first + wave_rows - 1;
+    const int wave_lo = window > 0 ? max(0, wave_first - window + 1) : 0;
+    // the steps: the workgroup's 0..n-1 from key T0, this wave's a..b, of which f0..f1-1 are seen
+    // whole by every row of the wave (the others need the comparison of every key with the row's range)
+    const int T0 = (wg_lo / KB) * KB;
+    const int n = (wg_last - T0) / KB + 1;
+    const int full_lo = window > 0 ? max(0, wave_last - window + 1) : 0, full_hi = wave_first;
+    // (the same for a whole wave, and said so: the loops below then run on scalar registers)
+    const int a = __builtin_amdgcn_readfirstlane(wave_rows > 0 ? (wave_lo - T0) / KB : n + 1);
+    const int b = __builtin_amdgcn_readfirstlane(wave_rows > 0 ? (wave_last - T0) / KB : n);
+    const int f0 = __builtin_amdgcn_readfirstlane(full_lo <= T0 ? 0 : (full_lo - T0 + KB - 1) / KB);
+    const int f1 = __builtin_amdgcn_readfirstlane((full_hi - T0 + 1) / KB);
+    auto whole = [&](int step) { return step >= f0 && step < f1; };
+
+    const int wave_u = __builtin_amdgcn_readfirstlane(tid / 64);     // the wave, in a scalar register (for the copies' addresses)
+    // Copy w = WAVES e + wave of a block moves 64 x 16 bytes: for keys the KPC rows from w KPC of the
+    // block (lane l: row l / CR, the chunk that belongs at chunk l % CR of that row, rows swizzled
+    // as in prefill_dma_block); for values 64 dims of the plane w / WPP (lane l: dim
+    // (w % WPP) 64 + l, the plane's 8 keys).  A page holds at least 8 keys, so what copy e moves of
+    // the keys and of the values lies in one page.  An address is a base in scalar registers plus
+    // an offset that a lane keeps for the whole kernel.
+    constexpr int KPC = 64 / CR;                      // key rows a copy moves (4 or 8)
+    constexpr int WPP = HD / 64;                      // copies that make up a plane of values
+    static_assert(KI == VI && KPC * WPP == 8, "copy e of the keys and of the values share a page");
+    auto swz_key = [](int key) {
+        const int f = (key & 3) | (((key >> 3) & 3) << 2);
+        return CR == 16 ? f : f >> 1;
+    };
+    uint32_t k_loff[KI], v_loff[VI];
+#pragma unroll
+    for (int e = 0; e < KI; ++e) {
+        const int w = e * WAVES + wave_u, first = w * KPC;  // the copy's first key in the block
+        const int k_row = first + lane / CR;
+        k_loff[e] = (uint32_t)((((first & (page_size - 1)) + lane / CR) * HD + ((lane % CR) ^ swz_key(k_row)) * 8) *
+                               sizeof(bf16_t));
+        v_loff[e] = (uint32_t)(((size_t)((w % WPP) * 64 + lane) * page_size + ((first & ~7) & (page_size - 1))) *
+                               sizeof(bf16_t));
+    }
+    const uint64_t page_bytes = (uint64_t)kv_heads * page_size * HD * sizeof(bf16_t);     // of the keys, and of the values
+    const uint64_t head_bytes = (uint64_t)kv_head * page_size * HD * sizeof(bf16_t);
+    // 64 entries of the block table at a time live in the lanes of one register (entry
+    // tab_first + l in lane l, those that name no page made 0: such keys are masked); a copy takes
+    // its page from there with v_readlane.  The register is filled again every 16 blocks, which
+    // walk at most 64 entries (pages of 8 keys).
+    int tab_first = 0, tab_pages = 0;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)lds;
+    // one copy of 64 x 16 bytes: LDS place (bytes from the start of the buffers) <- base + the lane's offset
+    auto dma = [&](uint32_t lds_byte, uint32_t lane_off, uint64_t base) {
+        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
+                     ::"s"(lds_base), "s"(lds_byte), "v"(lane_off), "s"(base)
+                     : "m0", "scc", "memory");
+    };
+    // start the copies of block `step` into its buffer (called for every step in turn; past the
+    // last block the last one is copied again, rather than a branch that would change what is in flight)
+    auto copy = [&](int step) {
+        const int t0 = T0 + min(step, n - 1) * KB;
+        if ((step & 15) == 0) {
+            tab_first = t0 >> page_shift;
+            // (loaded and waited for in assembly, like the copies: the compiler then knows of no load
+            // in the loop and leaves the counting of those in flight to the waits written here)
+            int page;
+            asm volatile("global_load_dword %0, %1, off\n\ts_waitcnt vmcnt(0)"
+                         : "=v"(page)
+                         : "v"(table + min(tab_first + lane, table_width - 1))
+                         : "memory");
+            tab_pages = (unsigned)page < (unsigned)num_pages ? page : 0;
+        }
+        const uint32_t kb = (uint32_t)(step & 3) * (uint32_t)(2 * TILE * sizeof(bf16_t));
+        const uint64_t in_page = (uint64_t)(t0 & (page_size - 1) & ~(KB - 1));     // pages of more than 32 keys
+        const uint64_t k_base = (uint64_t)(uintptr_t)k_cache + head_bytes + in_page * (HD * sizeof(bf16_t));
+        const uint64_t v_base = (uint64_t)(uintptr_t)v_cache + head_bytes + in_page * sizeof(bf16_t);
+#pragma unroll
+        for (int e = 0; e < KI; ++e) {
+            const int entry = (t0 + (e * WAVES + wave_u) * KPC) >> page_shift;
+            const uint64_t page_off = (uint64_t)(uint32_t)__builtin_amdgcn_readlane(tab_pages, entry - tab_first) * page_bytes;
+            dma(kb + (e * WAVES + wave_u) * 1024, k_loff[e], k_base + page_off);
+            dma(kb + (uint32_t)(TILE * sizeof(bf16_t)) + (e * WAVES + wave_u) * 1024, v_loff[e], v_base + page_off);
+        }
+    };
+    // the top of iteration i
+    auto top = [&](int i) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER) : "memory");     // this wave's part of block i+1 has landed
+        __syncthreads();                                               // everyone's has, and nobody reads block i-1 any more
+        copy(i + 3);
+    };
+
+    // LDS offsets (elements) of this lane's fragments in a buffer (values: plane c, dim 16 dt + r)
+    int ka_row[2], ka_col[NJ];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) ka_row[u] = (8 * (r / 4) + 4 * u + (r % 4)) * HD;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) ka_col[j] = ((c * NJ + j) ^ (CR == 16 ? r : r >> 1)) * 8;
+    const int vt_at = TILE + (c * HD + r) * 8;
+    auto keys_of = [&](int step, Frag (&ka)[2][NJ]) {
+        const bf16_t* ks = lds + (size_t)(step & 3) * 2 * TILE;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) ka[u][j].u = *reinterpret_cast<const uint4*>(ks + ka_row[u] + ka_col[j]);
+    };
+    auto values_of = [&](int step, Frag (&vt)[ND]) {
+        const bf16_t* vs = lds + (size_t)(step & 3) * 2 * TILE + vt_at;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) vt[dt].u = *reinterpret_cast<const uint4*>(vs + dt * 16 * 8);
+    };
+
+    f32x4 ex[CT][2];                                  // the exponents of the step whose weights come next
+    copy(0);
+    copy(1);
+    int i = -1;
+    for (; i < a - 1; ++i) top(i);                    // blocks before this wave's keys
+    if (a <= b) {
+        {                                             // i == a - 1: the scores of the wave's first step
+            top(i);
+            Frag ka[2][NJ];
+            keys_of(a, ka);
+            tiles_scores<NJ, ND, CT>(t, ka, ex);
+            if (whole(a))
+                tiles_exponents<NJ, ND, CT, false>(t, ex, T0 + a * KB + 8 * c, 4, scale_log2);
+            else
+                tiles_exponents<NJ, ND, CT, true>(t, ex, T0 + a * KB + 8 * c, 4, scale_log2);
+            ++i;
+        }
+        auto round = [&](auto MASK_T) {
+            constexpr bool MASK = decltype(MASK_T)::value;
+            top(i);
+            Frag ka[2][NJ], vt[ND], pb[CT];
+            f32x4 sc[CT][2];
+            keys_of(i + 1, ka);
+            values_of(i, vt);
+            tiles_pack<CT>(ex, pb);
+            tiles_scores<NJ, ND, CT>(t, ka, sc);
+            tiles_output<NJ, ND, CT>(t, vt, pb);
+            tiles_exponents<NJ, ND, CT, MASK>(t, sc, T0 + (i + 1) * KB + 8 * c, 4, scale_log2);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) ex[ct][u] = sc[ct][u];
+        };
+        while (i < b) {
+            for (; i < b && whole(i + 1); ++i) round(std::false_type{});     // the step after i is seen whole
+            for (; i < b && !whole(i + 1); ++i) round(std::true_type{});
+        }
+        {                                             // i == b: the output of the wave's last step
+            top(i);
+            Frag vt[ND], pb[CT];
+            values_of(b, vt);
+            tiles_pack<CT>(ex, pb);
+            tiles_output<NJ, ND, CT>(t, vt, pb);
+            ++i;
+        }
+    }
+    for (; i < n; ++i) top(i);                        // blocks after this wave's keys
+    // the copies that the last rounds started land before anything else uses the buffers
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        if (!live[ct]) continue;
+        const float l = tile_sum(t[ct]);
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        bf16_t* o = out + ((size_t)row[ct] * heads + head) * HD;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) {
+            uint2 packed;
+            packed.x = pack_bf16x2(t[ct].acc[dt][0] * inv, t[ct].acc[dt][1] * inv);
+            packed.y = pack_bf16x2(t[ct].acc[dt][2] * inv, t[ct].acc[dt][3] * inv);
+            *reinterpret_cast<uint2*>(o + dt * 16 + 4 * c) = packed;
+        }
+    }
+}
+
 // With raw.qkv the queries are taken from the raw projections (normed and rotated here, q
 // is not read); needs head_dim == 32*NJ.  DMA: blocks are copied straight into LDS
 // (prefill_dma_block; heads of 64 and 128).
@@ -1091,86 +1448,68 @@ __device__ __forceinline__ void prefill_dma_block(
 // than early ones; `pair` says how the work is evened out: 1: (ceil(row blocks / 2), ...)
 // workgroups that each take block (last - b) and then block b; 2: long blocks placed beside
 // short ones on a compute unit; 3: long blocks first; 0: as the grid says.
-template <int NJ, int ND, int CT, int KB, bool DMA>
-__global__ void __launch_bounds__(256, (ND <= 8 && (CT == 2 || DMA)) ? 2 : 1)
+template <int NJ, int ND, int CT, int KB, bool DMA, int WAVES = 4>
+__global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && ND <= 8 && (CT == 2 || DMA)) ? 2 : 1)
 attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                              const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                              const int* __restrict__ row_start, const int* __restrict__ seq_start,
                              int num_seqs, const int* __restrict__ tables, int table_width, int page_size,
                              int page_shift, int num_pages, int heads, int kv_heads,
                              float scale_log2, int window, int rq, int pair, RawQkv raw) {
-    const int rows_per_block = 4 * CT * rq;
+    const int rows_per_block = WAVES * CT * rq;
     int total = 0;
     for (int seq = 0; seq < num_seqs; ++seq)
         total += (row_start[seq + 1] - row_start[seq] + rows_per_block - 1) / rows_per_block;
     const int head_count = gridDim.y;
+    // the row block and head (and for pair = 1 a second row block) of this workgroup
+    int rb, hd_i = blockIdx.y, rb2 = -1;
     if (pair == 2) {
         // All workgroups are resident at once, two a compute unit, and late row blocks walk
         // more keys than early ones.  Workgroups are handed to the compute units in order
         // of their linear index, so index L and index L + total/2 tend to share a unit: the
         // second half of the indices gets the row blocks in reverse order (and the other
         // half of the heads), which puts a long block beside a short one.
-        const int all = total * head_count, half = all / 2;
-        const int linear = blockIdx.y * gridDim.x + blockIdx.x;
+        const int half = total * head_count / 2;
         if (blockIdx.x >= total) return;                       // the grid's slack
         const int lin = blockIdx.y * total + blockIdx.x;       // index among the real workgroups
-        int rb, hd_i;
         if (head_count % 2 == 0) {
             const int round = lin / half, p = lin % half;
             rb = round == 0 ? p % total : total - 1 - p % total;
             hd_i = p / total + round * (head_count / 2);
         } else {
             rb = blockIdx.x;
-            hd_i = blockIdx.y;
         }
-        (void)linear;
-        if constexpr (DMA)
-            prefill_dma_block<NJ, ND, CT>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
-                                          table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                          scale_log2, window, rq, rb, hd_i, raw);
-        else
-            prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
-                                          table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                          scale_log2, window, rq, rb, hd_i, raw);
-        return;
-    }
-    if (pair == 3) {
+    } else if (pair == 3) {
         // Long row blocks first: workgroups are handed out in the order of their index as
         // compute units become free, so the short blocks fill the gaps the long ones leave.
         // The heads vary fastest, so that what runs at the same time walks similar key ranges.
         if (blockIdx.x >= total) return;                      // the grid's slack
         const int idx = blockIdx.y * total + blockIdx.x;      // index among the real workgroups
-        const int rb = total - 1 - idx / head_count, hd_i = idx % head_count;
-        if constexpr (DMA)
-            prefill_dma_block<NJ, ND, CT>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
-                                          table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                          scale_log2, window, rq, rb, hd_i, raw);
-        else
-            prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
-                                          table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                          scale_log2, window, rq, rb, hd_i, raw);
-        return;
+        rb = total - 1 - idx / head_count;
+        hd_i = idx % head_count;
+    } else {
+        const int first = blockIdx.x, second = pair ? total - 1 - first : first;
+        if (first >= total || first > second) return;
+        rb = second;
+        if (second != first) rb2 = first;
     }
-    const int first = blockIdx.x, second = pair ? total - 1 - first : first;
-    if (first >= total || first > second) return;
-    if constexpr (DMA)
-            prefill_dma_block<NJ, ND, CT>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
-                                      table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                      scale_log2, window, rq, second, blockIdx.y, raw);
-        else
-            prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
-                                      table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                      scale_log2, window, rq, second, blockIdx.y, raw);
-    if (second != first) {
-        __syncthreads();
-        if constexpr (DMA)
+    for (;;) {
+        if constexpr (DMA && KB == 32)
+            prefill_pipe_block<NJ, ND, CT, WAVES>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+                                                  table_width, page_size, page_shift, num_pages, heads, kv_heads,
+                                                  scale_log2, window, rq, rb, hd_i, raw);
+        else if constexpr (DMA)
             prefill_dma_block<NJ, ND, CT>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                           table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                          scale_log2, window, rq, first, blockIdx.y, raw);
+                                          scale_log2, window, rq, rb, hd_i, raw);
         else
             prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
-                                          table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                          scale_log2, window, rq, first, blockIdx.y, raw);
+                                              table_width, page_size, page_shift, num_pages, heads, kv_heads,
+                                              scale_log2, window, rq, rb, hd_i, raw);
+        if (rb2 < 0) break;
+        rb = rb2;
+        rb2 = -1;
+        __syncthreads();                                      // (the buffers are used again)
     }
 }
 
@@ -1322,6 +1661,7 @@ static int launch_prefill(
         if (direct == 2) two = false;
         if (direct == 3 || (direct >= 4 && direct <= 7)) two = head_dim <= 128;
         if (direct == 8) two = false;
+        const bool pipe = direct != 9;                            // (9: the kernel that does not overlap the phases of a step)
         const int rows_per_block = 4 * rq * (two ? 2 : 1);
         const long blocks = (rows + rows_per_block - 1) / rows_per_block + num_seqs;   // upper bound
         if (blocks > 2147483647L) return tli_fail("attention_prefill: too many rows");
@@ -1340,7 +1680,9 @@ static int launch_prefill(
 #define TAIL_LDS scale * LOG2E, window, rq, pair, raw
 #define LDS_CALL(NJ, ND, CT, KB, DMA) attention_prefill_lds_kernel<NJ, ND, CT, KB, DMA><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS)
 #define CALL(NJ, ND)                                                                                    \
-    if ((ND == 4 || ND == 8) && two) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 2, 64, true); \
+    if ((ND == 4 || ND == 8) && two && pipe) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 2, 32, true); \
+    else if ((ND == 4 || ND == 8) && pipe) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 1, 32, true); \
+    else if ((ND == 4 || ND == 8) && two) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 2, 64, true); \
     else if (ND == 4 || ND == 8) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 1, 64, true); \
     else if (ND <= 8 && two) LDS_CALL(NJ, ((ND <= 8 && ND != 4 && ND != 8) ? ND : 1), 2, 64, false);    \
     else if (ND <= 8) LDS_CALL(NJ, ((ND <= 8 && ND != 4 && ND != 8) ? ND : 1), 1, 64, false);           \
