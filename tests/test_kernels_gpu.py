@@ -429,9 +429,7 @@ PREFILL_MODES = {"bfloat16-direct": 1, "bfloat16-lds1": 2, "bfloat16-lds2": 3,
                  # the orders in which workgroups take row blocks (none, pairs in sequence, pairs that
                  # complement each other, long blocks first), which the launcher picks by the step's size
                  "bfloat16-order0": 4, "bfloat16-order1": 5, "bfloat16-order2": 6, "bfloat16-order3": 7,
-                 "bfloat16-lds1-order3": 8,
-                 # the kernel for heads of 64 and 128 that does not overlap the phases of a step
-                 "bfloat16-unpipelined": 9}
+                 "bfloat16-lds1-order3": 8}
 
 
 @pytest.mark.parametrize("dtype", DTYPES + ["bfloat16-plain"] + list(PREFILL_MODES))

@@ -30,6 +30,7 @@ to a page id, -1 where no page is held.
 """
 from __future__ import annotations
 
+from array import array
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
@@ -110,6 +111,28 @@ class GroupLayout:
         return self.cache_layers.index(cache_layer)
 
 
+class PageTable(array):
+    """The block table of a request in one group: block -> page id or -1, 32-bit integers in
+    one piece of memory, so that a step packs it into its inputs with one copy
+    (``numpy.frombuffer``) however long it has grown.  Reads like a list: equal to any sequence of
+    the same numbers, and a slice of it is a list."""
+
+    def __new__(cls, pages=()):
+        return super().__new__(cls, "i", pages)
+
+    def __eq__(self, other):
+        return list(self) == list(other)
+
+    def __ne__(self, other):
+        return not self.__eq__(other)
+
+    __hash__ = None
+
+    def __getitem__(self, index):
+        item = super().__getitem__(index)
+        return item.tolist() if isinstance(index, slice) else item
+
+
 @dataclass
 class RequestCache:
     """What one live request holds."""
@@ -118,7 +141,7 @@ class RequestCache:
     num_tokens: int = 0                               # tokens whose keys are in the cache
     hashed_blocks: int = 0                            # leading pages already in the prefix cache
     prefix_hash: int = 0                              # chained hash of those pages
-    tables: List[List[int]] = field(default_factory=list)   # per group: block -> page or -1
+    tables: List[PageTable] = field(default_factory=list)    # per group: block -> page or -1
     reserved_tokens: int = 0                          # positions [0, reserved) are covered
 
 
@@ -199,7 +222,7 @@ class CacheManager:
         if not self._free_slots:
             raise CacheFull("no state slot is free")
         slot = self._free_slots.pop()
-        rc = RequestCache(key=key, slot=slot, tables=[[] for _ in self.groups])
+        rc = RequestCache(key=key, slot=slot, tables=[PageTable() for _ in self.groups])
         self._live[key] = rc
         return rc
 
@@ -360,7 +383,7 @@ class CacheManager:
                 if page >= 0:
                     g.pool.release(page)
                     self.pages_returned_total += 1
-            rc.tables[gi] = []
+            rc.tables[gi] = PageTable()
         self._free_slots.append(rc.slot)
         self._free_slots.sort(reverse=True)
 

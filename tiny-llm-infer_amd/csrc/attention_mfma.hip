@@ -987,210 +987,21 @@ __device__ __forceinline__ void prefill_lds_block(
     }
 }
 
-// ------------------------------------- prefill, blocks copied straight into LDS --
-// The same work again for heads of 64 and 128 (ND = 4, 8; NJ = ND/2), with the blocks of
-// 64 keys copied from the cache into LDS by the memory pipeline itself
-// (global_load_lds_dwordx4: lane l of a wave writes the 16 bytes it asked for at LDS
-// base + 16 l), into one of two buffers: the next block is on its way while this one is
-// multiplied, no register holds it meanwhile, and one barrier a block is enough.
-//
-// Such a copy leaves no room for padding between rows, so rows are swizzled instead: a
-// lane chooses which 16 bytes of the cache it asks for, and asks for those that belong at
-// its place.  Keys: row = key, 16-byte chunk q of the row lies at chunk q ^ f(key) with
-// f(key) = (key & 3) | ((key >> 3) & 3) << 2 (halved for rows of 8 chunks): the 16 lanes
-// that read one chunk column for an MFMA operand (keys 8 (r/4) + 4 u + r%4) then hit 16
-// different bank groups.  Values: eight planes of 8 keys, a plane [dim][8 keys]: the 16 lanes
-// that read one plane for an MFMA operand take 256 bytes in a row.
 typedef __attribute__((address_space(3))) void lds_void_t;
 
-template <int NJ, int ND, int CT>
-__device__ __forceinline__ void prefill_dma_block(
-    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
-    const bf16_t* __restrict__ v_cache, const int* __restrict__ row_start,
-    const int* __restrict__ seq_start, int num_seqs, const int* __restrict__ tables, int table_width,
-    int page_size, int page_shift, int num_pages, int heads, int kv_heads, float scale_log2, int window,
-    int rq, int block, int head_index, const RawQkv& raw) {
-    static_assert(ND == 2 * NJ && (ND == 4 || ND == 8), "heads of 64 or 128");
-    constexpr int KB = 64;
-    constexpr int HD = ND * 16;
-    constexpr int CR = HD / 8;                        // 16-byte chunks of a key row
-    constexpr int CV = KB / 8;                        // 16-byte chunks of a value (dim) row
-    constexpr int KI = KB * CR / 256, VI = HD * CV / 256;       // copies a wave issues for a block
-    constexpr int TILE = KB * HD;                     // elements of a block's keys (and of its values)
-    extern __shared__ uint4 lds_raw[];
-    bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw); // buffer b: keys at b * 2 TILE, values TILE further
-    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
-    const int group = heads / kv_heads;
-    const int head_tiles = (group + 15) / 16;
-    const int kv_head = head_index / head_tiles, head_tile = head_index % head_tiles;
-    const int heads_here = min(16, group - head_tile * 16);
-    const int rows_per_wave = CT * rq, rows_per_block = 4 * rows_per_wave;
-    int seq = 0, first_row = 0, n_rows = 0;
-    for (; seq < num_seqs; ++seq) {
-        first_row = row_start[seq];
-        n_rows = row_start[seq + 1] - first_row;
-        const int blocks = (n_rows + rows_per_block - 1) / rows_per_block;
-        if (block < blocks) break;
-        block -= blocks;
-    }
-    if (seq >= num_seqs) return;                      // the whole workgroup leaves together
-    const int start = seq_start[seq];
-    const int block0 = block * rows_per_block;        // first row of the workgroup in the portion
-    const int block_rows = min(rows_per_block, n_rows - block0);
-    const int local0 = block0 + wave * rows_per_wave;
-    const int wave_rows = max(0, min(rows_per_wave, n_rows - local0));
-    const int col_row = r / heads_here, col_head = head_tile * 16 + r % heads_here;
-    const int head = kv_head * group + col_head;
-    const int* table = tables + (size_t)seq * table_width;
-
-    Tile<NJ, ND> t[CT];
-    bool live[CT];
-    int row[CT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        const int local = ct * rq + col_row;
-        live[ct] = col_row < rq && local < wave_rows;
-        row[ct] = first_row + (live[ct] ? local0 + local : 0);
-        const int pos = start + local0 + local;
-        tile_init(t[ct]);
-        t[ct].pos = live[ct] ? pos : -1;
-        t[ct].lo = live[ct] ? (window > 0 ? max(0, pos - window + 1) : 0) : 0;
-        if (raw.qkv) {
-            const int at = live[ct] ? pos : start;
-            const float* cos_row = raw.cos ? raw.cos + (size_t)at * (HD / 2) : nullptr;
-            const float* sin_row = raw.cos ? raw.sin + (size_t)at * (HD / 2) : nullptr;
-            head_from_raw<NJ>(t[ct].q, raw.qkv + ((size_t)row[ct] * (heads + 2 * kv_heads) + head) * HD,
-                              raw.q_norm_w, raw.q_eps, cos_row, sin_row);
-        } else {
-            tile_load_q(t[ct], q + ((size_t)row[ct] * heads + head) * HD, HD, live[ct]);
-        }
-    }
-    const int wg_first = start + block0, wg_last = wg_first + block_rows - 1;
-    const int wg_lo = window > 0 ? max(0, wg_first - window + 1) : 0;
-    const int wave_first = start + local0, wave_last = wave_first + wave_rows - 1;
-    const int wave_lo = window > 0 ? max(0, wave_first - window + 1) : 0;
-    const int full_lo = window > 0 ? max(0, wave_last - window + 1) : 0, full_hi = wave_first;
-
-    const int wave_u = __builtin_amdgcn_readfirstlane(tid / 64);     // the wave, in a scalar register (for the copies' addresses)
-    // Copy w = 4 e + wave of a block (the waves take the copies in turn) moves 64 x 16 bytes: for
-    // keys the KPC rows from w KPC of the block (lane l: row l / CR, the chunk that belongs at
-    // chunk l % CR of that row); for values 64 dims of the plane w / WPP (lane l: dim
-    // (w % WPP) 64 + l, the plane's 8 keys).  A page holds at least 8 keys, so what copy e moves of
-    // the keys and what it moves of the values lies in one and the same page.  The copy's address
-    // is a base in scalar registers (the block's place in a page of more than 64 keys, the head,
-    // the page) plus an offset that a lane keeps for the whole kernel; the (at most 8) pages of a
-    // block are looked up by lanes 0..7 with one load and handed out with v_readlane.
-    constexpr int KPC = 64 / CR;                      // key rows a copy moves (4 or 8)
-    constexpr int WPP = HD / 64;                      // copies that make up a plane of values
-    static_assert(KI == VI && KPC * WPP == 8, "copy e of the keys and of the values share a page");
-    auto swz_key = [](int key) {
-        const int f = (key & 3) | (((key >> 3) & 3) << 2);
-        return CR == 16 ? f : f >> 1;
-    };
-    uint32_t k_loff[KI], v_loff[VI];
-    int page_at[KI];                                  // which of the block's pages copy e wants
-#pragma unroll
-    for (int e = 0; e < KI; ++e) {
-        const int w = e * 4 + wave_u, first = w * KPC;  // the copy's first key in the block
-        const int k_row = first + lane / CR;
-        k_loff[e] = (uint32_t)((((first & (page_size - 1)) + lane / CR) * HD + ((lane % CR) ^ swz_key(k_row)) * 8) *
-                               sizeof(bf16_t));
-        v_loff[e] = (uint32_t)(((size_t)((w % WPP) * 64 + lane) * page_size + ((first & ~7) & (page_size - 1))) *
-                               sizeof(bf16_t));
-        page_at[e] = __builtin_amdgcn_readfirstlane(first >> page_shift);
-    }
-    const uint64_t page_bytes = (uint64_t)kv_heads * page_size * HD * sizeof(bf16_t);     // of the keys, and of the values
-    const uint64_t head_bytes = (uint64_t)kv_head * page_size * HD * sizeof(bf16_t);
-    int lane_page = 0;                                // lane l < 8: page l of the block looked up last
-    auto lookup = [&](int t0) {
-        const int page = table[min((t0 >> page_shift) + (lane & 7), table_width - 1)];
-        lane_page = (unsigned)page < (unsigned)num_pages ? page : 0;      // no page: page 0, masked below
-    };
-    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)lds;
-    auto dma = [&](uint32_t lds_byte, uint32_t lane_off, uint64_t base) {
-        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + lds_byte);
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off), "s"(base)
-                     : "m0", "memory");
-    };
-    // start the copies of block t0 (whose pages were looked up last) into buffer `buf`
-    auto copy = [&](int t0, int buf) {
-        const uint32_t kb = (uint32_t)buf * (uint32_t)(2 * TILE * sizeof(bf16_t));
-        const uint64_t in_page = (uint64_t)(t0 & (page_size - 1) & ~63);     // pages of more than 64 keys
-        const uint64_t k_base = (uint64_t)(uintptr_t)k_cache + head_bytes + in_page * (HD * sizeof(bf16_t));
-        const uint64_t v_base = (uint64_t)(uintptr_t)v_cache + head_bytes + in_page * sizeof(bf16_t);
-#pragma unroll
-        for (int e = 0; e < KI; ++e) {
-            const uint64_t page_off = (uint64_t)(uint32_t)__builtin_amdgcn_readlane(lane_page, page_at[e]) * page_bytes;
-            dma(kb + (e * 4 + wave_u) * 1024, k_loff[e], k_base + page_off);
-            dma(kb + (uint32_t)(TILE * sizeof(bf16_t)) + (e * 4 + wave_u) * 1024, v_loff[e], v_base + page_off);
-        }
-    };
-
-    // LDS offsets (elements) of this lane's fragments inside a 32-key step of a buffer
-    // (values: plane 4 sub + c of the buffer, dim 16 dt + r: 16 lanes read 256 bytes in a row)
-    int ka_row[2], ka_col[NJ];
-#pragma unroll
-    for (int u = 0; u < 2; ++u) ka_row[u] = (8 * (r / 4) + 4 * u + (r % 4)) * HD;
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) ka_col[j] = ((c * NJ + j) ^ (CR == 16 ? r : r >> 1)) * 8;
-    const int vt_at = (c * HD + r) * 8;
-
-    int t0 = (wg_lo / KB) * KB;
-    const int t_last = (wg_last / KB) * KB;             // the last block; asked for again rather than branching
-    lookup(t0);
-    copy(t0, 0);
-    lookup(min(t0 + KB, t_last));
-    int buf = 0;
-    for (; t0 <= wg_last; t0 += KB, buf ^= 1) {
-        // this block has arrived (every lane waits for its own copies, then for the others),
-        // and everyone has finished reading the other buffer
-        __builtin_amdgcn_s_waitcnt(0x0F70);             // vmcnt(0)
-        __syncthreads();
-        copy(min(t0 + KB, t_last), buf ^ 1);
-        lookup(min(t0 + 2 * KB, t_last));
-        const bf16_t* ks = lds + (size_t)buf * 2 * TILE;
-        const bf16_t* vs = ks + TILE;
-#pragma unroll
-        for (int sub = 0; sub < KB / 32; ++sub) {
-            const int s0 = t0 + sub * 32;
-            if (wave_rows <= 0 || s0 > wave_last || s0 + 31 < wave_lo) continue;   // nothing this wave sees
-            Frag ka[2][NJ], vt[ND];
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int j = 0; j < NJ; ++j)
-                    ka[u][j].u = *reinterpret_cast<const uint4*>(ks + sub * 32 * HD + ka_row[u] + ka_col[j]);
-#pragma unroll
-            for (int dt = 0; dt < ND; ++dt)
-                vt[dt].u = *reinterpret_cast<const uint4*>(vs + (sub * 4 * HD + dt * 16) * 8 + vt_at);
-            if (s0 >= full_lo && s0 + 31 <= full_hi)
-                tiles_consume<NJ, ND, CT, false>(t, ka, vt, s0 + 8 * c, 4, scale_log2);
-            else
-                tiles_consume<NJ, ND, CT, true>(t, ka, vt, s0 + 8 * c, 4, scale_log2);
-        }
-    }
-    // the copy that the last round started lands before anything else uses the buffers
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        if (!live[ct]) continue;
-        const float l = tile_sum(t[ct]);
-        const float inv = l > 0.f ? 1.0f / l : 0.f;
-        bf16_t* o = out + ((size_t)row[ct] * heads + head) * HD;
-#pragma unroll
-        for (int dt = 0; dt < ND; ++dt) {
-            uint2 packed;
-            packed.x = pack_bf16x2(t[ct].acc[dt][0] * inv, t[ct].acc[dt][1] * inv);
-            packed.y = pack_bf16x2(t[ct].acc[dt][2] * inv, t[ct].acc[dt][3] * inv);
-            *reinterpret_cast<uint2*>(o + dt * 16 + 4 * c) = packed;
-        }
-    }
-}
-
 // -------------------------- prefill, copied straight into LDS, phases overlapped --
-// The same work once more for heads of 64 and 128, in steps of 32 keys through four LDS
-// buffers, with the phases of a wave's step overlapped: while the matrix pipeline works on the
+// The same work for heads of 64 and 128 (ND = 4, 8; NJ = ND/2), with the keys and values
+// copied from the cache into LDS by the memory pipeline itself (global_load_lds_dwordx4: lane
+// l of a wave writes the 16 bytes it asked for at LDS base + 16 l, no register holds them
+// meanwhile), 32 keys a step through four buffers.  Such a copy leaves no room for padding
+// between rows, so rows are swizzled instead: a lane chooses which 16 bytes of the cache it
+// asks for, and asks for those that belong at its place.  Keys: row = key, 16-byte chunk q of
+// the row lies at chunk q ^ f(key) with f(key) = (key & 3) | ((key >> 3) & 3) << 2 (halved for
+// rows of 8 chunks): the 16 lanes that read one chunk column for an MFMA operand (keys
+// 8 (r/4) + 4 u + r%4) then hit 16 different bank groups.  Values: four planes of 8 keys, a
+// plane [dim][8 keys]: the 16 lanes that read one plane for an MFMA operand take 256 bytes in
+// a row.
+// The phases of a wave's step are overlapped: while the matrix pipeline works on the
 // scores of step i+1 the vector units turn the exponents of step i into weights, and while it
 // adds up the values of step i they turn the scores of step i+1 into exponents.  A wave
 // issues one instruction at a time, and an MFMA that waits for the pipeline holds up what
@@ -1285,8 +1096,8 @@ __device__ __forceinline__ void prefill_pipe_block(
 
     const int wave_u = __builtin_amdgcn_readfirstlane(tid / 64);     // the wave, in a scalar register (for the copies' addresses)
     // Copy w = WAVES e + wave of a block moves 64 x 16 bytes: for keys the KPC rows from w KPC of the
-    // block (lane l: row l / CR, the chunk that belongs at chunk l % CR of that row, rows swizzled
-    // as in prefill_dma_block); for values 64 dims of the plane w / WPP (lane l: dim
+    // block (lane l: row l / CR, the chunk that belongs at chunk l % CR of that row); for values
+    // 64 dims of the plane w / WPP (lane l: dim
     // (w % WPP) 64 + l, the plane's 8 keys).  A page holds at least 8 keys, so what copy e moves of
     // the keys and of the values lies in one page.  An address is a base in scalar registers plus
     // an offset that a lane keeps for the whole kernel.
@@ -1442,8 +1253,8 @@ __device__ __forceinline__ void prefill_pipe_block(
 }
 
 // With raw.qkv the queries are taken from the raw projections (normed and rotated here, q
-// is not read); needs head_dim == 32*NJ.  DMA: blocks are copied straight into LDS
-// (prefill_dma_block; heads of 64 and 128).
+// is not read); needs head_dim == 32*NJ.  DMA: keys and values are copied straight into LDS
+// (prefill_pipe_block; heads of 64 and 128, KB = 32).
 // grid (row blocks, kv_heads * head_tiles).  Row blocks late in a sequence walk more keys
 // than early ones; `pair` says how the work is evened out: 1: (ceil(row blocks / 2), ...)
 // workgroups that each take block (last - b) and then block b; 2: long blocks placed beside
@@ -1493,23 +1304,18 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
         rb = second;
         if (second != first) rb2 = first;
     }
-    for (;;) {
-        if constexpr (DMA && KB == 32)
+    const int passes = rb2 < 0 ? 1 : 2;
+    for (int pass = 0; pass < passes; ++pass) {
+        if (pass) __syncthreads();                            // (the buffers are used again)
+        const int block = pass ? rb2 : rb;
+        if constexpr (DMA)
             prefill_pipe_block<NJ, ND, CT, WAVES>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                                   table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                                  scale_log2, window, rq, rb, hd_i, raw);
-        else if constexpr (DMA)
-            prefill_dma_block<NJ, ND, CT>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
-                                          table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                          scale_log2, window, rq, rb, hd_i, raw);
+                                                  scale_log2, window, rq, block, hd_i, raw);
         else
             prefill_lds_block<NJ, ND, CT, KB>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                               table_width, page_size, page_shift, num_pages, heads, kv_heads,
-                                              scale_log2, window, rq, rb, hd_i, raw);
-        if (rb2 < 0) break;
-        rb = rb2;
-        rb2 = -1;
-        __syncthreads();                                      // (the buffers are used again)
+                                              scale_log2, window, rq, block, hd_i, raw);
     }
 }
 
@@ -1661,7 +1467,7 @@ static int launch_prefill(
         if (direct == 2) two = false;
         if (direct == 3 || (direct >= 4 && direct <= 7)) two = head_dim <= 128;
         if (direct == 8) two = false;
-        const bool pipe = direct != 9;                            // (9: the kernel that does not overlap the phases of a step)
+        if (head_dim == 112) two = false;                         // (two tiles of that size do not fit a wave's registers)
         const int rows_per_block = 4 * rq * (two ? 2 : 1);
         const long blocks = (rows + rows_per_block - 1) / rows_per_block + num_seqs;   // upper bound
         if (blocks > 2147483647L) return tli_fail("attention_prefill: too many rows");
@@ -1670,9 +1476,9 @@ static int launch_prefill(
         if (direct == 8) pair = 3;                                // one tile, long blocks first
         dim3 grid((unsigned)(pair == 1 ? (blocks + 1) / 2 : blocks), kv_heads * head_tiles);
         const int kb = head_dim <= 128 ? 64 : 32;
-        // heads of 64 and 128: blocks copied straight into two LDS buffers
+        // heads of 64 and 128: 32 keys a step copied straight into four LDS buffers
         const bool dma = head_dim == 64 || head_dim == 128;
-        const size_t lds = dma ? (size_t)2 * 2 * 64 * head_dim * sizeof(bf16_t)
+        const size_t lds = dma ? (size_t)4 * 2 * 32 * head_dim * sizeof(bf16_t)
                                : ((size_t)kb * (head_dim + 8) + (size_t)head_dim * (kb + 8)) * sizeof(bf16_t);
 #define ARGS (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, row_start, \
              seq_start, num_seqs, tables, table_width, page_size, shift, num_pages, heads, kv_heads
@@ -1680,11 +1486,9 @@ static int launch_prefill(
 #define TAIL_LDS scale * LOG2E, window, rq, pair, raw
 #define LDS_CALL(NJ, ND, CT, KB, DMA) attention_prefill_lds_kernel<NJ, ND, CT, KB, DMA><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS)
 #define CALL(NJ, ND)                                                                                    \
-    if ((ND == 4 || ND == 8) && two && pipe) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 2, 32, true); \
-    else if ((ND == 4 || ND == 8) && pipe) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 1, 32, true); \
-    else if ((ND == 4 || ND == 8) && two) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 2, 64, true); \
-    else if (ND == 4 || ND == 8) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 1, 64, true); \
-    else if (ND <= 8 && two) LDS_CALL(NJ, ((ND <= 8 && ND != 4 && ND != 8) ? ND : 1), 2, 64, false);    \
+    if ((ND == 4 || ND == 8) && two) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 2, 32, true); \
+    else if (ND == 4 || ND == 8) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 1, 32, true); \
+    else if (ND <= 8 && ND != 7 && two) LDS_CALL(NJ, ((ND <= 8 && ND != 4 && ND != 8 && ND != 7) ? ND : 1), 2, 64, false); \
     else if (ND <= 8) LDS_CALL(NJ, ((ND <= 8 && ND != 4 && ND != 8) ? ND : 1), 1, 64, false);           \
     else LDS_CALL(NJ, ND, 1, 32, false)
         DISPATCH_HEAD_DIM(CALL)

@@ -240,15 +240,16 @@ class ModelRunner:
         buf[lay["slots"]] = slots
         if wanted + pads:
             buf[lay["sample_rows"]] = sample
-        pad_row = [self.pad_page] + [-1] * (width - 1)
         for g in range(len(self.cache.groups)):
-            flat = []
-            for rc in rcs:
+            # (a request's table is one piece of memory: a copy each, whatever their length)
+            rows_of = buf[lay[f"tables{g}"]].reshape(seqs + pads, width)
+            rows_of.fill(-1)
+            for i, rc in enumerate(rcs):
                 tab = rc.tables[g]
-                flat.extend(tab)
-                flat.extend([-1] * (width - len(tab)))
-            flat.extend(pad_row * pads)
-            buf[lay[f"tables{g}"]] = flat
+                if len(tab):
+                    rows_of[i, :len(tab)] = np.frombuffer(tab, dtype=np.int32)
+            if pads:
+                rows_of[seqs:, 0] = self.pad_page
         self.inputs.upload(lay["_end"].stop)
         dev = self.inputs.dev
         rows, seqs = rows + pads, seqs + pads
