@@ -332,3 +332,22 @@ def test_prefix_pages_are_shared_revived_and_forgotten():
     m.check()
     with pytest.raises(ValueError):
         CacheManager([FULL, WIN], page_size=4, num_pages=8, max_requests=1, prefix_caching=True)
+
+
+def test_a_block_table_reads_like_a_list_and_is_one_piece_of_memory():
+    """What the step function relies on when it packs the tables of a step: the table can be
+    viewed as int32 memory without a conversion, and goes on growing afterwards."""
+    import numpy as np
+    from tiny_llm_infer_amd.cache.manager import PageTable
+    t = PageTable()
+    assert len(t) == 0 and not t and t == []
+    for page in (7, 3, 9):
+        t.append(page)
+    assert t == [7, 3, 9] and t != [7, 3] and t[:2] == [7, 3] and t[1] == 3
+    assert list(reversed(t)) == [9, 3, 7]
+    row = np.full(8, -1, dtype=np.int32)
+    row[:len(t)] = np.frombuffer(t, dtype=np.int32)
+    assert row.tolist() == [7, 3, 9, -1, -1, -1, -1, -1]
+    t[0] = -1                      # a window has passed the page
+    t.append(11)                   # no view is held any more: the table grows
+    assert t == [-1, 3, 9, 11]
