@@ -85,8 +85,8 @@ def test_window_pages_are_given_back_when_passed():
     m.reserve("a", 50)
     m.advance("a", 50)
     # the next query is at 50 and reads 31..50: blocks 0..2 (slots 0..23) are passed
-    assert m.get("a").tables[1][:4] == [-1, -1, -1, 3]
-    assert m.get("a").tables[0][:4] == [0, 1, 2, 3]
+    assert list(m.get("a").tables[1][:4]) == [-1, -1, -1, 3]
+    assert list(m.get("a").tables[0][:4]) == [0, 1, 2, 3]
     held = 64 - m.free_pages()[1]
     assert held == 4
     for n in range(51, 200):
@@ -305,7 +305,7 @@ def test_prefix_pages_are_shared_revived_and_forgotten():
     b = a[:8] + [1, 2, 3]
     m.admit("b")
     assert m.adopt_prefix("b", b) == 8
-    assert m.get("b").tables[0] == m.get("a").tables[0][:2]
+    assert m.get("b").tables[0] == list(m.get("a").tables[0][:2])
     assert m.groups[0].pool.ref_count(m.get("a").tables[0][0]) == 2
     m.reserve("b", 11)
     assert m.get("b").tables[0][2] != m.get("a").tables[0][2]
@@ -343,7 +343,7 @@ def test_a_block_table_reads_like_a_list_and_is_one_piece_of_memory():
     assert len(t) == 0 and not t and t == []
     for page in (7, 3, 9):
         t.append(page)
-    assert t == [7, 3, 9] and t != [7, 3] and t[:2] == [7, 3] and t[1] == 3
+    assert t == [7, 3, 9] and t != [7, 3] and list(t[:2]) == [7, 3] and t[1] == 3
     assert list(reversed(t)) == [9, 3, 7]
     row = np.full(8, -1, dtype=np.int32)
     row[:len(t)] = np.frombuffer(t, dtype=np.int32)

@@ -114,8 +114,8 @@ class GroupLayout:
 class PageTable(array):
     """The block table of a request in one group: block -> page id or -1, 32-bit integers in
     one piece of memory, so that a step packs it into its inputs with one copy
-    (``numpy.frombuffer``) however long it has grown.  Reads like a list: equal to any sequence of
-    the same numbers, and a slice of it is a list."""
+    (``numpy.frombuffer``) however long it has grown.  Reads like a list, and is equal to any
+    sequence of the same numbers."""
 
     def __new__(cls, pages=()):
         return super().__new__(cls, "i", pages)
@@ -127,10 +127,6 @@ class PageTable(array):
         return not self.__eq__(other)
 
     __hash__ = None
-
-    def __getitem__(self, index):
-        item = super().__getitem__(index)
-        return item.tolist() if isinstance(index, slice) else item
 
 
 @dataclass
@@ -320,14 +316,13 @@ class CacheManager:
         tokens at positions [num_tokens, new_total)."""
         rc = self._live[key]
         out = []
+        nb = _blocks(new_total, self.page_size)
         for gi, g in enumerate(self.groups):
-            table = rc.tables[gi]
+            # every block from the first one a query at num_tokens reads up to the table's end is
+            # held (``reserve`` filled them, ``advance`` gives back only what lies before): what is
+            # missing are the blocks past the table's end
             first = self._first_needed_block(g, rc.num_tokens)
-            need = 0
-            for b in range(first, _blocks(new_total, self.page_size)):
-                if b >= len(table) or table[b] < 0:
-                    need += 1
-            out.append(need)
+            out.append(max(0, nb - max(first, len(rc.tables[gi]))))
         return out
 
     def can_reserve(self, key: Hashable, new_total: int) -> bool:
@@ -343,15 +338,15 @@ class CacheManager:
             raise ValueError("a request cannot shrink")
         if not self.can_reserve(key, new_total):
             raise CacheFull(f"not enough free pages to hold {new_total} tokens of {key!r}")
+        nb = _blocks(new_total, self.page_size)
         for gi, g in enumerate(self.groups):
             table = rc.tables[gi]
-            nb = _blocks(new_total, self.page_size)
-            while len(table) < nb:
-                table.append(-1)
+            held = len(table)
             first = self._first_needed_block(g, rc.num_tokens)
-            for b in range(first, nb):
-                if table[b] < 0:
-                    table[b] = self._take(gi)
+            while len(table) < min(first, nb):
+                table.append(-1)                  # (a window has jumped past these blocks)
+            for b in range(max(first, held), nb):
+                table.append(self._take(gi))
         rc.reserved_tokens = max(rc.reserved_tokens, new_total)
 
     def advance(self, key: Hashable, new_total: int) -> None:
@@ -400,6 +395,10 @@ class CacheManager:
                 for page in rc.tables[gi]:
                     if page >= 0:
                         held[page] = held.get(page, 0) + 1
+                # what ``pages_needed`` counts on: no hole from the first block that is read to the end
+                first = self._first_needed_block(g, rc.num_tokens)
+                if any(page < 0 for page in rc.tables[gi][first:]):
+                    raise PageError(f"group {gi}: the table of {rc.key!r} has a hole at or after block {first}")
             for page in range(g.pool.num_pages):
                 if g.pool.ref_count(page) != held.get(page, 0):
                     raise PageError(f"group {gi} page {page}: pool counts "

@@ -136,6 +136,10 @@ class HipOps:
     DECODE_WORKGROUPS = 256      # aim of the decode attention's key splitting: one workgroup a compute unit (measured
                                  # against 128, 192 and 512 at batch 1 to 64 and 128 to 30,000 keys: up to 10% over 512)
     DECODE_SPLIT_KEYS = 512      # a split walks at least this many keys (128, 256 and 1024 measured: no better)
+    # a step of prompt portions whose first sequences decode hands those to the decode kernel when
+    # they are this many, or when one of them has this many keys
+    DECODE_BESIDE_PROMPTS = 8
+    DECODE_BESIDE_PROMPTS_KEYS = 1024
 
     def __init__(self, device):
         self.device = torch.device(device)
@@ -624,7 +628,7 @@ class HipOps:
             if step.max_seq_len > npos:
                 raise KernelError(f"a position reaches {step.max_seq_len}, the rotation table has {npos}")
         out = torch.empty((T, heads * head_dim), dtype=qkv.dtype, device=self.device)
-        splits, per_split, partial = self._decode_splits(step, g, heads, kv_heads, head_dim, window)
+        splits, per_split, partial = self._decode_splits(step.num_rows, step.reach, g, heads, kv_heads, head_dim, window)
         self._call(self.lib.tli_qkv_attention_decode_bf16, None if sums is not None else qkv.data_ptr(),
                    out.data_ptr(), _ptr(partial),
                    kc.data_ptr(), vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
@@ -647,18 +651,41 @@ class HipOps:
         qw, qe = q_norm if q_norm is not None else (None, 0.0)
         cos, sin = (rotary[0], rotary[1]) if rotary is not None else (None, None)
         out = torch.empty((T, heads * head_dim), dtype=qkv.dtype, device=self.device)
+        # The sequences that decode (one row each) stand first in a step that the scheduler
+        # made.  The prefill kernel would give each of them workgroups that walk all their keys
+        # with one row; where that is much work they go to the decode kernel instead, which
+        # splits a row's keys over workgroups (their keys and values are in the cache by now).
+        first = 0
+        starts = step.h_row_start
+        while first < step.num_seqs and starts[first + 1] - starts[first] == 1:
+            first += 1
+        if first == step.num_seqs or heads // kv_heads > 16 or self.prefill_direct:
+            first = 0
+        if first and (first >= self.DECODE_BESIDE_PROMPTS or max(step.h_seq_len[:first]) >= self.DECODE_BESIDE_PROMPTS_KEYS):
+            kw, ke = k_norm if k_norm is not None else (None, 0.0)
+            longest = max(step.h_seq_len[:first])
+            splits, per_split, partial = self._decode_splits(first, max(128, 1 << (longest - 1).bit_length()), g, heads,
+                                                             kv_heads, head_dim, window)
+            self._call(self.lib.tli_qkv_attention_decode_bf16, qkv.data_ptr(), out.data_ptr(), _ptr(partial),
+                       kc.data_ptr(), vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
+                       g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], first, heads, kv_heads,
+                       head_dim, _ptr(qw), float(qe), _ptr(kw), float(ke), _ptr(cos), _ptr(sin),
+                       0, float(scale), int(window or 0), splits, per_split, None, 0, self._stream())
+        else:
+            first = 0
         self._call(self.lib.tli_qkv_attention_prefill_bf16, qkv.data_ptr(), out.data_ptr(), kc.data_ptr(),
-                   vc.data_ptr(), step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs,
-                   T, g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], heads, kv_heads,
+                   vc.data_ptr(), step.row_start.data_ptr() + 4 * first, step.seq_start.data_ptr() + 4 * first,
+                   step.num_seqs - first, T - first, g.tables.data_ptr() + 4 * first * g.table_width, g.table_width,
+                   g.page_size, kc.shape[0], heads, kv_heads,
                    head_dim, _ptr(qw), float(qe), _ptr(cos), _ptr(sin), float(scale), int(window or 0),
                    int(self.prefill_direct), self._stream())
         return out
 
-    def _decode_splits(self, step, g, heads, kv_heads, head_dim, window):
-        """How the keys of a decode step are split over workgroups: they are when the
-        batch alone would leave most of the 256 compute units idle."""
-        T = step.num_rows
-        reach = step.reach if not window else min(step.reach, (window + 31) // 32 * 32 + 32)
+    def _decode_splits(self, T, reach, g, heads, kv_heads, head_dim, window):
+        """How the keys of ``T`` rows that decode (``reach``: a power of two that the longest
+        of their sequences fits) are split over workgroups: they are when the batch alone
+        would leave most of the 256 compute units idle."""
+        reach = reach if not window else min(reach, (window + 31) // 32 * 32 + 32)
         groups = T * kv_heads * ((heads // kv_heads + 15) // 16)
         # a split costs a merge pass: only worth it when a workgroup would walk many keys
         splits = max(1, min((self.DECODE_WORKGROUPS + groups - 1) // groups, reach // self.DECODE_SPLIT_KEYS, 64))
@@ -675,7 +702,7 @@ class HipOps:
     def _attention_decode(self, q, out, step, kc, vc, g, heads, kv_heads, head_dim, scale, window):
         """One row per sequence."""
         T = step.num_rows
-        splits, per_split, partial = self._decode_splits(step, g, heads, kv_heads, head_dim, window)
+        splits, per_split, partial = self._decode_splits(step.num_rows, step.reach, g, heads, kv_heads, head_dim, window)
         self._call(self.lib.tli_attention_decode_bf16, q.data_ptr(), out.data_ptr(), _ptr(partial),
                    kc.data_ptr(), vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
                    g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], T, heads, kv_heads,
