@@ -296,13 +296,34 @@ static int launch_mid(const bf16_t* x, const bf16_t* w, void* y, float* part, in
 // at no more than one a compute unit where it can).
 static int mid_tiles_per_wave(int N, int gated) { return gated || (N + 15) / 16 >= 8 * 192 ? 2 : 1; }
 
+// How a product of this shape is dealt out: column tiles a wave and ranges of k.  As many
+// workgroups as fit the 256 compute units once (more cost more than they bring, measured at
+// the layer sizes of Qwen3-8B to 32B): with one tile a wave (four waves: 64 columns a workgroup)
+// as many ranges as that allows, 5,120 columns in 3 ranges (240 workgroups; 4 ranges of 128
+// columns, 160 workgroups, were 9% slower); where the columns alone are more than 128 groups
+// but fewer than 192, two tiles a wave and the ranges that go with them (10,240 columns: 80
+// groups in 3 ranges).  A range keeps at least two slices of 128.
+static void mid_plan(int N, int K, int gated, int* tiles_a_wave, int* ranges) {
+    const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
+    auto ranges_for = [&](int groups) { return max(1, min(min(256 / max(groups, 1), k_steps / 2), 16)); };
+    int rt = mid_tiles_per_wave(N, gated);
+    int groups = (n_tiles + 4 * rt - 1) / (4 * rt);
+    int splits = groups >= 192 ? 1 : ranges_for(groups);
+    if (!gated && rt == 1 && groups * splits < 192) {
+        const int groups2 = (n_tiles + 7) / 8, splits2 = ranges_for(groups2);
+        if (groups2 * splits2 > groups * splits) {
+            rt = 2;
+            splits = splits2;
+        }
+    }
+    *tiles_a_wave = rt;
+    *ranges = splits;
+}
+
 // How many ranges of k a product of this shape is cut into (the caller sizes `part` by it).
 extern "C" int tli_gemm_mid_splits(int N, int K, int gated) {
-    const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
-    const int per_group = 4 * mid_tiles_per_wave(N, gated);
-    const int groups = (n_tiles + per_group - 1) / per_group;
-    int splits = 1;
-    while (groups * splits < 192 && splits * 2 <= k_steps && splits < 16) splits *= 2;
+    int rt, splits;
+    mid_plan(N, K, gated, &rt, &splits);
     return splits;
 }
 
@@ -331,7 +352,9 @@ extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* p
         // more workgroups than compute units cost more than they bring (measured at the layer
         // sizes of Qwen3-14B and 32B): a gated product then takes eight waves a workgroup, a
         // plain one whose k ranges push it over takes two column tiles a wave
-        int rt = mid_tiles_per_wave(N, gated), waves = 4;
+        int rt, planned, waves = 4;
+        mid_plan(N, K, gated, &rt, &planned);
+        if (splits != planned) rt = mid_tiles_per_wave(N, gated);     // (ranges forced by the caller)
         const int groups = ((N + 15) / 16 + 4 * rt - 1) / (4 * rt);
         if (gated && groups > 256) waves = 8;
         if (!gated && rt == 1 && (long)groups * splits > 256) rt = 2;
