@@ -570,11 +570,13 @@ RAW_CASES = [
     (6, 3, 256, True, True, 16, [90, 17], [7, 17], 64, True),
     (4, 2, 128, False, False, 32, [45], [45], None, True),
     (16, 1, 64, True, True, 16, [48, 9], [5, 9], None, False),
-    # sequences that decode in front of portions of prompts, as the scheduler puts them: one with
-    # many keys, or many of them, go to the decode kernel and the rest of the step to the prefill kernel
+    # sequences that decode in front of portions of prompts, as the scheduler puts them: where one of
+    # them has many more keys than the portions, or they are many, they go to the decode kernel and the
+    # rest of the step to the prefill kernel
     (32, 8, 128, True, True, 16, [1500, 40, 300, 64], [1, 1, 130, 64], None, True),
-    (8, 8, 64, True, True, 8, [130, 257, 16, 17, 9, 700, 33, 64, 65, 200, 31], [1] * 9 + [150, 31], 19, True),
+    (8, 8, 64, True, True, 8, [130, 257, 16, 17, 9, 700] * 6 + [200, 31], [1] * 36 + [150, 31], 19, True),
     (8, 2, 128, True, True, 16, [90, 1900, 513], [1, 1, 257], 300, True),
+    (8, 2, 128, True, True, 16, [90, 300, 513], [1, 1, 257], None, True),          # (these stay in the one kernel)
 ]
 
 

@@ -136,10 +136,12 @@ class HipOps:
     DECODE_WORKGROUPS = 256      # aim of the decode attention's key splitting: one workgroup a compute unit (measured
                                  # against 128, 192 and 512 at batch 1 to 64 and 128 to 30,000 keys: up to 10% over 512)
     DECODE_SPLIT_KEYS = 512      # a split walks at least this many keys (128, 256 and 1024 measured: no better)
-    # a step of prompt portions whose first sequences decode hands those to the decode kernel when
-    # they are this many, or when one of them has this many keys
-    DECODE_BESIDE_PROMPTS = 8
-    DECODE_BESIDE_PROMPTS_KEYS = 1024
+    # A step of prompt portions whose first sequences decode: those go to the decode kernel when the
+    # longest of them has this many times the keys of the longest portion, or as many keys when they
+    # are this many rows (measured at 2 to 63 rows of 200 to 6,000 keys beside portions of 300 to
+    # 2,048 tokens: a second kernel costs 15 to 30 us, which a few short rows do not bring back)
+    DECODE_BESIDE_PROMPTS_KEYS = 2.0
+    DECODE_BESIDE_PROMPTS = 32
 
     def __init__(self, device):
         self.device = torch.device(device)
@@ -653,17 +655,19 @@ class HipOps:
         out = torch.empty((T, heads * head_dim), dtype=qkv.dtype, device=self.device)
         # The sequences that decode (one row each) stand first in a step that the scheduler
         # made.  The prefill kernel would give each of them workgroups that walk all their keys
-        # with one row; where that is much work they go to the decode kernel instead, which
-        # splits a row's keys over workgroups (their keys and values are in the cache by now).
+        # with one row; where those would be the last to finish they go to the decode kernel instead,
+        # which splits a row's keys over workgroups (their keys and values are in the cache by now).
         first = 0
         starts = step.h_row_start
         while first < step.num_seqs and starts[first + 1] - starts[first] == 1:
             first += 1
         if first == step.num_seqs or heads // kv_heads > 16 or self.prefill_direct:
             first = 0
-        if first and (first >= self.DECODE_BESIDE_PROMPTS or max(step.h_seq_len[:first]) >= self.DECODE_BESIDE_PROMPTS_KEYS):
+        longest = max(step.h_seq_len[:first]) if first else 0
+        beside = max(step.h_seq_len[first:step.num_seqs]) if first else 0
+        if first and (longest >= self.DECODE_BESIDE_PROMPTS_KEYS * beside
+                      or (first >= self.DECODE_BESIDE_PROMPTS and longest >= beside)):
             kw, ke = k_norm if k_norm is not None else (None, 0.0)
-            longest = max(step.h_seq_len[:first])
             splits, per_split, partial = self._decode_splits(first, max(128, 1 << (longest - 1).bit_length()), g, heads,
                                                              kv_heads, head_dim, window)
             self._call(self.lib.tli_qkv_attention_decode_bf16, qkv.data_ptr(), out.data_ptr(), _ptr(partial),
