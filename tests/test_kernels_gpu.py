@@ -135,7 +135,10 @@ def test_skinny_linear_against_plain_kernel_and_reference(ops, mnk, out):
         assert torch.equal(streamed, got)      # same additions in the same order, other addresses
     else:                                      # 17..128 rows: the kernel that shares x through LDS
         assert float((streamed.double().cpu() - want).abs().max()) <= bound
-        shapes = ((1, 224), (2, 228), (4, 314), (3, 418), (5, 424), (7, 218)) if M <= 64 else ((1, 224), (3, 214), (5, 0))
+        # (ranges of k, launch shape: depth of the rings, column tiles a wave, waves; also numbers of
+        # waves that do not divide the copies of a slice of x)
+        shapes = (((1, 224), (2, 228), (4, 314), (3, 418), (5, 424), (7, 218), (2, 223), (1, 225), (3, 226), (1, 227))
+                  if M <= 64 else ((1, 224), (3, 214), (5, 0), (1, 223), (2, 225), (1, 227)))
         for splits, cfg in shapes:
             ops.mid_splits, ops.mid_cfg = splits, cfg
             try:

@@ -51,8 +51,10 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
     constexpr int STAGES = DEPTH + 1;                        // W: DEPTH slices on their way, one in use
     constexpr int XSLOTS = DEPTH + 2;                        // x: one slice further ahead
     constexpr int SLICE = ROWS * 128;                        // elements of a slice of x
-    constexpr int XI = ROWS / (4 * WAVES);                   // copies a wave issues for a slice (64 x 16 bytes each)
-    static_assert(ROWS % (4 * WAVES) == 0, "a slice is a whole number of copies for every wave");
+    constexpr int COPIES = ROWS / 4;                         // copies of 64 x 16 bytes that make up a slice
+    // copies a wave issues for a slice: the same number for every wave (where the waves do not divide
+    // the copies, the last one is made again by the waves that would have none)
+    constexpr int XI = (COPIES + WAVES - 1) / WAVES;
     extern __shared__ uint4 xs_raw[];
     bf16_t* xs = reinterpret_cast<bf16_t*>(xs_raw);          // [XSLOTS][ROWS][128], rows swizzled
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
@@ -99,17 +101,20 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
     // instead (they meet the zeros that pad W).
     const bf16_t* x_row[XI];
     int x_col[XI];
+    uint32_t x_dst[XI];                                      // where copy e lands in a slot (bytes)
 #pragma unroll
     for (int e = 0; e < XI; ++e) {
-        const int place = (e * WAVES + wave) * 64 + lane, row = place / 16;
+        const int copy = min(e * WAVES + wave, COPIES - 1);
+        const int place = copy * 64 + lane, row = place / 16;
         x_row[e] = x + (size_t)min(row, M - 1) * K;
         x_col[e] = ((place % 16) ^ (row & 15)) * 8;
+        x_dst[e] = (uint32_t)copy * 1024u;
     }
     // (The copy is written in assembly: told of it, the compiler waits for every load in
     // flight before the next LDS read, because the copy writes LDS.  Untold, it counts
     // fewer loads in flight than there are when it waits for W fragments, and so waits for
     // somewhat more than it needs: for the copies issued before the fragments it lets fly.)
-    const uint32_t xs_base = (uint32_t)(uintptr_t)(lds_void_m*)xs + (uint32_t)wave * 1024u;
+    const uint32_t xs_base = (uint32_t)(uintptr_t)(lds_void_m*)xs;
     auto fetch_x = [&](int logical) {
         const int step = at(logical);
         const uint32_t slot_base = xs_base + (uint32_t)((logical - step_begin) % XSLOTS) * (SLICE * 2);
@@ -117,7 +122,7 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
         for (int e = 0; e < XI; ++e) {
             const int k = step * 128 + x_col[e];
             const bf16_t* src = x_row[e] + (k < K ? k : 0);
-            const uint32_t dst = __builtin_amdgcn_readfirstlane(slot_base + (uint32_t)(e * WAVES * 1024));
+            const uint32_t dst = __builtin_amdgcn_readfirstlane(slot_base + x_dst[e]);
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                          :: "s"(dst), "v"(src) : "m0");
         }
@@ -302,12 +307,28 @@ static int mid_tiles_per_wave(int N, int gated) { return gated || (N + 15) / 16 
 // as many ranges as that allows, 5,120 columns in 3 ranges (240 workgroups; 4 ranges of 128
 // columns, 160 workgroups, were 9% slower); where the columns alone are more than 128 groups
 // but fewer than 192, two tiles a wave and the ranges that go with them (10,240 columns: 80
-// groups in 3 ranges).  A range keeps at least two slices of 128.
-static void mid_plan(int N, int K, int gated, int* tiles_a_wave, int* ranges) {
+// groups in 3 ranges).  A range keeps at least two slices of 128.  Gated products: see below.
+static void mid_plan(int N, int K, int gated, int* tiles_a_wave, int* waves_a_group, int* ranges) {
     const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
     auto ranges_for = [&](int groups) { return max(1, min(min(256 / max(groups, 1), k_steps / 2), 16)); };
-    int rt = mid_tiles_per_wave(N, gated);
-    int groups = (n_tiles + 4 * rt - 1) / (4 * rt);
+    int rt = mid_tiles_per_wave(N, gated), waves = 4;
+    if (gated) {
+        // a wave takes one pair of gate and up tiles; three to eight waves a workgroup, whichever
+        // comes closest to 256 workgroups from below (24,576 columns: 256 workgroups of 3 waves,
+        // 5% faster at 64 rows and 11% at 128 than 192 of 4; 34,816 columns: 218 of 5 waves, 12 to 17%
+        // faster than 136 of 8); eight where even those are more than 256
+        const int pairs = (n_tiles + 1) / 2;
+        int best = 0;
+        waves = 8;
+        for (int w = 3; w <= 8; ++w) {
+            const int groups = (pairs + w - 1) / w;
+            if (groups <= 256 && groups > best) {
+                best = groups;
+                waves = w;
+            }
+        }
+    }
+    int groups = (n_tiles + waves * rt - 1) / (waves * rt);
     int splits = groups >= 192 ? 1 : ranges_for(groups);
     if (!gated && rt == 1 && groups * splits < 192) {
         const int groups2 = (n_tiles + 7) / 8, splits2 = ranges_for(groups2);
@@ -317,13 +338,14 @@ static void mid_plan(int N, int K, int gated, int* tiles_a_wave, int* ranges) {
         }
     }
     *tiles_a_wave = rt;
+    *waves_a_group = waves;
     *ranges = splits;
 }
 
 // How many ranges of k a product of this shape is cut into (the caller sizes `part` by it).
 extern "C" int tli_gemm_mid_splits(int N, int K, int gated) {
-    int rt, splits;
-    mid_plan(N, K, gated, &rt, &splits);
+    int rt, waves, splits;
+    mid_plan(N, K, gated, &rt, &waves, &splits);
     return splits;
 }
 
@@ -352,12 +374,13 @@ extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* p
         // more workgroups than compute units cost more than they bring (measured at the layer
         // sizes of Qwen3-14B and 32B): a gated product then takes eight waves a workgroup, a
         // plain one whose k ranges push it over takes two column tiles a wave
-        int rt, planned, waves = 4;
-        mid_plan(N, K, gated, &rt, &planned);
-        if (splits != planned) rt = mid_tiles_per_wave(N, gated);     // (ranges forced by the caller)
-        const int groups = ((N + 15) / 16 + 4 * rt - 1) / (4 * rt);
-        if (gated && groups > 256) waves = 8;
-        if (!gated && rt == 1 && (long)groups * splits > 256) rt = 2;
+        int rt, planned, waves;
+        mid_plan(N, K, gated, &rt, &waves, &planned);
+        if (splits != planned) {                                      // (ranges forced by the caller)
+            rt = mid_tiles_per_wave(N, gated);
+            const int groups = ((N + 15) / 16 + waves * rt - 1) / (waves * rt);
+            if (!gated && rt == 1 && (long)groups * splits > 256) rt = 2;
+        }
         cfg = 200 + 10 * rt + waves;
     }
     if (gated && (cfg / 10) % 10 < 2) return tli_fail("gemm_mid: a gated product needs pairs of row tiles");
@@ -365,6 +388,7 @@ extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* p
     switch (cfg) {
         MID_CASE(2, 1, 4) MID_CASE(3, 1, 4) MID_CASE(2, 1, 8) MID_CASE(4, 1, 8)
         MID_CASE(2, 2, 4) MID_CASE(4, 2, 4) MID_CASE(2, 2, 8)
+        MID_CASE(2, 2, 3) MID_CASE(2, 2, 5) MID_CASE(2, 2, 6) MID_CASE(2, 2, 7)
         default: return tli_fail("gemm_mid: unknown configuration %d", cfg);
     }
 }
