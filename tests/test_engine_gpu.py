@@ -129,7 +129,16 @@ def test_command_line_bench(model_folders):
     assert proc.returncode == 0, proc.stderr[-2000:]
     out = proc.stdout.strip().split("\n")
     assert out[0].startswith("run=0 output_tokens=") and "output_tokens_per_second=" in out[-1]
-    assert out[-1].startswith("aggregate_runs=2")
+    fields = lambda line: dict(f.split("=") for f in line.split() if "=" in f)
+    runs = [fields(line) for line in out if line.startswith("run=")]
+    total = fields(next(line for line in out if line.startswith("aggregate_runs=")))
+    # every request ends at a length between the two bounds, the runs add up, nothing stays held
+    assert len(runs) == 2 and all(9 <= int(r["output_tokens"]) <= 15 for r in runs)
+    assert int(total["aggregate_runs"]) == 2 and int(total["output_tokens"]) == sum(int(r["output_tokens"]) for r in runs)
+    assert abs(float(total["elapsed_seconds"]) - sum(float(r["elapsed_seconds"]) for r in runs)) < 1e-3
+    stats = fields(next(line for line in proc.stderr.split("\n") if line.startswith("engine_steps=")))
+    free, pages = stats["pages_free"].split("/")
+    assert free == pages and int(stats["engine_steps"]) > 0
 
 
 def test_command_line_plain_kernels_and_prefill_only(model_folders):
