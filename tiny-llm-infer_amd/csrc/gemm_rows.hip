@@ -422,6 +422,9 @@ static int rows_pick(int M, int N, int K, int splits, int gated) {
     const long k_steps = (K + 127) / 128, per = (k_steps + splits - 1) / splits;
     const double cost2 = shared(a_die(16)) * 256.0, cost4 = shared(a_die(12)) * 192.0 * 1.06;
     const double cost3 = alone(a_die(32)) * 512.0 * 0.84, cost6 = alone(a_die(16)) * 256.0 * 0.88;
+    // (from three rounds of the 512-column shape on, it was the fastest at every layer size measured:
+    // the costs above are those of the first rounds)
+    if (alone(a_die(32)) >= 3.0) return 3;
     int best = 2;
     double cost = cost2;
     if (cost3 < cost) { best = 3; cost = cost3; }
