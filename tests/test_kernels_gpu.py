@@ -432,7 +432,9 @@ PREFILL_MODES = {"bfloat16-direct": 1, "bfloat16-lds1": 2, "bfloat16-lds2": 3,
                  # the orders in which workgroups take row blocks (none, pairs in sequence, pairs that
                  # complement each other, long blocks first), which the launcher picks by the step's size
                  "bfloat16-order0": 4, "bfloat16-order1": 5, "bfloat16-order2": 6, "bfloat16-order3": 7,
-                 "bfloat16-lds1-order3": 8}
+                 "bfloat16-lds1-order3": 8,
+                 # heads of 64 and 128: two sets of waves a workgroup that share out a block's keys; one set
+                 "bfloat16-two-sets": 10, "bfloat16-one-set": 11}
 
 
 @pytest.mark.parametrize("dtype", DTYPES + ["bfloat16-plain"] + list(PREFILL_MODES))

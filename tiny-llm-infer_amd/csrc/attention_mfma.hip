@@ -1013,9 +1013,15 @@ typedef __attribute__((address_space(3))) void lds_void_t;
 //                        step i+1 (its bases may move: the sums are rescaled after the output)
 // A wave sees the steps a..b of the workgroup's 0..n-1 (late rows see more keys than early
 // ones); before and after them it only takes part in the barriers and the copies.
-// (WAVES = 8, one workgroup a compute unit that asks the L2 caches for every key half as
-// often, was measured 3 to 6% slower than two workgroups of four.)
-template <int NJ, int ND, int CT, int WAVES>
+// KG = 2: the workgroup has two sets of four waves with the same rows; a block brings 64 keys,
+// of which the first set takes the first 32 and the second set the rest, and the second set's
+// sums are added to the first's through LDS at the end.  A workgroup then walks its keys in
+// half as many rounds, which is what counts where the longest workgroups decide the time (a
+// prompt of 2,048 tokens: the last rows walk 64 steps of 32 keys while the chip has room for
+// every workgroup at once).
+// (Workgroups of eight waves with twice the rows, which ask the L2 caches for every key half as
+// often, were measured 3 to 6% slower than two workgroups of four.)
+template <int NJ, int ND, int CT, int KG>
 __device__ __forceinline__ void prefill_pipe_block(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ row_start,
@@ -1023,21 +1029,23 @@ __device__ __forceinline__ void prefill_pipe_block(
     int page_size, int page_shift, int num_pages, int heads, int kv_heads, float scale_log2, int window,
     int rq, int block, int head_index, const RawQkv& raw) {
     static_assert(ND == 2 * NJ && (ND == 4 || ND == 8), "heads of 64 or 128");
-    constexpr int KB = 32;
+    constexpr int KB = 32;                            // keys of a step
+    constexpr int BK = KB * KG;                       // keys of a block: a step for each set of waves
+    constexpr int WAVES = 4 * KG;
     constexpr int HD = ND * 16;
     constexpr int CR = HD / 8;                        // 16-byte chunks of a key row
-    constexpr int KI = KB * CR / (64 * WAVES), VI = HD * 4 / (64 * WAVES);     // copies a wave issues for a block: keys, values
+    constexpr int KI = BK * CR / (64 * WAVES), VI = HD * (BK / 8) / (64 * WAVES);     // copies a wave issues for a block: keys, values
     static_assert(KI >= 1 && VI >= 1, "every wave takes part in the copies");
     constexpr int PER = KI + VI;
-    constexpr int TILE = KB * HD;                     // elements of a block's keys (and of its values)
+    constexpr int TILE = BK * HD;                     // elements of a block's keys (and of its values)
     extern __shared__ uint4 lds_raw[];
     bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw); // buffer b: keys at b * 2 TILE, values TILE further
-    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
+    const int tid = threadIdx.x, lane = tid % 64, wave = (tid / 64) % 4, r = lane % 16, c = lane / 16;
     const int group = heads / kv_heads;
     const int head_tiles = (group + 15) / 16;
     const int kv_head = head_index / head_tiles, head_tile = head_index % head_tiles;
     const int heads_here = min(16, group - head_tile * 16);
-    const int rows_per_wave = CT * rq, rows_per_block = WAVES * rows_per_wave;
+    const int rows_per_wave = CT * rq, rows_per_block = 4 * rows_per_wave;
     int seq = 0, first_row = 0, n_rows = 0;
     for (; seq < num_seqs; ++seq) {
         first_row = row_start[seq];
@@ -1082,19 +1090,24 @@ __device__ __forceinline__ void prefill_pipe_block(
     const int wg_lo = window > 0 ? max(0, wg_first - window + 1) : 0;
     const int wave_first = start + local0, wave_last = wave_first + wave_rows - 1;
     const int wave_lo = window > 0 ? max(0, wave_first - window + 1) : 0;
-    // the steps: the workgroup's 0..n-1 from key T0, this wave's a..b, of which f0..f1-1 are seen
-    // whole by every row of the wave (the others need the comparison of every key with the row's range)
-    const int T0 = (wg_lo / KB) * KB;
-    const int n = (wg_last - T0) / KB + 1;
+    // The blocks: the workgroup's 0..n-1 from key T0.  Block i holds step KG i + set for each set of
+    // waves; this wave's steps are those of its blocks a..b, of which the steps f0..f1-1 are seen
+    // whole by every row of the wave (the others need the comparison of every key with the row's range).
+    const int wave_u = __builtin_amdgcn_readfirstlane(tid / 64);     // the wave, in a scalar register (for the copies' addresses)
+    const int set = wave_u / 4;                       // which of the KG sets of four waves
+    const int T0 = (wg_lo / BK) * BK;
+    const int n = (wg_last - T0) / BK + 1;
     const int full_lo = window > 0 ? max(0, wave_last - window + 1) : 0, full_hi = wave_first;
+    const int step_lo = (wave_lo - T0) / KB, step_hi = (wave_last - T0) / KB;      // the wave's steps of 32 keys
+    const bool any = wave_rows > 0 && step_hi >= set && (step_lo - set + KG - 1) / KG <= (step_hi - set) / KG;
     // (the same for a whole wave, and said so: the loops below then run on scalar registers)
-    const int a = __builtin_amdgcn_readfirstlane(wave_rows > 0 ? (wave_lo - T0) / KB : n + 1);
-    const int b = __builtin_amdgcn_readfirstlane(wave_rows > 0 ? (wave_last - T0) / KB : n);
+    const int a = __builtin_amdgcn_readfirstlane(any ? max(0, step_lo - set + KG - 1) / KG : n + 1);
+    const int b = __builtin_amdgcn_readfirstlane(any ? (step_hi - set) / KG : n);
     const int f0 = __builtin_amdgcn_readfirstlane(full_lo <= T0 ? 0 : (full_lo - T0 + KB - 1) / KB);
     const int f1 = __builtin_amdgcn_readfirstlane((full_hi - T0 + 1) / KB);
-    auto whole = [&](int step) { return step >= f0 && step < f1; };
+    auto whole = [&](int block) { return KG * block + set >= f0 && KG * block + set < f1; };
+    auto first_key = [&](int block) { return T0 + (KG * block + set) * KB; };      // of this wave's step in a block
 
-    const int wave_u = __builtin_amdgcn_readfirstlane(tid / 64);     // the wave, in a scalar register (for the copies' addresses)
     // Copy w = WAVES e + wave of a block moves 64 x 16 bytes: for keys the KPC rows from w KPC of the
     // block (lane l: row l / CR, the chunk that belongs at chunk l % CR of that row); for values
     // 64 dims of the plane w / WPP (lane l: dim
@@ -1122,7 +1135,7 @@ __device__ __forceinline__ void prefill_pipe_block(
     const uint64_t head_bytes = (uint64_t)kv_head * page_size * HD * sizeof(bf16_t);
     // 64 entries of the block table at a time live in the lanes of one register (entry
     // tab_first + l in lane l, those that name no page made 0: such keys are masked); a copy takes
-    // its page from there with v_readlane.  The register is filled again every 16 blocks, which
+    // its page from there with v_readlane.  The register is filled again every 512 keys, which
     // walk at most 64 entries (pages of 8 keys).
     int tab_first = 0, tab_pages = 0;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t*)lds;
@@ -1135,8 +1148,8 @@ __device__ __forceinline__ void prefill_pipe_block(
     // start the copies of block `step` into its buffer (called for every step in turn; past the
     // last block the last one is copied again, rather than a branch that would change what is in flight)
     auto copy = [&](int step) {
-        const int t0 = T0 + min(step, n - 1) * KB;
-        if ((step & 15) == 0) {
+        const int t0 = T0 + min(step, n - 1) * BK;
+        if ((step & (16 / KG - 1)) == 0) {
             tab_first = t0 >> page_shift;
             // (loaded and waited for in assembly, like the copies: the compiler then knows of no load
             // in the loop and leaves the counting of those in flight to the waits written here)
@@ -1148,7 +1161,7 @@ __device__ __forceinline__ void prefill_pipe_block(
             tab_pages = (unsigned)page < (unsigned)num_pages ? page : 0;
         }
         const uint32_t kb = (uint32_t)(step & 3) * (uint32_t)(2 * TILE * sizeof(bf16_t));
-        const uint64_t in_page = (uint64_t)(t0 & (page_size - 1) & ~(KB - 1));     // pages of more than 32 keys
+        const uint64_t in_page = (uint64_t)(t0 & (page_size - 1) & ~(BK - 1));     // pages of more keys than a block
         const uint64_t k_base = (uint64_t)(uintptr_t)k_cache + head_bytes + in_page * (HD * sizeof(bf16_t));
         const uint64_t v_base = (uint64_t)(uintptr_t)v_cache + head_bytes + in_page * sizeof(bf16_t);
 #pragma unroll
@@ -1166,13 +1179,14 @@ __device__ __forceinline__ void prefill_pipe_block(
         copy(i + 3);
     };
 
-    // LDS offsets (elements) of this lane's fragments in a buffer (values: plane c, dim 16 dt + r)
+    // LDS offsets (elements) of this lane's fragments in a buffer: the keys from row 32 set of the
+    // block (values: plane 4 set + c, dim 16 dt + r)
     int ka_row[2], ka_col[NJ];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) ka_row[u] = (8 * (r / 4) + 4 * u + (r % 4)) * HD;
+    for (int u = 0; u < 2; ++u) ka_row[u] = (KB * set + 8 * (r / 4) + 4 * u + (r % 4)) * HD;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) ka_col[j] = ((c * NJ + j) ^ (CR == 16 ? r : r >> 1)) * 8;
-    const int vt_at = TILE + (c * HD + r) * 8;
+    const int vt_at = TILE + ((4 * set + c) * HD + r) * 8;
     auto keys_of = [&](int step, Frag (&ka)[2][NJ]) {
         const bf16_t* ks = lds + (size_t)(step & 3) * 2 * TILE;
 #pragma unroll
@@ -1198,9 +1212,9 @@ __device__ __forceinline__ void prefill_pipe_block(
             keys_of(a, ka);
             tiles_scores<NJ, ND, CT>(t, ka, ex);
             if (whole(a))
-                tiles_exponents<NJ, ND, CT, false>(t, ex, T0 + a * KB + 8 * c, 4, scale_log2);
+                tiles_exponents<NJ, ND, CT, false>(t, ex, first_key(a) + 8 * c, 4, scale_log2);
             else
-                tiles_exponents<NJ, ND, CT, true>(t, ex, T0 + a * KB + 8 * c, 4, scale_log2);
+                tiles_exponents<NJ, ND, CT, true>(t, ex, first_key(a) + 8 * c, 4, scale_log2);
             ++i;
         }
         auto round = [&](auto MASK_T) {
@@ -1213,7 +1227,7 @@ __device__ __forceinline__ void prefill_pipe_block(
             tiles_pack<CT>(ex, pb);
             tiles_scores<NJ, ND, CT>(t, ka, sc);
             tiles_output<NJ, ND, CT>(t, vt, pb);
-            tiles_exponents<NJ, ND, CT, MASK>(t, sc, T0 + (i + 1) * KB + 8 * c, 4, scale_log2);
+            tiles_exponents<NJ, ND, CT, MASK>(t, sc, first_key(i + 1) + 8 * c, 4, scale_log2);
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
@@ -1235,6 +1249,54 @@ __device__ __forceinline__ void prefill_pipe_block(
     for (; i < n; ++i) top(i);                        // blocks after this wave's keys
     // the copies that the last rounds started land before anything else uses the buffers
     __builtin_amdgcn_s_waitcnt(0x0F70);
+
+    if constexpr (KG > 1) {
+        // the other sets hand their sums over through LDS ([set - 1][wave][tile][lane]: base, sum of
+        // the weights, sums of the values), the first set adds them up in set order
+        constexpr int STRIDE = ND * 4 + 2;
+        static_assert((size_t)(KG - 1) * 4 * CT * 64 * STRIDE * sizeof(float) <= (size_t)4 * 2 * TILE * sizeof(bf16_t),
+                      "the sums fit the buffers");
+        float* sums = reinterpret_cast<float*>(lds_raw);
+        __syncthreads();                                  // nobody reads keys or values any more
+        if (set > 0) {
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                float* dst = sums + ((((size_t)(set - 1) * 4 + wave) * CT + ct) * 64 + lane) * STRIDE;
+                dst[0] = t[ct].m;
+                dst[1] = tile_sum(t[ct]);
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) dst[2 + dt * 4 + i4] = t[ct].acc[dt][i4];
+            }
+        }
+        __syncthreads();
+        if (set > 0) return;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            float m = t[ct].m;
+            for (int other = 1; other < KG; ++other)
+                m = fmaxf(m, sums[((((size_t)(other - 1) * 4 + wave) * CT + ct) * 64 + lane) * STRIDE]);
+            const float base = (m == -INFINITY) ? 0.f : m;
+            float f = __builtin_amdgcn_exp2f(t[ct].m - base);
+            float l = tile_sum(t[ct]) * f;
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) t[ct].acc[dt][i4] *= f;
+            for (int other = 1; other < KG; ++other) {
+                const float* src = sums + ((((size_t)(other - 1) * 4 + wave) * CT + ct) * 64 + lane) * STRIDE;
+                f = __builtin_amdgcn_exp2f(src[0] - base);
+                l += src[1] * f;
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) t[ct].acc[dt][i4] += src[2 + dt * 4 + i4] * f;
+            }
+            t[ct].ls = (f32x4){l, l, l, l};
+            t[ct].l = 0.f;
+        }
+    }
 
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
@@ -1259,15 +1321,15 @@ __device__ __forceinline__ void prefill_pipe_block(
 // than early ones; `pair` says how the work is evened out: 1: (ceil(row blocks / 2), ...)
 // workgroups that each take block (last - b) and then block b; 2: long blocks placed beside
 // short ones on a compute unit; 3: long blocks first; 0: as the grid says.
-template <int NJ, int ND, int CT, int KB, bool DMA, int WAVES = 4>
-__global__ void __launch_bounds__(WAVES * 64, (WAVES == 4 && ND <= 8 && (CT == 2 || DMA)) ? 2 : 1)
+template <int NJ, int ND, int CT, int KB, bool DMA, int KG = 1>
+__global__ void __launch_bounds__(KG * 256, (KG == 1 && ND <= 8 && (CT == 2 || DMA)) ? 2 : 1)
 attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                              const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                              const int* __restrict__ row_start, const int* __restrict__ seq_start,
                              int num_seqs, const int* __restrict__ tables, int table_width, int page_size,
                              int page_shift, int num_pages, int heads, int kv_heads,
                              float scale_log2, int window, int rq, int pair, RawQkv raw) {
-    const int rows_per_block = WAVES * CT * rq;
+    const int rows_per_block = 4 * CT * rq;
     int total = 0;
     for (int seq = 0; seq < num_seqs; ++seq)
         total += (row_start[seq + 1] - row_start[seq] + rows_per_block - 1) / rows_per_block;
@@ -1309,7 +1371,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
         if (pass) __syncthreads();                            // (the buffers are used again)
         const int block = pass ? rb2 : rb;
         if constexpr (DMA)
-            prefill_pipe_block<NJ, ND, CT, WAVES>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
+            prefill_pipe_block<NJ, ND, CT, KG>(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, tables,
                                                   table_width, page_size, page_shift, num_pages, heads, kv_heads,
                                                   scale_log2, window, rq, block, hd_i, raw);
         else
@@ -1459,25 +1521,44 @@ static int launch_prefill(
                         "of at least 8 (%d), through LDS", head_dim, page_size);
     const RawQkv raw = raw_in ? *raw_in : RawQkv{};
     if (page_size >= 8 && direct != 1) {
-        // through LDS, blocks of 64 keys (32 for large heads).  Two column tiles a wave when
-        // that still gives two workgroups for every compute unit (long row blocks then come
-        // first); else one tile a wave.
+        // through LDS.  Two column tiles a wave when that still gives two workgroups for every
+        // compute unit (long row blocks then come first); else one tile a wave.
+        const long blocks1 = (rows + 4 * rq - 1) / (4 * rq) + num_seqs;
         const long blocks2 = (rows + 8 * rq - 1) / (8 * rq) + num_seqs;
         bool two = head_dim <= 128 && blocks2 * kv_heads * head_tiles >= 512;
+        // Heads of 64 and 128, while the chip has room for every workgroup at once: the longest
+        // workgroups decide the time, and two sets of waves a workgroup walk a workgroup's keys in
+        // half the rounds (one workgroup a compute unit then: two tiles a wave where one tile would
+        // make more than 256 workgroups).  Measured from 256 to 4,096 tokens, and portions of 512 to
+        // 2,048 tokens behind up to 30,720: up to a third faster while all workgroups run at once
+        // (256), a tenth faster up to 512 workgroups whose rows have no keys before them (the short
+        // ones fill the second round), 3 to 15% slower there with keys before them (direct = 13 says
+        // so: the lengths are on the device) and slower beyond.
+        const bool dma = head_dim == 64 || head_dim == 128;
+        const long groups2 = (blocks2 - num_seqs) * kv_heads * head_tiles;
+        bool sets = dma && groups2 <= (direct == 13 ? 256 : 512);
+        if (sets) two = (blocks1 - num_seqs) * kv_heads * head_tiles > 256;
+        // rows with keys before them are all about as long: two tiles a wave, which read the keys
+        // once for both, already pay when one round of them fills the chip (1,536 rows behind
+        // 6,656 keys: a fifth faster than one tile a wave)
+        else if (dma && direct == 13 && groups2 > 256) two = true;
         if (direct == 2) two = false;
         if (direct == 3 || (direct >= 4 && direct <= 7)) two = head_dim <= 128;
         if (direct == 8) two = false;
         if (head_dim == 112) two = false;                         // (two tiles of that size do not fit a wave's registers)
+        if (direct == 12) two = true;                             // (measurements: 10 two sets, 11 one set, 12 two tiles in two sets)
+        if (direct == 10 || direct == 12) sets = dma;
+        if (direct == 11) sets = false;
         const int rows_per_block = 4 * rq * (two ? 2 : 1);
         const long blocks = (rows + rows_per_block - 1) / rows_per_block + num_seqs;   // upper bound
         if (blocks > 2147483647L) return tli_fail("attention_prefill: too many rows");
         int pair = two ? 3 : (blocks * kv_heads * head_tiles >= 1024 ? 1 : 2);
         if (direct >= 4 && direct <= 7) pair = direct - 4;        // measurements: 4..7 force the pairing mode, two tiles
         if (direct == 8) pair = 3;                                // one tile, long blocks first
+        if (sets && !(direct >= 4 && direct <= 7)) pair = 3;      // (one workgroup a compute unit: long blocks first)
         dim3 grid((unsigned)(pair == 1 ? (blocks + 1) / 2 : blocks), kv_heads * head_tiles);
         const int kb = head_dim <= 128 ? 64 : 32;
         // heads of 64 and 128: 32 keys a step copied straight into four LDS buffers
-        const bool dma = head_dim == 64 || head_dim == 128;
         const size_t lds = dma ? (size_t)4 * 2 * 32 * head_dim * sizeof(bf16_t)
                                : ((size_t)kb * (head_dim + 8) + (size_t)head_dim * (kb + 8)) * sizeof(bf16_t);
 #define ARGS (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, row_start, \
@@ -1485,6 +1566,27 @@ static int launch_prefill(
 #define TAIL scale * LOG2E, window, rq
 #define TAIL_LDS scale * LOG2E, window, rq, pair, raw
 #define LDS_CALL(NJ, ND, CT, KB, DMA) attention_prefill_lds_kernel<NJ, ND, CT, KB, DMA><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS)
+        if (sets) {
+            const size_t lds2 = 2 * lds;
+#define SETS_CALL(NJ, ND, CT)                                                                            \
+    {                                                                                                    \
+        auto kernel = attention_prefill_lds_kernel<NJ, ND, CT, 32, true, 2>;                             \
+        static bool allowed = false;                                                                     \
+        if (lds2 > 65536 && !allowed) {                                                                  \
+            if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,     \
+                                    (int)lds2) != hipSuccess)                                            \
+                return tli_fail("attention_prefill: cannot have %zu bytes of LDS", lds2);                \
+            allowed = true;                                                                              \
+        }                                                                                                \
+        kernel<<<grid, 512, lds2, s>>>(ARGS, TAIL_LDS);                                                  \
+    }
+            if (head_dim == 128 && two) SETS_CALL(4, 8, 2)
+            else if (head_dim == 128) SETS_CALL(4, 8, 1)
+            else if (two) SETS_CALL(2, 4, 2)
+            else SETS_CALL(2, 4, 1)
+#undef SETS_CALL
+            return tli_check_launch("attention_prefill_lds");
+        }
 #define CALL(NJ, ND)                                                                                    \
     if ((ND == 4 || ND == 8) && two) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 2, 32, true); \
     else if (ND == 4 || ND == 8) LDS_CALL(((ND == 4 || ND == 8) ? ND / 2 : 2), ((ND == 4 || ND == 8) ? ND : 4), 1, 32, true); \

@@ -154,7 +154,7 @@ class HipOps:
         self.plain_products = False  # every matrix product through the plain kernel
         self.separate_norms = False  # tests: decode steps run their norms as kernels of their own
         self.unfused_decode = False  # tests: decode steps through qkv_to_cache and paged_attention too
-        self.prefill_direct = 0      # tests: 1 = the prefill attention kernel without LDS staging; 2, 3 = with, 1 or 2 tiles a wave; 4..8 = a forced order of row blocks
+        self.prefill_direct = 0      # tests: 1 = the prefill attention kernel without LDS staging; 2, 3 = with, 1 or 2 tiles a wave; 4..8 = a forced order of row blocks; 10, 11 = heads of 64 and 128 with two sets of waves a workgroup, with one; 13 = as 0 for rows with many keys before them
         self.mid_cfg = 0             # measurements: launch shape and k ranges of the 17..128-row kernel
         self.mid_splits = 0
         self.skinny_cfg = 0          # measurements: force a launch shape of the weight-streaming kernel
@@ -573,7 +573,7 @@ class HipOps:
             self._call(self.lib.tli_attention_prefill_bf16, q.data_ptr(), out.data_ptr(), kc.data_ptr(),
                        vc.data_ptr(), step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs,
                        T, g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], heads, kv_heads,
-                       head_dim, float(scale), int(window or 0), int(self.prefill_direct),
+                       head_dim, float(scale), int(window or 0), self._prefill_mode(step, T),
                        self._stream())
             return out
         self._call(self.lib.tli_attention_plain, q.data_ptr(), out.data_ptr(), kc.data_ptr(),
@@ -677,13 +677,22 @@ class HipOps:
                        0, float(scale), int(window or 0), splits, per_split, None, 0, self._stream())
         else:
             first = 0
+        direct = self._prefill_mode(step, T - first)
         self._call(self.lib.tli_qkv_attention_prefill_bf16, qkv.data_ptr(), out.data_ptr(), kc.data_ptr(),
                    vc.data_ptr(), step.row_start.data_ptr() + 4 * first, step.seq_start.data_ptr() + 4 * first,
                    step.num_seqs - first, T - first, g.tables.data_ptr() + 4 * first * g.table_width, g.table_width,
                    g.page_size, kc.shape[0], heads, kv_heads,
                    head_dim, _ptr(qw), float(qe), _ptr(cos), _ptr(sin), float(scale), int(window or 0),
-                   int(self.prefill_direct), self._stream())
+                   direct, self._stream())
         return out
+
+    def _prefill_mode(self, step, rows):
+        """The mode argument of the prefill attention kernels.  Their launch rule wants to know
+        whether the rows have many keys before them, and the lengths themselves are on the
+        device: 13 says that they have (the longest sequence is a quarter longer than all rows)."""
+        if not self.prefill_direct and step.max_seq_len > rows + rows // 4:
+            return 13
+        return int(self.prefill_direct)
 
     def _decode_splits(self, T, reach, g, heads, kv_heads, head_dim, window):
         """How the keys of ``T`` rows that decode (``reach``: a power of two that the longest
