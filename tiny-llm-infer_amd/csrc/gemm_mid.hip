@@ -93,7 +93,9 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
         for (int t = 0; t < RT; ++t)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                a[S][t][j].u = *reinterpret_cast<const uint4*>(w_tile[t] + (size_t)step * 2048 + j * 512);
+                // (read once a step, a whole KiB an instruction: not to be kept by the caches, which
+                // hold what every kernel begins with; see gemm_skinny.hip)
+                a[S][t][j].q = __builtin_nontemporal_load(reinterpret_cast<const u32x4m*>(w_tile[t] + (size_t)step * 2048 + j * 512));
     };
     // What this lane asks for in copy e of a slice: LDS place (e WAVES + wave) 64 + lane, that
     // is row place / 16 and the chunk that belongs at chunk place % 16 of that row.  Rows past
