@@ -45,6 +45,29 @@ __device__ __forceinline__ void from_f32(bf16_t* p, float v) { *p = f32_to_bf16(
 __device__ __forceinline__ bf16_t cache_value(bf16_t v) { return (v & 0x7F80u) == 0x7F80u ? (bf16_t)0 : v; }
 __device__ __forceinline__ float cache_value(float v) { return (__float_as_uint(v) & 0x7F800000u) == 0x7F800000u ? 0.f : v; }
 
+// Four values that a lane holds for four consecutive columns, as one store where the row allows it
+// (`left`: columns from dst to the row's end; `whole`: every row starts a multiple of four columns
+// in, so that the store is aligned), else one by one.
+__device__ __forceinline__ void store4(float* dst, const float (&v)[4], int left, bool whole) {
+    if (left >= 4 && whole) {
+        *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (i < left) dst[i] = v[i];
+}
+__device__ __forceinline__ void store4(bf16_t* dst, const float (&v)[4], int left, bool whole) {
+    if (left >= 4 && whole) {
+        *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16),
+                                                    (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16));
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (i < left) dst[i] = f32_to_bf16(v[i]);
+}
+
 // Makes LDS writes of this wavefront's lanes visible to its other lanes.
 __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

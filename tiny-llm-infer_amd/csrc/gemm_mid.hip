@@ -209,6 +209,10 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
             for (int m = 0; m < MT; ++m) {
                 const int row = m * 16 + r;
                 if (row >= M) continue;
+                if (n0 + 3 < N && (N & 3) == 0) {           // (the lane's four sums in one store)
+                    *reinterpret_cast<f32x4*>(dst + (size_t)row * N + n0) = acc[t][m];
+                    continue;
+                }
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     if (n0 + i < N) dst[(size_t)row * N + n0 + i] = acc[t][m][i];
@@ -225,12 +229,13 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
             for (int m = 0; m < MT; ++m) {
                 const int row = m * 16 + r;
                 if (row >= M) continue;
+                float o[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (n0 + i < n_out) {
-                        const float g = acc[t][m][i], u = acc[t + 1][m][i];
-                        from_f32(y + (size_t)row * n_out + n0 + i, g / (1.0f + expf(-g)) * u);
-                    }
+                for (int i = 0; i < 4; ++i) {
+                    const float g = acc[t][m][i], u = acc[t + 1][m][i];
+                    o[i] = g / (1.0f + expf(-g)) * u;
+                }
+                store4(y + (size_t)row * n_out + n0, o, n_out - n0, (n_out & 3) == 0);
             }
         }
         return;
@@ -242,9 +247,8 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
         for (int m = 0; m < MT; ++m) {
             const int row = m * 16 + r;
             if (row >= M) continue;
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (n0 + i < N) from_f32(y + (size_t)row * N + n0 + i, acc[t][m][i]);
+            const float o[4] = {acc[t][m][0], acc[t][m][1], acc[t][m][2], acc[t][m][3]};
+            store4(y + (size_t)row * N + n0, o, N - n0, (N & 3) == 0);
         }
     }
 }
@@ -368,7 +372,7 @@ extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* p
     if (splits < 1 || splits > 64) return tli_fail("gemm_mid: %d splits", splits);
     if (splits > 1 && !part) return tli_fail("gemm_mid: splits need a buffer for partial sums");
     if (!y && (splits < 2 || gated)) return tli_fail("gemm_mid: only a plain product with split k can leave its partial sums");
-    if (((uintptr_t)x | (uintptr_t)w) & 15) return tli_fail("gemm_mid: operands must be 16-byte aligned");
+    if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)part | (uintptr_t)y) & 15) return tli_fail("gemm_mid: operands must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xp = (const bf16_t*)x;
     const bf16_t* wp = (const bf16_t*)w;

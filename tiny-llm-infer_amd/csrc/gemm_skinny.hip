@@ -277,10 +277,10 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
                 }
             }
             if (row < M) {
+                float o[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (n0 + i < n_out)
-                        from_f32(y + (size_t)row * n_out + n0 + i, g[i] / (1.0f + expf(-g[i])) * u[i]);
+                for (int i = 0; i < 4; ++i) o[i] = g[i] / (1.0f + expf(-g[i])) * u[i];
+                store4(y + (size_t)row * n_out + n0, o, n_out - n0, (n_out & 3) == 0);
             }
         }
         return;
@@ -296,15 +296,17 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
         const int n0 = n_base + t * 16 + c * 4;
         if (FUSE == FUSE_RESIDUAL) {
             // (MT == 1 and tile == wave: the values asked for at the start are this tile's)
-            float ssq = 0.f;
+            float ssq = 0.f, h[4], hw[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (row < M && n0 + i < N) {
-                    const float h = h_old[i] + s[i];
-                    fuse.resid[(size_t)row * N + n0 + i] = h;
-                    fuse.xw[(size_t)row * N + n0 + i] = f32_to_bf16(nw[i] * h);
-                    ssq += h * h;
-                }
+            for (int i = 0; i < 4; ++i) {
+                h[i] = h_old[i] + s[i];
+                hw[i] = nw[i] * h[i];
+                if (row < M && n0 + i < N) ssq += h[i] * h[i];
+            }
+            if (row < M) {
+                store4(fuse.resid + (size_t)row * N + n0, h, N - n0, (N & 3) == 0);
+                store4(fuse.xw + (size_t)row * N + n0, hw, N - n0, (N & 3) == 0);
+            }
             ssq = quad_rows_sum(ssq);                  // over the tile's 16 columns
             if (c == 0 && row < M) fuse.ssq_out[(size_t)(blockIdx.x * RT + t) * M + row] = ssq;
             continue;
@@ -313,11 +315,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
 #pragma unroll
             for (int i = 0; i < 4; ++i) s[i] *= rstd[m];
         }
-        if (row < M) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (n0 + i < N) from_f32(y + (size_t)row * N + n0 + i, s[i]);
-        }
+        if (row < M) store4(y + (size_t)row * N + n0, s, N - n0, (N & 3) == 0);
     }
 }
 
@@ -380,7 +378,7 @@ extern "C" int tli_gemm_skinny_bf16(const void* x, const void* w, void* y, int M
     if (tiled < 0 || tiled > 2) return tli_fail("gemm_skinny: bad layout code %d", tiled);
     if (tiled == 2 && (N % 32 || y_dtype != TLI_BF16))
         return tli_fail("gemm_skinny: a gated product needs N %% 32 == 0 and bfloat16 output");
-    if (((uintptr_t)x | (uintptr_t)w) & 15) return tli_fail("gemm_skinny: operands must be 16-byte aligned");
+    if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 15) return tli_fail("gemm_skinny: operands must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xp = (const bf16_t*)x;
     const bf16_t* wp = (const bf16_t*)w;
@@ -421,7 +419,8 @@ extern "C" int tli_gemm_skinny_fused_bf16(const void* x, const void* w, void* y,
     if (resid && (gated || !norm_w || !xw || !ssq_out)) return tli_fail("gemm_skinny into the residual: missing arguments");
     if (ssq_in && (parts_in <= 0 || !y)) return tli_fail("gemm_skinny with sums of squares: missing arguments");
     if (gated && N % 32) return tli_fail("gemm_skinny: a gated product needs N %% 32 == 0");
-    if (((uintptr_t)x | (uintptr_t)w) & 15) return tli_fail("gemm_skinny: operands must be 16-byte aligned");
+    if (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y | (uintptr_t)resid | (uintptr_t)xw) & 15)
+        return tli_fail("gemm_skinny: operands must be 16-byte aligned");
     const SkinnyFuse f{ssq_in, parts_in, eps, resid, norm_w, (bf16_t*)xw, ssq_out};
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xp = (const bf16_t*)x;
