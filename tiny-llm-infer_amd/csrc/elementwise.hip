@@ -120,11 +120,17 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const void* __
             if (d.any()) {
                 float dv[4];
                 if (d.parts > 0) {
+                    // four planes a round, all asked for before any is added (in plane order; a plane
+                    // past the last is the last again and is not added)
                     float a[4] = {0.f, 0.f, 0.f, 0.f};
-                    for (int s = 0; s < d.parts; ++s) {
-                        load4(d.p + s * d.plane + i, dv);
+                    for (int s = 0; s < d.parts; s += 4) {
+                        float pv[4][4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) a[e] += dv[e];
+                        for (int k = 0; k < 4; ++k) load4(d.p + (size_t)min(s + k, d.parts - 1) * d.plane + i, pv[k]);
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) a[e] = s + k < d.parts ? a[e] + pv[k][e] : a[e];
                     }
 #pragma unroll
                     for (int e = 0; e < 4; ++e) dv[e] = bf16_to_f32(f32_to_bf16(a[e]));
