@@ -279,12 +279,8 @@ static int launch_mid_rows(const bf16_t* x, const bf16_t* w, void* y, float* par
 #undef MID_LAUNCH
     if (tli_check_launch("gemm_mid")) return 1;
     if (splits > 1 && y) {
-        const size_t total = (size_t)M * (gated ? N / 2 : N);
-        const unsigned blocks = (unsigned)((total + 255) / 256);
-        if (y_dtype == TLI_BF16)
-            gemm_mid_reduce_kernel<bf16_t><<<blocks, 256, 0, s>>>(part, (bf16_t*)y, M, N, splits, gated);
-        else
-            gemm_mid_reduce_kernel<float><<<blocks, 256, 0, s>>>(part, (float*)y, M, N, splits, gated);
+        if (y_dtype == TLI_BF16) launch_gemm_reduce(part, (bf16_t*)y, M, N, splits, gated, s);
+        else launch_gemm_reduce(part, (float*)y, M, N, splits, gated, s);
         return tli_check_launch("gemm_mid_reduce");
     }
     return 0;
@@ -404,13 +400,8 @@ extern "C" int tli_gemm_mid_reduce(const float* part, void* y, int M, int N, int
     if (M <= 0 || N <= 0) return 0;
     if (!part || !y || splits < 1) return tli_fail("gemm_mid_reduce: bad arguments");
     hipStream_t s = (hipStream_t)stream;
-    const size_t total = (size_t)M * N;
-    const unsigned blocks = (unsigned)((total + 255) / 256);
-    if (y_dtype == TLI_BF16)
-        gemm_mid_reduce_kernel<bf16_t><<<blocks, 256, 0, s>>>(part, (bf16_t*)y, M, N, splits, 0);
-    else if (y_dtype == TLI_F32)
-        gemm_mid_reduce_kernel<float><<<blocks, 256, 0, s>>>(part, (float*)y, M, N, splits, 0);
-    else
-        return tli_fail("gemm_mid_reduce: bad output dtype %d", y_dtype);
+    if (y_dtype == TLI_BF16) launch_gemm_reduce(part, (bf16_t*)y, M, N, splits, 0, s);
+    else if (y_dtype == TLI_F32) launch_gemm_reduce(part, (float*)y, M, N, splits, 0, s);
+    else return tli_fail("gemm_mid_reduce: bad output dtype %d", y_dtype);
     return tli_check_launch("gemm_mid_reduce");
 }

@@ -378,8 +378,7 @@ static int launch_rows(const bf16_t* x, const bf16_t* w, bf16_t* y, float* part,
 #undef ROWS_LAUNCH
     if (tli_check_launch("gemm_rows")) return 1;
     if (splits > 1 && y) {
-        const size_t total = (size_t)M * (gated ? N / 2 : N);
-        gemm_mid_reduce_kernel<bf16_t><<<(unsigned)((total + 255) / 256), 256, 0, s>>>(part, y, M, N, splits, gated);
+        launch_gemm_reduce(part, y, M, N, splits, gated, s);
         return tli_check_launch("gemm_rows: sum of the partial products");
     }
     return 0;
