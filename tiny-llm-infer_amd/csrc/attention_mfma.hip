@@ -612,25 +612,38 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     }
 
     // a wave's blocks are 128 keys apart; the next block is asked for before this one is
-    // multiplied (the last block is asked for once more instead of branching round the loads)
+    // multiplied (in the loop the last block is asked for once more instead of branching round
+    // the loads).  A wave with one block or two, which is most waves of a short context, has
+    // them written out without the loop and asks for nothing twice: that second request was a
+    // tenth of the kernel's time there.
     int t0 = begin + wave * 32;
     if (t0 < end) {
         const int last = t0 + (end - 1 - t0) / 128 * 128;
         KeyBlock<NJ, ND> b0, b1;
         decode_fetch(b0, cv, seg, seg_first, seg_len, t0);
-        while (true) {
-            decode_fetch(b1, cv, seg, seg_first, seg_len, min(t0 + 128, last));
+        if (last == t0) {
+            tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 4 * c, 16, scale);
+        } else if (last == t0 + 128) {
+            decode_fetch(b1, cv, seg, seg_first, seg_len, last);
             __builtin_amdgcn_sched_barrier(0);
             tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 4 * c, 16, scale);
             __builtin_amdgcn_sched_barrier(0);
-            if (t0 + 128 > last) break;
-            t0 += 128;
-            decode_fetch(b0, cv, seg, seg_first, seg_len, min(t0 + 128, last));
-            __builtin_amdgcn_sched_barrier(0);
-            tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, t0 + 4 * c, 16, scale);
-            __builtin_amdgcn_sched_barrier(0);
-            if (t0 + 128 > last) break;
-            t0 += 128;
+            tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, last + 4 * c, 16, scale);
+        } else {
+            while (true) {
+                decode_fetch(b1, cv, seg, seg_first, seg_len, min(t0 + 128, last));
+                __builtin_amdgcn_sched_barrier(0);
+                tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 4 * c, 16, scale);
+                __builtin_amdgcn_sched_barrier(0);
+                if (t0 + 128 > last) break;
+                t0 += 128;
+                decode_fetch(b0, cv, seg, seg_first, seg_len, min(t0 + 128, last));
+                __builtin_amdgcn_sched_barrier(0);
+                tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, t0 + 4 * c, 16, scale);
+                __builtin_amdgcn_sched_barrier(0);
+                if (t0 + 128 > last) break;
+                t0 += 128;
+            }
         }
     }
 
