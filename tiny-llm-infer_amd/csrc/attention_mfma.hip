@@ -612,39 +612,38 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     }
 
     // a wave's blocks are 128 keys apart; the next block is asked for before this one is
-    // multiplied (in the loop the last block is asked for once more instead of branching round
-    // the loads).  A wave with one block or two, which is most waves of a short context, has
-    // them written out without the loop and asks for nothing twice: that second request was a
-    // tenth of the kernel's time there.
+    // multiplied, two sets of registers taking turns.  Nothing is asked for twice and no load
+    // of the loop is under a branch: the blocks are dealt to the two sets from the end, so that
+    // the last block always comes into the first set and is multiplied after the loop; a wave
+    // with an even number of blocks begins with one block in the second set.  (Asking for the
+    // last block once more instead, as a loop without this must, was a tenth of the kernel's
+    // time at the few hundred keys of a short context, where most waves have one block or two.)
     int t0 = begin + wave * 32;
     if (t0 < end) {
         const int last = t0 + (end - 1 - t0) / 128 * 128;
         KeyBlock<NJ, ND> b0, b1;
-        decode_fetch(b0, cv, seg, seg_first, seg_len, t0);
-        if (last == t0) {
-            tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 4 * c, 16, scale);
-        } else if (last == t0 + 128) {
-            decode_fetch(b1, cv, seg, seg_first, seg_len, last);
+        if (((last - t0) / 128) & 1) {          // an even number of blocks
+            decode_fetch(b1, cv, seg, seg_first, seg_len, t0);
+            decode_fetch(b0, cv, seg, seg_first, seg_len, t0 + 128);
             __builtin_amdgcn_sched_barrier(0);
-            tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 4 * c, 16, scale);
+            tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, t0 + 4 * c, 16, scale);
             __builtin_amdgcn_sched_barrier(0);
-            tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, last + 4 * c, 16, scale);
+            t0 += 128;
         } else {
-            while (true) {
-                decode_fetch(b1, cv, seg, seg_first, seg_len, min(t0 + 128, last));
-                __builtin_amdgcn_sched_barrier(0);
-                tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 4 * c, 16, scale);
-                __builtin_amdgcn_sched_barrier(0);
-                if (t0 + 128 > last) break;
-                t0 += 128;
-                decode_fetch(b0, cv, seg, seg_first, seg_len, min(t0 + 128, last));
-                __builtin_amdgcn_sched_barrier(0);
-                tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, t0 + 4 * c, 16, scale);
-                __builtin_amdgcn_sched_barrier(0);
-                if (t0 + 128 > last) break;
-                t0 += 128;
-            }
+            decode_fetch(b0, cv, seg, seg_first, seg_len, t0);
         }
+        while (t0 != last) {                      // the first set holds block t0, an even number of blocks follow
+            decode_fetch(b1, cv, seg, seg_first, seg_len, t0 + 128);
+            __builtin_amdgcn_sched_barrier(0);
+            tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 4 * c, 16, scale);
+            __builtin_amdgcn_sched_barrier(0);
+            decode_fetch(b0, cv, seg, seg_first, seg_len, t0 + 256);
+            __builtin_amdgcn_sched_barrier(0);
+            tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, t0 + 128 + 4 * c, 16, scale);
+            __builtin_amdgcn_sched_barrier(0);
+            t0 += 256;
+        }
+        tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 4 * c, 16, scale);
     }
 
     // merge the four waves: waves 1..3 hand over (m, l, acc), wave 0 combines in wave order
