@@ -1157,10 +1157,9 @@ __device__ __forceinline__ void prefill_pipe_block(
                      ::"s"(lds_base), "s"(lds_byte), "v"(lane_off), "s"(base)
                      : "m0", "scc", "memory");
     };
-    // start the copies of block `step` into its buffer (called for every step in turn; past the
-    // last block the last one is copied again, rather than a branch that would change what is in flight)
+    // start the copies of block `step` < n into its buffer (called for every block in turn)
     auto copy = [&](int step) {
-        const int t0 = T0 + min(step, n - 1) * BK;
+        const int t0 = T0 + step * BK;
         if ((step & (16 / KG - 1)) == 0) {
             tab_first = t0 >> page_shift;
             // (loaded and waited for in assembly, like the copies: the compiler then knows of no load
@@ -1184,11 +1183,19 @@ __device__ __forceinline__ void prefill_pipe_block(
             dma(kb + (uint32_t)(TILE * sizeof(bf16_t)) + (e * WAVES + wave_u) * 1024, v_loff[e], v_base + page_off);
         }
     };
-    // the top of iteration i
+    // the top of iteration i.  In flight are this wave's copies of block i+1 and, if there is one,
+    // of block i+2, in that order: past the last block nothing is copied (copying the last one again
+    // instead was a third more copies for a workgroup of average length at 2,048 tokens), and the
+    // wait counts what is there.  (i and the number of blocks are in scalar registers: the
+    // branches are the same for the whole workgroup.)
+    const int n_s = __builtin_amdgcn_readfirstlane(n);
     auto top = [&](int i) {
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER) : "memory");     // this wave's part of block i+1 has landed
+        if (i + 2 < n_s)
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER) : "memory");     // this wave's part of block i+1 has landed
+        else
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();                                               // everyone's has, and nobody reads block i-1 any more
-        copy(i + 3);
+        if (i + 3 < n_s) copy(i + 3);
     };
 
     // LDS offsets (elements) of this lane's fragments in a buffer: the keys from row 32 set of the
@@ -1214,7 +1221,7 @@ __device__ __forceinline__ void prefill_pipe_block(
 
     f32x4 ex[CT][2];                                  // the exponents of the step whose weights come next
     copy(0);
-    copy(1);
+    if (1 < n_s) copy(1);
     int i = -1;
     for (; i < a - 1; ++i) top(i);                    // blocks before this wave's keys
     if (a <= b) {
