@@ -509,6 +509,63 @@ __device__ __forceinline__ void head_from_raw(Frag (&out)[NJ], const bf16_t* src
                               pack_bf16x2(x[j][4], x[j][5]), pack_bf16x2(x[j][6], x[j][7]));
 }
 
+// The decode kernel's prologue shares the work on a head out over the four waves by slices of 8
+// dims a lane (slice j of a lane: dims c*8*NJ + 8j ..): a wave fetches its slices, the waves
+// exchange their parts of the sum of squares through LDS, and each finishes its slices.
+// Eight elements of a head at `src` (bfloat16), or, with psrc, their sums over `parts` planes of
+// float32 partial sums in part order (two planes a round, both asked for before either is
+// added), rounded to bfloat16 as the product's own reduction would have.
+__device__ __forceinline__ void slice_fetch(float (&x)[8], const bf16_t* src, const float* psrc, int parts,
+                                            size_t part_stride) {
+    if (psrc) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = 0.f;
+        for (int p = 0; p < parts; p += 2) {
+            const bool pair = p + 1 < parts;
+            const float* from0 = psrc + (size_t)p * part_stride;
+            const float* from1 = psrc + (size_t)(pair ? p + 1 : p) * part_stride;
+            const f32x4 a0 = *reinterpret_cast<const f32x4*>(from0), a1 = *reinterpret_cast<const f32x4*>(from0 + 4);
+            const f32x4 b0 = *reinterpret_cast<const f32x4*>(from1), b1 = *reinterpret_cast<const f32x4*>(from1 + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                x[e] += a0[e];
+                x[e] += pair ? b0[e] : 0.f;
+                x[4 + e] += a1[e];
+                x[4 + e] += pair ? b1[e] : 0.f;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = bf16_to_f32(f32_to_bf16(x[e]));
+    } else {
+        Frag f;
+        f.u = *reinterpret_cast<const uint4*>(src);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = bf16_to_f32(f.e[e]);
+    }
+}
+
+// A slice after the norm (factor `scale`, weights nw8 or null) and the half-split rotation
+// (cos8, sin8 of the slice's dims, or null), as the score MFMAs take it.  The rotation partner
+// of a lane is lane ^ 32 (head_dim == 32*NJ: the first half of the head lies in lane groups 0, 1).
+__device__ __forceinline__ uint4 slice_finish(float (&x)[8], const float* nw8, float scale, const float* cos8,
+                                              const float* sin8) {
+    const int c = (threadIdx.x % 64) / 16;
+    if (nw8) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = nw8[e] * x[e] * scale;
+    }
+    if (cos8) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float partner = __shfl_xor(x[e], 32, 64);
+            const float cs = cos8[e], sn = sin8[e];
+            // first half: x cos - partner sin; second half: partner sin + x cos
+            x[e] = c < 2 ? x[e] * cs - partner * sn : partner * sn + x[e] * cs;
+        }
+    }
+    return make_uint4(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]), pack_bf16x2(x[4], x[5]), pack_bf16x2(x[6], x[7]));
+}
+
 // grid (splits, kv_heads * head_tiles, rows); 256 threads.  FUSED: queries come from the
 // raw projections `raw` (q is not read), and the workgroup whose keys include the row's
 // own position writes that key and value into the cache first; needs head_dim == 32*NJ
@@ -521,7 +578,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
                         const int* __restrict__ tables, int table_width, int page_size, int page_shift,
                         int num_pages, int heads, int kv_heads, int head_dim, float scale, int window,
                         int splits, int keys_per_split, RawQkv raw) {
-    extern __shared__ float lds[];       // 3 waves x 64 lanes x (ND*4 + 2), then this split's table entries
+    extern __shared__ float lds[];       // 3 waves x 64 lanes x (ND*4 + 2), then this split's table entries, FUSED: the prologue's sums of squares and slices of q
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, c = lane / 16;
     const int split = blockIdx.x, row = blockIdx.z;
     const int group = heads / kv_heads;
@@ -540,23 +597,6 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     tile_init(t);
     t.pos = live ? pos : -1;
     t.lo = live ? lo : 0;
-    const bf16_t* raw_row = nullptr;
-    const float* sums_row = nullptr;         // this row in the first plane of partial sums, if the projections come so
-    const float *cos_row = nullptr, *sin_row = nullptr;
-    if (FUSED) {
-        raw_row = raw.qkv + (size_t)row * (heads + 2 * kv_heads) * head_dim;
-        if (raw.partial_sums) sums_row = raw.partial_sums + (size_t)row * (heads + 2 * kv_heads) * head_dim;
-        if (raw.cos) {
-            cos_row = raw.cos + (size_t)pos * (head_dim / 2);
-            sin_row = raw.sin + (size_t)pos * (head_dim / 2);
-        }
-        // (an idle column computes on head 0; it is masked by its pos of -1)
-        head_from_raw<NJ>(t.q, raw_row + (size_t)(live ? head : 0) * head_dim, raw.q_norm_w, raw.q_eps, cos_row, sin_row,
-                          sums_row ? sums_row + (size_t)(live ? head : 0) * head_dim : nullptr, raw.parts, raw.part_stride);
-    } else {
-        tile_load_q(t, q + ((size_t)row * heads + (live ? head : 0)) * head_dim, head_dim, live);
-    }
-
     // this split's keys, in 32-key blocks that the waves take in turn
     const int first_block = lo / 32;
     const int begin = first_block * 32 + split * keys_per_split;
@@ -566,48 +606,104 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     int* seg = reinterpret_cast<int*>(lds + 3 * 64 * (ND * 4 + 2));
     const int seg_first = begin >> page_shift;
     const int seg_len = begin < end ? ((end - 1) >> page_shift) - seg_first + 1 : 0;
-    for (int i = threadIdx.x; i < seg_len; i += 256)
-        seg[i] = seg_first + i < table_width ? table[seg_first + i] : -1;
-    __syncthreads();
-    if (FUSED && raw.write_cache) {
-        // the row's own key and value: written by the workgroup that reads them below
-        if (begin <= pos && pos < end) {
-            const int page = seg[(pos >> page_shift) - seg_first];
-            const int slot = pos & (page_size - 1);
-            if ((unsigned)page < (unsigned)num_pages) {
-                if (wave == 0) {
-                    Frag kf[NJ];
-                    head_from_raw<NJ>(kf, raw_row + (size_t)(heads + kv_head) * head_dim, raw.k_norm_w, raw.k_eps,
-                                      cos_row, sin_row,
-                                      sums_row ? sums_row + (size_t)(heads + kv_head) * head_dim : nullptr, raw.parts,
-                                      raw.part_stride);
-                    bf16_t* dst = k_cache + (((size_t)page * kv_heads + kv_head) * page_size + slot) * head_dim + c * 8 * NJ;
-                    if (r == 0) {
+    if (FUSED) {
+        // The prologue (see slice_fetch): wave w has the slices j = w, w + 4, .. of the lane's query
+        // head and, where this workgroup writes the row's own key, of the key head.
+        constexpr int SJ = (NJ + 3) / 4;                  // slices a wave at most
+        float* ssq = reinterpret_cast<float*>(seg + (((keys_per_split >> page_shift) + 2 + 3) & ~3));   // [q, k][wave][16]
+        uint4* q_slices = reinterpret_cast<uint4*>(ssq + 2 * 4 * 16);                                   // [NJ][64]
+        const size_t width = (size_t)(heads + 2 * kv_heads) * head_dim;
+        const bf16_t* raw_row = raw.qkv + (size_t)row * width;
+        const float* sums_row = raw.partial_sums ? raw.partial_sums + (size_t)row * width : nullptr;
+        const bool own = raw.write_cache && begin <= pos && pos < end;       // the row's own key and value are this workgroup's
+        // (an idle column computes on head 0; it is masked by its pos of -1)
+        const size_t q_off = (size_t)(live ? head : 0) * head_dim + c * 8 * NJ;
+        const size_t k_off = (size_t)(heads + kv_head) * head_dim + c * 8 * NJ;
+        float xq[SJ][8], xk[SJ][8];
+        float sq = 0.f, sk = 0.f;
 #pragma unroll
-                        for (int j = 0; j < NJ; ++j) *reinterpret_cast<uint4*>(dst + j * 8) = kf[j].u;
-                    }
-                } else if (wave == 1) {
-                    const bf16_t* src = raw_row + (size_t)(heads + kv_heads + kv_head) * head_dim;
-                    bf16_t* dst = v_cache + ((size_t)page * kv_heads + kv_head) * head_dim * page_size + slot;
-                    if (sums_row) {
-                        const float* from = sums_row + (size_t)(heads + kv_heads + kv_head) * head_dim;
-                        for (int d = lane; d < head_dim; d += 64) {
-                            float v = 0.f;
-                            for (int p = 0; p < raw.parts; p += 2) {
-                                const bool pair = p + 1 < raw.parts;
-                                const float a = from[(size_t)p * raw.part_stride + d];
-                                const float b = from[(size_t)(pair ? p + 1 : p) * raw.part_stride + d];
-                                v += a;
-                                v += pair ? b : 0.f;
-                            }
-                            dst[(size_t)d * page_size] = cache_value(f32_to_bf16(v));
-                        }
-                    } else {
-                        for (int d = lane; d < head_dim; d += 64) dst[(size_t)d * page_size] = cache_value(src[d]);
-                    }
+        for (int jj = 0; jj < SJ; ++jj) {
+            const int j = jj * 4 + wave;
+            if (j < NJ) {
+                slice_fetch(xq[jj], raw_row + q_off + j * 8, sums_row ? sums_row + q_off + j * 8 : nullptr, raw.parts,
+                            raw.part_stride);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sq += xq[jj][e] * xq[jj][e];
+                if (own) {
+                    slice_fetch(xk[jj], raw_row + k_off + j * 8, sums_row ? sums_row + k_off + j * 8 : nullptr, raw.parts,
+                                raw.part_stride);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) sk += xk[jj][e] * xk[jj][e];
                 }
             }
         }
+        sq = quad_rows_sum(sq);
+        sk = quad_rows_sum(sk);
+        if (c == 0) {
+            ssq[wave * 16 + r] = sq;
+            ssq[(4 + wave) * 16 + r] = sk;
+        }
+        for (int i = threadIdx.x; i < seg_len; i += 256)
+            seg[i] = seg_first + i < table_width ? table[seg_first + i] : -1;
+        __syncthreads();
+        const float q_ss = ssq[r] + ssq[16 + r] + ssq[32 + r] + ssq[48 + r];
+        const float k_ss = ssq[64 + r] + ssq[80 + r] + ssq[96 + r] + ssq[112 + r];
+        const float q_scale = 1.0f / sqrtf(q_ss / (float)(32 * NJ) + raw.q_eps);
+        const float k_scale = 1.0f / sqrtf(k_ss / (float)(32 * NJ) + raw.k_eps);
+        const float *cos_row = nullptr, *sin_row = nullptr;
+        if (raw.cos) {
+            cos_row = raw.cos + (size_t)pos * (head_dim / 2) + (c & 1) * 8 * NJ;
+            sin_row = raw.sin + (size_t)pos * (head_dim / 2) + (c & 1) * 8 * NJ;
+        }
+        int own_page = -1;
+        const int slot = pos & (page_size - 1);
+        if (own) own_page = seg[(pos >> page_shift) - seg_first];
+        const bool store = own && (unsigned)own_page < (unsigned)num_pages;
+#pragma unroll
+        for (int jj = 0; jj < SJ; ++jj) {
+            const int j = jj * 4 + wave;
+            if (j < NJ) {
+                const float* cos8 = cos_row ? cos_row + j * 8 : nullptr;
+                const float* sin8 = sin_row ? sin_row + j * 8 : nullptr;
+                q_slices[j * 64 + lane] = slice_finish(xq[jj], raw.q_norm_w ? raw.q_norm_w + c * 8 * NJ + j * 8 : nullptr,
+                                                       q_scale, cos8, sin8);
+                if (own) {
+                    const uint4 kf = slice_finish(xk[jj], raw.k_norm_w ? raw.k_norm_w + c * 8 * NJ + j * 8 : nullptr,
+                                                  k_scale, cos8, sin8);
+                    if (store && r == 0)
+                        *reinterpret_cast<uint4*>(k_cache + (((size_t)own_page * kv_heads + kv_head) * page_size + slot) * head_dim +
+                                                  c * 8 * NJ + j * 8) = kf;
+                }
+            }
+        }
+        if (store && wave == 3) {
+            // the value: two elements a lane
+            const bf16_t* src = raw_row + (size_t)(heads + kv_heads + kv_head) * head_dim;
+            bf16_t* dst = v_cache + ((size_t)own_page * kv_heads + kv_head) * head_dim * page_size + slot;
+            if (sums_row) {
+                const float* from = sums_row + (size_t)(heads + kv_heads + kv_head) * head_dim;
+                for (int d = lane; d < head_dim; d += 64) {
+                    float v = 0.f;
+                    for (int p = 0; p < raw.parts; p += 2) {
+                        const bool pair = p + 1 < raw.parts;
+                        const float a = from[(size_t)p * raw.part_stride + d];
+                        const float b = from[(size_t)(pair ? p + 1 : p) * raw.part_stride + d];
+                        v += a;
+                        v += pair ? b : 0.f;
+                    }
+                    dst[(size_t)d * page_size] = cache_value(f32_to_bf16(v));
+                }
+            } else {
+                for (int d = lane; d < head_dim; d += 64) dst[(size_t)d * page_size] = cache_value(src[d]);
+            }
+        }
+        __syncthreads();           // the slices of q are in LDS, the row's own key and value in the cache
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) t.q[j].u = q_slices[j * 64 + lane];
+    } else {
+        tile_load_q(t, q + ((size_t)row * heads + (live ? head : 0)) * head_dim, head_dim, live);
+        for (int i = threadIdx.x; i < seg_len; i += 256)
+            seg[i] = seg_first + i < table_width ? table[seg_first + i] : -1;
         __syncthreads();
     }
 
@@ -1463,7 +1559,7 @@ static int launch_decode(const void* q, void* out, float* partial, void* k_cache
     dim3 grid(splits, kv_heads * head_tiles, rows);
     const int shift = log2_exact(page_size);
     // the table entries of one split are kept in LDS
-    const size_t seg_bytes = ((size_t)(keys_per_split >> shift) + 2) * sizeof(int);
+    const size_t seg_bytes = ((((size_t)(keys_per_split >> shift) + 2) + 3) & ~(size_t)3) * sizeof(int);      // (16-byte aligned: the prologue's exchange comes behind it)
     if (seg_bytes > 8192)
         return tli_fail("attention_decode: %d keys per split in pages of %d are more than 2046 pages; use more splits",
                         keys_per_split, page_size);
@@ -1471,7 +1567,7 @@ static int launch_decode(const void* q, void* out, float* partial, void* k_cache
 #define ARGS (const bf16_t*)q, (bf16_t*)out, partial, (bf16_t*)k_cache, (bf16_t*)v_cache, positions, seq_of_row, \
              tables, table_width, page_size, shift, num_pages, heads, kv_heads, head_dim, scale * LOG2E, window, \
              splits, keys_per_split
-#define LDS_BYTES(ND) (3 * 64 * (ND * 4 + 2) * sizeof(float) + seg_bytes)
+#define LDS_BYTES(ND) (3 * 64 * (ND * 4 + 2) * sizeof(float) + seg_bytes + (raw ? 2 * 4 * 16 * sizeof(float) + (ND / 2) * 64 * sizeof(uint4) : 0))
 #define CALL(NJ, ND)                                                                                        \
     if (raw) attention_decode_kernel<NJ, ND, NJ * 2 == ND><<<grid, 256, LDS_BYTES(ND), s>>>(ARGS, *raw);   \
     else attention_decode_kernel<NJ, ND, false><<<grid, 256, LDS_BYTES(ND), s>>>(ARGS, none)
