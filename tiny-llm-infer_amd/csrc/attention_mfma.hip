@@ -366,13 +366,16 @@ struct KeyBlock {
     Frag vt[ND];
 };
 
-// Ask for the 32 keys t0 .. t0+31 (same lane-to-key plan as tiles_step).  `seg` holds the
-// block table entries seg_first .. seg_first+seg_len-1 in LDS.  No load is predicated, so
-// that the fragments of the next block can be in flight while this one is multiplied
-// (after a branch that may have issued loads the compiler waits for all loads in flight):
-// a key without a page reads page 0 instead.  Such keys lie outside lo..pos, their
-// scores are masked, and their values meet a weight of exactly 0; the cache is allocated
-// zeroed, so they are finite.
+// Ask for the 32 keys t0 .. t0+31.  Row 4c'+i of score tile u is the key t0 + 8c' + 4u + i
+// (tile_consume is told so: key_c0 = t0 + 8c, u_stride = 4): the eight keys that a lane group
+// multiplies the values of are then consecutive, and a lane takes them from the transposed
+// values in one 16-byte load; both key rows of a lane (tile 0 and 1, four keys apart) and all
+// its values lie in one page each, which holds at least 8 keys.  `seg` holds the block table
+// entries seg_first .. seg_first+seg_len-1 in LDS.  No load is predicated, so that the
+// fragments of the next block can be in flight while this one is multiplied (after a branch
+// that may have issued loads the compiler waits for all loads in flight): a key without a page
+// reads page 0 instead.  Such keys lie outside lo..pos, their scores are masked, and their
+// values meet a weight of exactly 0; the cache is allocated zeroed, so they are finite.
 template <int NJ, int ND>
 __device__ __forceinline__ void decode_fetch(KeyBlock<NJ, ND>& b, const CacheView& cv, const int* seg,
                                              int seg_first, int seg_len, int t0) {
@@ -383,27 +386,22 @@ __device__ __forceinline__ void decode_fetch(KeyBlock<NJ, ND>& b, const CacheVie
         return (unsigned)page < (unsigned)cv.num_pages ? page : 0;
     };
     const int in_page = cv.page_size - 1;
+    const int key_k = t0 + 8 * (r / 4) + (r % 4);                    // tile 0; tile 1 is four keys on
+    const bf16_t* kp = cv.k + (((size_t)page_at(key_k) * cv.kv_heads + cv.kv_head) * cv.page_size +
+                               (key_k & in_page)) * cv.head_dim;
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-        const int key = t0 + u * 16 + r;
-        const bf16_t* kp = cv.k + (((size_t)page_at(key) * cv.kv_heads + cv.kv_head) * cv.page_size +
-                                   (key & in_page)) * cv.head_dim;
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             const int d = c * 8 * NJ + j * 8;                        // past head_dim the query is zero
-            b.ka[u][j].u = *reinterpret_cast<const uint4*>(kp + (d < cv.head_dim ? d : 0));
+            b.ka[u][j].u = *reinterpret_cast<const uint4*>(kp + (size_t)u * 4 * cv.head_dim + (d < cv.head_dim ? d : 0));
         }
-    }
-    const int key_a = t0 + 4 * c, key_b = t0 + 16 + 4 * c;
-    const size_t head_stride = (size_t)cv.head_dim * cv.page_size;
-    const bf16_t* va = cv.v + ((size_t)page_at(key_a) * cv.kv_heads + cv.kv_head) * head_stride + (key_a & in_page);
-    const bf16_t* vb = cv.v + ((size_t)page_at(key_b) * cv.kv_heads + cv.kv_head) * head_stride + (key_b & in_page);
+    const int key_v = t0 + 8 * c;
+    const bf16_t* vp = cv.v + ((size_t)page_at(key_v) * cv.kv_heads + cv.kv_head) * ((size_t)cv.head_dim * cv.page_size) +
+                       (key_v & in_page);
 #pragma unroll
-    for (int dt = 0; dt < ND; ++dt) {
-        const size_t off = (size_t)(dt * 16 + r) * cv.page_size;
-        b.vt[dt].h[0] = *reinterpret_cast<const uint2*>(va + off);
-        b.vt[dt].h[1] = *reinterpret_cast<const uint2*>(vb + off);
-    }
+    for (int dt = 0; dt < ND; ++dt)
+        b.vt[dt].u = *reinterpret_cast<const uint4*>(vp + (size_t)(dt * 16 + r) * cv.page_size);
 }
 
 // The step's raw projections [rows][(heads + 2 kv_heads) * head_dim] and what turns them
@@ -722,7 +720,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
             decode_fetch(b1, cv, seg, seg_first, seg_len, t0);
             decode_fetch(b0, cv, seg, seg_first, seg_len, t0 + 128);
             __builtin_amdgcn_sched_barrier(0);
-            tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, t0 + 4 * c, 16, scale);
+            tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, t0 + 8 * c, 4, scale);
             __builtin_amdgcn_sched_barrier(0);
             t0 += 128;
         } else {
@@ -731,15 +729,15 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
         while (t0 != last) {                      // the first set holds block t0, an even number of blocks follow
             decode_fetch(b1, cv, seg, seg_first, seg_len, t0 + 128);
             __builtin_amdgcn_sched_barrier(0);
-            tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 4 * c, 16, scale);
+            tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 8 * c, 4, scale);
             __builtin_amdgcn_sched_barrier(0);
             decode_fetch(b0, cv, seg, seg_first, seg_len, t0 + 256);
             __builtin_amdgcn_sched_barrier(0);
-            tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, t0 + 128 + 4 * c, 16, scale);
+            tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, t0 + 128 + 8 * c, 4, scale);
             __builtin_amdgcn_sched_barrier(0);
             t0 += 256;
         }
-        tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 4 * c, 16, scale);
+        tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 8 * c, 4, scale);
     }
 
     // merge the four waves: waves 1..3 hand over (m, l, acc), wave 0 combines in wave order
@@ -1551,6 +1549,7 @@ static int launch_decode(const void* q, void* out, float* partial, void* k_cache
                         splits, keys_per_split);
     if (splits > 1 && !partial) return tli_fail("attention_decode: splits need a partial buffer");
     if (rows > 65535) return tli_fail("attention_decode: %d rows exceed the grid limit", rows);
+    if (page_size < 8) return tli_fail("attention_decode: pages of %d keys, the kernel takes pages of at least 8", page_size);
     hipStream_t s = (hipStream_t)stream;
     const int group = heads / kv_heads, head_tiles = (group + 15) / 16;
     if (raw && (head_dim % 64 || group > 16))

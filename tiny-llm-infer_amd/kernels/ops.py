@@ -568,7 +568,7 @@ class HipOps:
         self._check_cache(kc, vc, g, kv_heads, head_dim, q.dtype, step)
         out = torch.empty_like(q)
         if q.dtype == torch.bfloat16 and head_dim <= 256 and g.page_size >= 4 and not self.force_plain:
-            if step.max_rows_per_seq == 1:
+            if step.max_rows_per_seq == 1 and g.page_size >= 8:
                 return self._attention_decode(q, out, step, kc, vc, g, heads, kv_heads, head_dim, scale, window)
             self._call(self.lib.tli_attention_prefill_bf16, q.data_ptr(), out.data_ptr(), kc.data_ptr(),
                        vc.data_ptr(), step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs,
@@ -593,7 +593,7 @@ class HipOps:
             sums = qkv
             if not (step.max_rows_per_seq == 1 and qkv.dtype == torch.bfloat16 and cache is not None
                     and head_dim % 64 == 0 and head_dim <= 256 and heads // kv_heads <= 16
-                    and cache.group.page_size >= 4 and not self.force_plain and not self.unfused_decode
+                    and cache.group.page_size >= 8 and not self.force_plain and not self.unfused_decode
                     and (rotary is None or rotary[2] == head_dim)):
                 qkv, sums = self.resolve(qkv), None
         fusable = (qkv.dtype == torch.bfloat16 and cache is not None and head_dim % 64 == 0
@@ -604,7 +604,7 @@ class HipOps:
             return self._qkv_attention_prefill(qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm,
                                                rotary, scale, window)
         fused = (fusable and step.max_rows_per_seq == 1 and heads // kv_heads <= 16
-                 and cache.group.page_size >= 4)
+                 and cache.group.page_size >= 8)
         if not fused:
             q = self.qkv_to_cache(qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary)
             return self.paged_attention(q, step, cache, heads, kv_heads, head_dim, scale, window)
