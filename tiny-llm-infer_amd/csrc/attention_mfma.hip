@@ -576,7 +576,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
                         const int* __restrict__ tables, int table_width, int page_size, int page_shift,
                         int num_pages, int heads, int kv_heads, int head_dim, float scale, int window,
                         int splits, int keys_per_split, RawQkv raw) {
-    extern __shared__ float lds[];       // 3 waves x 64 lanes x (ND*4 + 2), then this split's table entries, FUSED: the prologue's sums of squares and slices of q
+    extern __shared__ float lds[];       // 4 waves x 64 lanes x (ND*4 + 2), then this split's table entries, FUSED: the prologue's sums of squares and slices of q
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, c = lane / 16;
     const int split = blockIdx.x, row = blockIdx.z;
     const int group = heads / kv_heads;
@@ -601,7 +601,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     const int end = min(pos + 1, begin + keys_per_split);
     // its part of the block table goes to LDS once, so that a block's addresses do not
     // wait for a table entry from memory first
-    int* seg = reinterpret_cast<int*>(lds + 3 * 64 * (ND * 4 + 2));
+    int* seg = reinterpret_cast<int*>(lds + 4 * 64 * (ND * 4 + 2));
     const int seg_first = begin >> page_shift;
     const int seg_len = begin < end ? ((end - 1) >> page_shift) - seg_first + 1 : 0;
     if (FUSED) {
@@ -740,10 +740,11 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
         tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 8 * c, 4, scale);
     }
 
-    // merge the four waves: waves 1..3 hand over (m, l, acc), wave 0 combines in wave order
+    // merge the four waves: each hands over (m, l, acc) through LDS and combines, in wave order,
+    // the dims 16 dt .. of the tiles dt = wave, wave + 4, .., which it then writes
     const int stride = ND * 4 + 2;
-    if (wave > 0) {
-        float* dst = lds + ((size_t)(wave - 1) * 64 + lane) * stride;
+    {
+        float* dst = lds + ((size_t)wave * 64 + lane) * stride;
         dst[0] = t.m;
         dst[1] = tile_sum(t);
 #pragma unroll
@@ -752,47 +753,50 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
             for (int i = 0; i < 4; ++i) dst[2 + dt * 4 + i] = t.acc[dt][i];
     }
     __syncthreads();
-    if (wave != 0) return;
-    float m = t.m;
-    for (int w = 0; w < 3; ++w) m = fmaxf(m, lds[((size_t)w * 64 + lane) * stride]);
-    const float base = (m == -INFINITY) ? 0.f : m;
-    float f = __builtin_amdgcn_exp2f(t.m - base);
-    float l = tile_sum(t) * f;
-#pragma unroll
-    for (int dt = 0; dt < ND; ++dt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) t.acc[dt][i] *= f;
-    for (int w = 0; w < 3; ++w) {
-        const float* src = lds + ((size_t)w * 64 + lane) * stride;
-        f = __builtin_amdgcn_exp2f(src[0] - base);
-        l += src[1] * f;
-#pragma unroll
-        for (int dt = 0; dt < ND; ++dt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) t.acc[dt][i] += src[2 + dt * 4 + i] * f;
-    }
     if (!live) return;
-    if (splits == 1) {
-        const float inv = l > 0.f ? 1.0f / l : 0.f;
-        bf16_t* o = out + ((size_t)row * heads + head) * head_dim;
+    float f[4];
+    float m = -INFINITY;
 #pragma unroll
-        for (int dt = 0; dt < ND; ++dt) {
+    for (int w = 0; w < 4; ++w) {
+        f[w] = lds[((size_t)w * 64 + lane) * stride];
+        m = w ? fmaxf(m, f[w]) : f[w];
+    }
+    const float base = (m == -INFINITY) ? 0.f : m;
+    float l = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        f[w] = __builtin_amdgcn_exp2f(f[w] - base);
+        const float lw = lds[((size_t)w * 64 + lane) * stride + 1] * f[w];
+        l = w ? l + lw : lw;
+    }
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    bf16_t* o = out + ((size_t)row * heads + head) * head_dim;
+    // partial[row][head][split][head_dim + 2]: unnormalised sum, then maximum (in units of log2)
+    // and sum of weights
+    float* pdst = splits == 1 ? nullptr : partial + (((size_t)row * heads + head) * splits + split) * (head_dim + 2);
+#pragma unroll
+    for (int dd = 0; dd < (ND + 3) / 4; ++dd) {
+        const int dt = dd * 4 + wave;
+        if (dt >= ND) break;
+        f32x4 a;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float* src = lds + ((size_t)w * 64 + lane) * stride + 2 + dt * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = w ? a[i] + src[i] * f[w] : src[i] * f[w];
+        }
+        if (splits == 1) {
             uint2 packed;
-            packed.x = (uint32_t)f32_to_bf16(t.acc[dt][0] * inv) | ((uint32_t)f32_to_bf16(t.acc[dt][1] * inv) << 16);
-            packed.y = (uint32_t)f32_to_bf16(t.acc[dt][2] * inv) | ((uint32_t)f32_to_bf16(t.acc[dt][3] * inv) << 16);
+            packed.x = (uint32_t)f32_to_bf16(a[0] * inv) | ((uint32_t)f32_to_bf16(a[1] * inv) << 16);
+            packed.y = (uint32_t)f32_to_bf16(a[2] * inv) | ((uint32_t)f32_to_bf16(a[3] * inv) << 16);
             *reinterpret_cast<uint2*>(o + dt * 16 + 4 * c) = packed;
+        } else {
+            *reinterpret_cast<f32x4*>(pdst + dt * 16 + 4 * c) = a;
         }
-    } else {
-        // partial[row][head][split][head_dim + 2]: unnormalised sum, then maximum (in units of log2)
-        // and sum of weights
-        float* dst = partial + (((size_t)row * heads + head) * splits + split) * (head_dim + 2);
-#pragma unroll
-        for (int dt = 0; dt < ND; ++dt)
-            *reinterpret_cast<f32x4*>(dst + dt * 16 + 4 * c) = t.acc[dt];
-        if (c == 0) {
-            dst[head_dim] = m;
-            dst[head_dim + 1] = l;
-        }
+    }
+    if (splits > 1 && wave == 0 && c == 0) {
+        pdst[head_dim] = m;
+        pdst[head_dim + 1] = l;
     }
 }
 
@@ -1566,11 +1570,26 @@ static int launch_decode(const void* q, void* out, float* partial, void* k_cache
 #define ARGS (const bf16_t*)q, (bf16_t*)out, partial, (bf16_t*)k_cache, (bf16_t*)v_cache, positions, seq_of_row, \
              tables, table_width, page_size, shift, num_pages, heads, kv_heads, head_dim, scale * LOG2E, window, \
              splits, keys_per_split
-#define LDS_BYTES(ND) (3 * 64 * (ND * 4 + 2) * sizeof(float) + seg_bytes + (raw ? 2 * 4 * 16 * sizeof(float) + (ND / 2) * 64 * sizeof(uint4) : 0))
+#define LDS_BYTES(ND) (4 * 64 * (ND * 4 + 2) * sizeof(float) + seg_bytes + (raw ? 2 * 4 * 16 * sizeof(float) + (ND / 2) * 64 * sizeof(uint4) : 0))
+    // (more than 64 KiB of LDS, which the widest heads need, has to be allowed for a kernel once)
+#define ONE(NJ, ND, F, R)                                                                                   \
+    {                                                                                                       \
+        auto kernel = attention_decode_kernel<NJ, ND, F>;                                                   \
+        const size_t bytes = LDS_BYTES(ND);                                                                 \
+        static bool allowed = false;                                                                        \
+        if (bytes > 65536 && !allowed) {                                                                    \
+            if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,        \
+                                    (int)bytes + 8192) != hipSuccess)                                       \
+                return tli_fail("attention_decode: cannot have %zu bytes of LDS", bytes);                   \
+            allowed = true;                                                                                 \
+        }                                                                                                   \
+        kernel<<<grid, 256, bytes, s>>>(ARGS, R);                                                           \
+    }
 #define CALL(NJ, ND)                                                                                        \
-    if (raw) attention_decode_kernel<NJ, ND, NJ * 2 == ND><<<grid, 256, LDS_BYTES(ND), s>>>(ARGS, *raw);   \
-    else attention_decode_kernel<NJ, ND, false><<<grid, 256, LDS_BYTES(ND), s>>>(ARGS, none)
+    if (raw) ONE(NJ, ND, NJ * 2 == ND, *raw)                                                                \
+    else ONE(NJ, ND, false, none)
     DISPATCH_HEAD_DIM(CALL)
+#undef ONE
 #undef CALL
 #undef LDS_BYTES
 #undef ARGS
