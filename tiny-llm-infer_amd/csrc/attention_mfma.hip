@@ -542,17 +542,32 @@ __device__ __forceinline__ void slice_fetch(float (&x)[8], const bf16_t* src, co
     }
 }
 
-// A slice after the norm (factor `scale`, weights nw8 or null) and the half-split rotation
-// (cos8, sin8 of the slice's dims, or null), as the score MFMAs take it.  The rotation partner
+// Eight floats at p (16-byte aligned), or zeros for a null p.
+__device__ __forceinline__ void load8(float (&v)[8], const float* p) {
+    if (p) {
+        const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[e] = a[e];
+            v[4 + e] = b[e];
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = 0.f;
+    }
+}
+
+// A slice after the norm (if normed: factor `scale`, weights nw8) and the half-split rotation
+// (if rotate: cos8, sin8 of the slice's dims), as the score MFMAs take it.  The rotation partner
 // of a lane is lane ^ 32 (head_dim == 32*NJ: the first half of the head lies in lane groups 0, 1).
-__device__ __forceinline__ uint4 slice_finish(float (&x)[8], const float* nw8, float scale, const float* cos8,
-                                              const float* sin8) {
+__device__ __forceinline__ uint4 slice_finish(float (&x)[8], bool normed, const float (&nw8)[8], float scale,
+                                              bool rotate, const float (&cos8)[8], const float (&sin8)[8]) {
     const int c = (threadIdx.x % 64) / 16;
-    if (nw8) {
+    if (normed) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) x[e] = nw8[e] * x[e] * scale;
     }
-    if (cos8) {
+    if (rotate) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const float partner = __shfl_xor(x[e], 32, 64);
@@ -618,11 +633,19 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
         const size_t q_off = (size_t)(live ? head : 0) * head_dim + c * 8 * NJ;
         const size_t k_off = (size_t)(heads + kv_head) * head_dim + c * 8 * NJ;
         float xq[SJ][8], xk[SJ][8];
+        // (the constants of a slice's norm and rotation are asked for with the slice, before the barrier)
+        float nq[SJ][8], nk[SJ][8], cs[SJ][8], sn[SJ][8];
+        const float* rot_at = raw.cos ? raw.cos + (size_t)pos * (head_dim / 2) + (c & 1) * 8 * NJ : nullptr;
+        const float* rot_sin = raw.cos ? raw.sin + (size_t)pos * (head_dim / 2) + (c & 1) * 8 * NJ : nullptr;
         float sq = 0.f, sk = 0.f;
 #pragma unroll
         for (int jj = 0; jj < SJ; ++jj) {
             const int j = jj * 4 + wave;
             if (j < NJ) {
+                load8(cs[jj], rot_at ? rot_at + j * 8 : nullptr);
+                load8(sn[jj], rot_sin ? rot_sin + j * 8 : nullptr);
+                load8(nq[jj], raw.q_norm_w ? raw.q_norm_w + c * 8 * NJ + j * 8 : nullptr);
+                load8(nk[jj], raw.k_norm_w ? raw.k_norm_w + c * 8 * NJ + j * 8 : nullptr);
                 slice_fetch(xq[jj], raw_row + q_off + j * 8, sums_row ? sums_row + q_off + j * 8 : nullptr, raw.parts,
                             raw.part_stride);
 #pragma unroll
@@ -648,11 +671,6 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
         const float k_ss = ssq[64 + r] + ssq[80 + r] + ssq[96 + r] + ssq[112 + r];
         const float q_scale = 1.0f / sqrtf(q_ss / (float)(32 * NJ) + raw.q_eps);
         const float k_scale = 1.0f / sqrtf(k_ss / (float)(32 * NJ) + raw.k_eps);
-        const float *cos_row = nullptr, *sin_row = nullptr;
-        if (raw.cos) {
-            cos_row = raw.cos + (size_t)pos * (head_dim / 2) + (c & 1) * 8 * NJ;
-            sin_row = raw.sin + (size_t)pos * (head_dim / 2) + (c & 1) * 8 * NJ;
-        }
         int own_page = -1;
         const int slot = pos & (page_size - 1);
         if (own) own_page = seg[(pos >> page_shift) - seg_first];
@@ -661,13 +679,11 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
         for (int jj = 0; jj < SJ; ++jj) {
             const int j = jj * 4 + wave;
             if (j < NJ) {
-                const float* cos8 = cos_row ? cos_row + j * 8 : nullptr;
-                const float* sin8 = sin_row ? sin_row + j * 8 : nullptr;
-                q_slices[j * 64 + lane] = slice_finish(xq[jj], raw.q_norm_w ? raw.q_norm_w + c * 8 * NJ + j * 8 : nullptr,
-                                                       q_scale, cos8, sin8);
+                q_slices[j * 64 + lane] = slice_finish(xq[jj], raw.q_norm_w != nullptr, nq[jj], q_scale,
+                                                       raw.cos != nullptr, cs[jj], sn[jj]);
                 if (own) {
-                    const uint4 kf = slice_finish(xk[jj], raw.k_norm_w ? raw.k_norm_w + c * 8 * NJ + j * 8 : nullptr,
-                                                  k_scale, cos8, sin8);
+                    const uint4 kf = slice_finish(xk[jj], raw.k_norm_w != nullptr, nk[jj], k_scale,
+                                                  raw.cos != nullptr, cs[jj], sn[jj]);
                     if (store && r == 0)
                         *reinterpret_cast<uint4*>(k_cache + (((size_t)own_page * kv_heads + kv_head) * page_size + slot) * head_dim +
                                                   c * 8 * NJ + j * 8) = kf;
