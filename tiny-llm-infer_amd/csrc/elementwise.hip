@@ -19,6 +19,22 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
     if (id < 0 || id >= vocab) id = 0;          // the host rejects such ids before the launch
     const T* src = table + (size_t)id * hidden;
     float* dst = out + (size_t)row * hidden;
+    if (sizeof(T) == 2 && hidden % 8 == 0 && !(((uintptr_t)table | (uintptr_t)out) & 15)) {
+        // eight elements a thread and turn: one 16-byte load, two 16-byte stores
+        for (int i = threadIdx.x * 8; i < hidden; i += blockDim.x * 8) {
+            const uint4 v = *reinterpret_cast<const uint4*>(src + i);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+            float f[8];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                f[2 * e] = __uint_as_float(w[e] << 16);
+                f[2 * e + 1] = __uint_as_float(w[e] & 0xFFFF0000u);
+            }
+            *reinterpret_cast<float4*>(dst + i) = make_float4(f[0], f[1], f[2], f[3]);
+            *reinterpret_cast<float4*>(dst + i + 4) = make_float4(f[4], f[5], f[6], f[7]);
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32(src[i]);
 }
 
