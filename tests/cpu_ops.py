@@ -84,8 +84,8 @@ class CpuOps:
             pages = tables[seq, pos // page].long()
             assert (pages >= 0).all(), "a row writes to a page that is not held"
             slots = pos % page
-            cache.k[pages, :, slots] = k.to(cache.k.dtype)
-            cache.v[pages, :, :, slots] = v.to(cache.v.dtype)        # values are kept transposed
+            cache.record("k")[pages, :, slots] = k.to(cache.record("k").dtype)
+            cache.record("v")[pages, :, :, slots] = v.to(cache.record("v").dtype)        # values are kept transposed
         return q.reshape(T, qd).to(qkv.dtype)
 
     def qkv_attention(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary, scale, window):
@@ -107,8 +107,8 @@ class CpuOps:
             idx = torch.arange(lo, p + 1)
             pages = tables[seq_l[r], idx // page].long()
             assert (pages >= 0).all(), "a row reads a page that is not held"
-            kk = cache.k[pages, :, idx % page].to(torch.float32)     # [n, kv, d]
-            vv = cache.v[pages, :, :, idx % page].to(torch.float32)
+            kk = cache.record("k")[pages, :, idx % page].to(torch.float32)     # [n, kv, d]
+            vv = cache.record("v")[pages, :, :, idx % page].to(torch.float32)
             for h in range(heads):
                 s = (kk[:, h // mul] @ qf[r, h]) * scale
                 w = torch.softmax(s, dim=0)

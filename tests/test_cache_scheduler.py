@@ -163,6 +163,57 @@ def test_random_orders_lose_no_page(seed):
     assert m.pages_taken_total == m.pages_returned_total > 80      # pages were used again
 
 
+def test_a_window_group_gets_no_more_pages_than_its_requests_can_hold():
+    """Given the most tokens a step brings, a window group's pool is the smaller one: for every
+    live request the window's blocks and two for the edges, and a step's tokens on top."""
+    from tiny_llm_infer_amd.cache.manager import group_needs, window_group_pages
+    assert window_group_pages(20, 8, 3, 64) == 3 * (3 + 2) + 8
+    m = CacheManager([FULL, WIN, FULL], page_size=8, num_pages=500, max_requests=3, max_step_tokens=64)
+    assert m.pages_per_group() == [500, 23] and m.num_pages == 500
+    assert CacheManager([FULL, WIN], 8, 10, 3, max_step_tokens=64).pages_per_group() == [10, 10]    # never more than asked
+    assert CacheManager([FULL, WIN], 8, 500, 3).pages_per_group() == [500, 500]                    # nothing known about steps
+    assert CacheManager([WIN, FULL], 8, [7, 9], 1).pages_per_group() == [7, 9]                     # one count a group
+    assert group_needs([WIN, None, FULL, WIN]) == [WIN, FULL]
+    with pytest.raises(ValueError, match="page counts"):
+        CacheManager([WIN, FULL], 8, [7], 1)
+    # what one request holds at most: everything where all keys are kept, window + portion where not
+    assert m.most_pages_needed(1000, 64) == [125, 3 + 2 + 8]
+    assert m.most_pages_needed(30, 64) == [4, 4]
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_the_smaller_window_pool_is_never_the_one_that_runs_out(seed):
+    """Random requests run in random portions, three live at a time, a step's portions within
+    its token budget: the window group's pool, sized as above, always has the pages."""
+    rng = random.Random(seed)
+    budget, live_max = 48, 3
+    m = CacheManager([FULL, WIN], page_size=4, num_pages=4000, max_requests=live_max, max_step_tokens=budget)
+    assert m.pages_per_group()[1] == live_max * (5 + 2) + 12
+    live, low = {}, m.pages_per_group()[1]
+    for it in range(400):
+        while len(live) < live_max:
+            key = f"q{it}-{len(live)}-{rng.random()}"
+            m.admit(key)
+            live[key] = [0, rng.randrange(1, 300)]
+        left = budget
+        for key in list(live):
+            at, size = live[key]
+            n = min(size - at, left, rng.choice([1, 1, 2, 5, 17, 48]))
+            if n <= 0:
+                continue
+            left -= n
+            m.reserve(key, at + n)                     # (raises CacheFull if the window pool were too small)
+            low = min(low, m.free_pages()[1])
+            live[key][0] = at + n
+        for key in list(live):
+            m.advance(key, live[key][0])
+            if live[key][0] == live[key][1]:
+                m.release(key)
+                del live[key]
+        m.check()
+    assert low < 12                                    # the pool was nearly used up, so the bound is no loose one
+
+
 # ----------------------------------------------------------------- scheduler --
 def _seq(i, n, max_tokens=4):
     return Sequence(i, list(range(n)), n, SamplingParams(max_tokens=max_tokens, ignore_eos=True))
@@ -351,3 +402,30 @@ def test_a_block_table_reads_like_a_list_and_is_one_piece_of_memory():
     t[0] = -1                      # a window has passed the page
     t.append(11)                   # no view is held any more: the table grows
     assert t == [-1, 3, 9, 11]
+
+
+def test_layers_with_a_window_take_their_pages_portion_by_portion():
+    """An admitted request holds all the pages of its prompt where all keys are kept, and in a
+    window group only what the next portion needs: a long prompt passes through a window pool
+    that could never hold it whole."""
+    cache = CacheManager([FULL, WIN], page_size=8, num_pages=200, max_requests=2, max_step_tokens=32)
+    assert cache.pages_per_group() == [200, 2 * 5 + 4]
+    s = Scheduler(SchedulerConfig(max_num_seqs=2, max_num_batched_tokens=32), cache)
+    a, b = _seq(1, 400, max_tokens=3), _seq(2, 90, max_tokens=3)
+    s.add(a)
+    s.add(b)
+    steps = 0
+    while not s.is_finished():
+        p = s.schedule()
+        assert p.items and p.num_tokens <= 32
+        held = [n - f for n, f in zip(cache.pages_per_group(), cache.free_pages())]
+        assert held[1] <= 14
+        _run(s, p)
+        cache.check()
+        steps += 1
+    assert a.completion_size == 3 and b.completion_size == 3 and s.num_preemptions == 0
+    assert cache.free_pages() == [200, 14]
+    # a request too long for the pool of the layers that keep all keys is still an error
+    s.add(_seq(3, 8 * 200 + 1))
+    with pytest.raises(SchedulerError, match="more than all"):
+        s.schedule()

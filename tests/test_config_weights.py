@@ -172,6 +172,62 @@ def test_sharded_checkpoint_and_broken_files(tmp_path):
         Checkpoint(str(empty))
 
 
+def test_files_of_the_safetensors_package_are_read_and_ours_are_read_by_it(tmp_path):
+    """A file that the ``safetensors`` package wrote (its own header padding, a ``__metadata__``
+    entry, its order of tensors, tensors in bfloat16, float16 and float32, sharded with an
+    index) is read tensor for tensor, and a file that this repository wrote opens in the
+    package with the same contents."""
+    st = pytest.importorskip("safetensors.torch")
+    from safetensors import safe_open
+    g = torch.Generator().manual_seed(3)
+    tensors = {"z.last": torch.randn(5, 7, generator=g).bfloat16(),
+               "a.first": torch.randn(3, generator=g).half(),
+               "m.mid": torch.randn(2, 3, 4, generator=g),
+               "i.table": torch.arange(6, dtype=torch.int64).reshape(2, 3),
+               "s.scalarish": torch.randn(1, generator=g).bfloat16()}
+    st.save_file(tensors, str(tmp_path / "model.safetensors"), metadata={"format": "pt", "note": "written by the package"})
+    ck = Checkpoint(str(tmp_path))
+    assert sorted(ck.names()) == sorted(tensors)
+    for name, t in tensors.items():
+        assert ck.dtype(name) == t.dtype and tuple(ck.shape(name)) == tuple(t.shape)
+        assert torch.equal(ck.read(name), t)
+    ck.close()
+    decls = [TensorDecl("z.last", (5, 7)), TensorDecl("a.first", (3,)), TensorDecl("m.mid", (2, 3, 4)),
+             TensorDecl("i.table", (2, 3), "int"), TensorDecl("s.scalarish", (1,))]
+    got = dict(load_tensors(str(tmp_path), decls, torch.bfloat16, "cpu"))
+    assert [got[d.name].dtype for d in decls] == [torch.bfloat16, torch.bfloat16, torch.float32, torch.int32, torch.bfloat16]
+    assert torch.equal(got["a.first"], tensors["a.first"].to(torch.bfloat16)) and torch.equal(got["m.mid"], tensors["m.mid"])
+    # sharded by the package's writer, with an index that also carries metadata
+    shards = tmp_path / "sharded"
+    shards.mkdir()
+    names = list(tensors)
+    st.save_file({n: tensors[n] for n in names[:2]}, str(shards / "model-00001-of-00002.safetensors"), metadata={"format": "pt"})
+    st.save_file({n: tensors[n] for n in names[2:]}, str(shards / "model-00002-of-00002.safetensors"))
+    (shards / "model.safetensors.index.json").write_text(json.dumps({
+        "metadata": {"total_size": 1},
+        "weight_map": {n: f"model-0000{1 if i < 2 else 2}-of-00002.safetensors" for i, n in enumerate(names)}}))
+    ck = Checkpoint(str(shards))
+    assert all(torch.equal(ck.read(n), t) for n, t in tensors.items())
+    ck.close()
+    # and the other way round
+    ours = str(tmp_path / "ours.safetensors")
+    write_safetensors(ours, list(tensors.items()))
+    with safe_open(ours, framework="pt") as fh:
+        assert sorted(fh.keys()) == sorted(tensors)
+        for name, t in tensors.items():
+            assert torch.equal(fh.get_tensor(name), t)
+    assert all(torch.equal(v, tensors[k]) for k, v in st.load_file(ours).items())
+
+
+def test_a_model_folder_written_here_loads_in_the_package(model_folders):
+    st = pytest.importorskip("safetensors.torch")
+    folder = model_folders["C"]
+    theirs = st.load_file(os.path.join(folder, "model.safetensors"))
+    ck = Checkpoint(folder)
+    assert sorted(theirs) == sorted(ck.names())
+    assert all(torch.equal(theirs[n], ck.read(n)) for n in ck.names())
+
+
 def test_run_order_is_checked():
     from dataclasses import replace
     from tiny_llm_infer_amd.config import LayerCall

@@ -105,6 +105,26 @@ def test_linear(ops, dtype, mnk):
           scale=float(want.abs().max()) * (1.0 if dtype == torch.float32 else 0.05))
 
 
+@pytest.mark.parametrize("mnk", [(300, 5120, 17408), (300, 5120, 25600), (64, 51200, 5120)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_plain_product_at_the_widths_it_is_the_reference_for(ops, dtype, mnk):
+    """The plain kernel is what the tuned products are compared with at the widths of the
+    larger models; here it is itself compared with float64 at those widths (the sum over
+    17,408 and 25,600 terms, 51,200 outputs)."""
+    M, N, K = mnk
+    g = torch.Generator(device=DEV).manual_seed(K)
+    x = torch.randn((M, K), generator=g, device=DEV).to(dtype)
+    w = (torch.randn((N, K), generator=g, device=DEV) * 0.02).to(dtype)
+    want = x.double() @ w.double().t()
+    got = ops.linear_plain(x, w, out_dtype=torch.float32)
+    # A float32 sum of K terms in a fixed order is off by about sqrt(K) roundings of 2^-24 of the
+    # sum's own size (the largest of 1.5 million outputs by five times the typical one); one term
+    # left out or taken twice would be off by 1/sqrt(K) of it, a hundred times more.
+    err = float((got.double() - want).abs().max())
+    allowed = 1e-7 * math.sqrt(K) * float(want.abs().max())
+    assert err <= allowed, f"error {err} against {float(want.abs().max())}, allowed {allowed}"
+
+
 SKINNY = [(1, 4096, 4096), (8, 6144, 4096), (8, 4096, 12288), (16, 301, 80), (17, 1000, 264),
           (33, 24576, 512), (64, 130, 4096), (5, 151936, 128), (48, 70, 8),
           (65, 1000, 264), (100, 4096, 4096), (128, 130, 1032), (96, 6144, 512), (40, 96, 64), (70, 40, 200)]
@@ -316,8 +336,14 @@ def test_linear_rows_do_not_depend_on_the_batch(ops):
 
 
 # ------------------------------------------------------ cache and attention --
-class FakeStep:
-    pass
+def kv_layer_cache(group, layer=0, writes=True):
+    """The cache of one layer call with the attention part's two records at hand as .k and .v."""
+    from tiny_llm_infer_amd.parts.base import LayerCache
+
+    class KeysAndValues(LayerCache):
+        k = property(lambda self: self.record("k"))       # [pages, kv heads, page_size, head_dim]
+        v = property(lambda self: self.record("v"))       # [pages, kv heads, head_dim, page_size]
+    return KeysAndValues(group, layer, writes)
 
 
 def make_step(seq_lens, new_counts, page, num_pages, seed, kv_heads, head_dim, dtype, window=None):
@@ -357,7 +383,7 @@ def make_step(seq_lens, new_counts, page, num_pages, seed, kv_heads, head_dim, d
                     h_seq_len=list(seq_lens), h_slots=list(range(len(seq_lens))),
                     max_rows_per_seq=max(new_counts), max_seq_len=max(seq_lens),
                     reach=max(128, 1 << (max(seq_lens) - 1).bit_length()), groups=[g])
-    step.cache = LayerCache(g, 0, True)
+    step.cache = kv_layer_cache(g)
     return step, tables, pos, seq
 
 

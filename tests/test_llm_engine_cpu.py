@@ -56,6 +56,30 @@ def test_admission_checks(model_folders):
     eng.add_request([1] * 30, SamplingParams(max_tokens=3))     # exactly fits: 30 + 3 - 1 = 32
 
 
+def test_a_request_that_the_cache_can_never_hold_is_refused_when_it_is_added(model_folders):
+    """4 pages of 8 tokens: a prompt of 27 tokens with 14 new ones would reach 40 tokens in the
+    cache, be preempted for ever and take every other request down with it.  It is refused at
+    once; what was added before it finishes as if nothing had happened."""
+    folder = model_folders["A"]
+    cfg, w = plain_qwen3.read_model(folder)
+    eng = _engine(folder, "A", num_kv_blocks=4)
+    first = random_prompt(256, 6, 3)
+    eng.add_request(first, SamplingParams(max_tokens=14, ignore_eos=True))
+    with pytest.raises(ValueError, match="need 5 cache pages of 8 tokens, the cache has 4"):
+        eng.add_request(random_prompt(256, 27, 4), SamplingParams(max_tokens=14, ignore_eos=True))
+    eng.add_request(random_prompt(256, 27, 4), SamplingParams(max_tokens=6, ignore_eos=True))      # 32 tokens: fits
+    done = []
+    while not eng.is_finished():
+        done += eng.step()
+    assert sorted(len(r.token_ids) for r in done) == [6, 14]
+    assert [r.token_ids for r in done if len(r.token_ids) == 14] == [plain_qwen3.greedy(cfg, w, first, 14)]
+    eng.runner.cache.check()
+    assert eng.runner.cache.free_pages() == [4]
+    with pytest.raises(ValueError, match="cache pages"):
+        eng.generate([first, random_prompt(256, 27, 4)], SamplingParams(max_tokens=14))            # checked before any is added
+    assert eng.is_finished()
+
+
 def test_eos_stops_a_request(model_folders):
     folder = model_folders["A"]
     cfg, w = plain_qwen3.read_model(folder)
@@ -132,7 +156,7 @@ def test_steps_put_on_the_device_ahead_change_nothing(model_folders):
         outs.append(eng.generate(prompts, params))
         assert (eng.num_steps_ahead > 5) == ahead
         eng.runner.cache.check()
-        assert eng.runner.cache.free_pages() == [64, 64] and eng.is_finished()
+        assert eng.runner.cache.free_pages() == [64, 24] and eng.is_finished()     # (the window group's pool is the smaller one)
     assert [r.token_ids for r in outs[0]] == [r.token_ids for r in outs[1]]
     assert len(outs[1][0].token_ids) <= 5 and len(outs[1][2].token_ids) <= 3
 
@@ -173,3 +197,21 @@ def test_step_ahead_counts_the_pages_of_the_whole_batch(model_folders):
         eng.runner.cache.check()
         assert eng.runner.cache.free_pages() == [5] and eng.is_finished()
     assert outs[0] == outs[1] == want
+
+
+def test_a_window_group_has_the_smaller_pool(model_folders):
+    """Configuration B with room for 4 requests of 640 tokens: the windowed layers (window 40,
+    pages of 16) get 4 * (3 + 2) + 2 pages, not 160, and long prompts pass through them
+    portion by portion; the tokens are the plain greedy ones and nothing is preempted."""
+    folder = model_folders["B"]
+    eng = _engine(folder, "B", num_kv_blocks=160, max_model_len=640)
+    cache = eng.runner.cache
+    assert cache.pages_per_group() == [160, 22]
+    assert [t["k"].shape[:2] for t in eng.runner.group_tensors] == [(1, 161), (2, 23)]
+    prompts = [random_prompt(384, n, 11 * n) for n in (150, 3, 77, 240)]
+    got = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
+    cfg, w = plain_qwen3.read_model(folder)
+    assert [r.token_ids for r in got] == [plain_qwen3.greedy(cfg, w, p, 12) for p in prompts]
+    assert eng.scheduler.num_preemptions == 0
+    cache.check()
+    assert cache.free_pages() == [160, 22]

@@ -415,4 +415,4 @@ def test_a_request_of_9000_tokens_through_the_engine(long_request, dtype):
         print(f"9000 tokens, {dtype}, {cut}: worst error {err / scale:.2e} of the largest logit, at token {row}")
         assert err <= tol * scale, f"{dtype}/{cut}: error {err:.3e} at token {row} (logit scale {scale:.3e})"
         runner.cache.check()
-        assert all(f == runner.cache.num_pages for f in runner.cache.free_pages())
+        assert runner.cache.free_pages() == runner.cache.pages_per_group()

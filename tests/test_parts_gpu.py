@@ -47,8 +47,8 @@ def test_rope_part_tables(envs, dtype):
     part = build_part("position", PartSpec("rope_neox", {"head_dim": 48, "theta": 50000.0,
                                                           "max_positions": 200}))
     part.load({}, envs[dtype])
-    cos, sin, rd = part.rotary()
-    assert rd == 48 and cos.shape == (200, 24)
+    cos, sin, rd, pairing = part.rotary()
+    assert rd == 48 and cos.shape == (200, 24) and pairing == "half"
     ang = P.rope_angles(48, 50000.0, list(range(200)))
     assert torch.allclose(cos.cpu().double(), torch.cos(torch.from_numpy(ang).double()), atol=1e-7)
     assert torch.allclose(sin.cpu().double(), torch.sin(torch.from_numpy(ang).double()), atol=1e-7)
@@ -133,6 +133,114 @@ def test_attention_part_whole_sequence(envs, dtype, window):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hd,rd", [(32, 32), (64, 64), (64, 24), (128, 128)])
+def test_attention_part_with_a_rotation_of_neighbours(envs, dtype, hd, rd):
+    """A position encoding defined here that turns the pairs (2i, 2i + 1), over the whole head
+    or the first ``rd`` elements: a whole sequence and then single tokens through the stock
+    attention part (heads of 64 and 128: the kernels that take the raw projections) against
+    float64 mathematics written out here."""
+    from tiny_llm_infer_amd.config import PartSpec
+    from tiny_llm_infer_amd.parts import PositionEncoding, build_part, register_part
+    from tiny_llm_infer_amd.parts.base import RotaryTables
+    heads, kv, hidden, T, more, theta = 4, 2, 80, 37, 5, 300.0
+    half = rd // 2
+    angles = torch.arange(256, dtype=torch.float64)[:, None] * theta ** (-2.0 * torch.arange(half, dtype=torch.float64) / rd)[None, :]
+
+    class Neighbours(PositionEncoding):
+        def load(self, weights, env):
+            super().load(weights, env)
+            self.cos, self.sin = torch.cos(angles).float().to(env.device), torch.sin(angles).float().to(env.device)
+
+        def rotary(self):
+            return RotaryTables(self.cos, self.sin, rd, "interleaved")
+
+    register_part("position", "toy_neighbours", Neighbours, replace=True)
+    base = _attention_spec(heads, kv, hd, hidden, None)
+    spec = PartSpec(base.kind, base.params, base.names, dict(base.parts, position=PartSpec("toy_neighbours")))
+    part = build_part("mixer", spec)
+    w = _weights(part.tensors(), dtype, seed=14)
+    part.load(w, envs[dtype])
+    total = T + more
+    step, tables, pos, seq = make_step([T], [T], 8, 8, 0, kv, hd, dtype)
+    x = rnd((total, hidden), dtype, 15)
+    ops = envs[dtype].ops
+    outs = [ops.resolve(part.forward(x[:T].to(DEV), step))]
+    for t in range(T, total):                      # the same pages, one token more at a time
+        step2, tables2, _, _ = make_step([t + 1], [1], 8, 8, 0, kv, hd, dtype)
+        step2.cache.group.tensors["k"].copy_(step.cache.group.tensors["k"])
+        step2.cache.group.tensors["v"].copy_(step.cache.group.tensors["v"])
+        assert (tables2[0, :(t + 7) // 8] == tables[0, :(t + 7) // 8]).all()       # (the same pages in the same order)
+        outs.append(ops.resolve(part.forward(x[t:t + 1].to(DEV), step2)))
+        step = step2
+        tables = tables2
+    got = torch.cat(outs)
+    # float64
+    f = {k: v.cpu().double() for k, v in w.items()}
+    xd = x.double()
+    q = (xd @ f["q"].t()).reshape(total, heads, hd)
+    k = (xd @ f["k"].t()).reshape(total, kv, hd)
+    v = (xd @ f["v"].t()).reshape(total, kv, hd)
+    q, k = P.rmsnorm(q, f["qn"], 1e-6), P.rmsnorm(k, f["kn"], 1e-6)
+    c, s_ = torch.cos(angles[:total])[:, None, :], torch.sin(angles[:total])[:, None, :]
+
+    def turn(t):
+        out = t.clone()
+        a, b = t[..., 0:rd:2], t[..., 1:rd:2]
+        out[..., 0:rd:2] = a * c - b * s_
+        out[..., 1:rd:2] = a * s_ + b * c
+        return out
+    o = P.causal_attention(turn(q), turn(k), v, hd ** -0.5)
+    want = o.reshape(total, heads * hd) @ f["o"].t()
+    close(got, want, dtype, f"attention with neighbours paired, head {hd}, rotary {rd}")
+
+
+def test_attention_part_refuses_what_its_kernels_do_not_do(envs):
+    """An inner norm of another kind than the RMS norm, and a pairing of rotated elements that
+    is not known, are refused when the part takes its weights, with a message; they are never
+    computed as something else."""
+    from tiny_llm_infer_amd.config import PartSpec
+    from tiny_llm_infer_amd.parts import Norm, PositionEncoding, build_part, register_part
+    from tiny_llm_infer_amd.parts.base import RotaryTables
+    from tiny_llm_infer_amd.weights import TensorDecl
+
+    class MeanFree(Norm):
+        def tensors(self):
+            return [TensorDecl(self.spec.names["weight"], (self.spec.params["size"],), "ones_normal")]
+
+        def load(self, weights, env):
+            super().load(weights, env)
+            self.weight, self.eps = weights[self.spec.names["weight"]].float(), 1e-6     # (what an RMS norm holds too)
+
+        def forward(self, resid, delta, rows=None, num_rows=None):
+            raise AssertionError("not run here")
+
+    class Crossed(PositionEncoding):
+        def rotary(self):
+            z = torch.zeros(256, 16, device=DEV)
+            return RotaryTables(z, z, 32, "crossed")
+
+    register_part("norm", "toy_mean_free", MeanFree, replace=True)
+    register_part("position", "toy_crossed", Crossed, replace=True)
+    base = _attention_spec(4, 2, 32, 80, None)
+    env = envs[torch.bfloat16]
+    bad_norm = PartSpec(base.kind, base.params, base.names,
+                        dict(base.parts, k_norm=PartSpec("toy_mean_free", {"size": 32}, {"weight": "kn"})))
+    part = build_part("mixer", bad_norm)
+    with pytest.raises(ValueError, match="k norm of an attention layer is 'toy_mean_free'"):
+        part.load(_weights(part.tensors(), torch.bfloat16), env)
+    part = build_part("mixer", PartSpec(base.kind, base.params, base.names, dict(base.parts, position=PartSpec("toy_crossed"))))
+    with pytest.raises(ValueError, match="pairing 'crossed' is not known"):
+        part.load(_weights(part.tensors(), torch.bfloat16), env)
+    # and the kernel library itself turns halves only
+    from tiny_llm_infer_amd.kernels.ops import KernelError
+    step, *_ = make_step([5], [5], 8, 2, 0, 2, 32, torch.bfloat16)
+    z = torch.zeros(256, 16, device=DEV)
+    with pytest.raises(KernelError, match="not the pairing 'interleaved'"):
+        env.ops.qkv_attention(rnd((5, 8 * 32), torch.bfloat16, 1).to(DEV), step, step.cache, 4, 2, 32, None, None,
+                              (z, z, 32, "interleaved"), 1.0, None)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_prenorm_block(envs, dtype):
     from tiny_llm_infer_amd.config import PartSpec
     from tiny_llm_infer_amd.parts import build_part
@@ -167,7 +275,8 @@ def test_toy_mixer_with_state_of_its_own(tmp_path):
     """A mixer defined here, keeping a running sum per request in a state slot:
     y_t = W . mean(x_0..x_t).  It is registered, built into a model of a toy
     architecture and stepped in several cuts through the framework's runner,
-    cache manager and replay, none of which is changed for it."""
+    cache manager and replay, none of which is changed for it.  The last block of the toy
+    has no feed-forward: norm, mixer, sum."""
     import json
 
     import numpy as np
@@ -228,7 +337,10 @@ def test_toy_mixer_with_state_of_its_own(tmp_path):
             "prenorm", PartSpec("running_mean", {"size": c.size}, {"w": f"l{i}.mix"}),
             PartSpec("swiglu", {"hidden_size": c.size, "intermediate_size": c.inter},
                      {"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}),
-            {"mixer": rms(f"l{i}.n1"), "ffn": rms(f"l{i}.n2")}) for i in range(c.layers))
+            {"mixer": rms(f"l{i}.n1"), "ffn": rms(f"l{i}.n2")}) for i in range(c.layers - 1))
+        last = c.layers - 1
+        blocks += (BlockSpec("prenorm", PartSpec("running_mean", {"size": c.size}, {"w": f"l{last}.mix"}), None,
+                             {"mixer": rms(f"l{last}.n1")}),)
         return ModelSpec("ToyStateLM", c.size, c.vocab, 4096,
                          PartSpec("token_embedding", {"vocab_size": c.vocab, "hidden_size": c.size}, {"weight": "emb"}),
                          blocks, tuple(LayerCall(i) for i in range(c.layers)), rms("norm"),
@@ -236,7 +348,7 @@ def test_toy_mixer_with_state_of_its_own(tmp_path):
                                   {"weight": "emb"}))
 
     register_architecture("ToyStateLM", lambda d, origin: ToyConfig(d), toy_spec, replace=True)
-    cfg = {"architectures": ["ToyStateLM"], "size": 40, "inter": 56, "layers": 2, "vocab": 97}
+    cfg = {"architectures": ["ToyStateLM"], "size": 40, "inter": 56, "layers": 3, "vocab": 97}
     folder = write_random_model(str(tmp_path / "toy"), "ToyStateLM", ToyConfig(cfg), seed=3)
 
     # the plain version of the toy, whole sequences
@@ -244,10 +356,13 @@ def test_toy_mixer_with_state_of_its_own(tmp_path):
 
     def plain(ids):
         h = w["emb"][torch.tensor(ids)]
-        for i in range(2):
+        for i in range(3):
             n = P.rmsnorm(h, w[f"l{i}.n1"], 1e-6)
             mean = torch.cumsum(n, 0) / torch.arange(1, len(ids) + 1, dtype=torch.float64)[:, None]
             r = h + mean @ w[f"l{i}.mix"].t()
+            if i == 2:
+                h = r                  # the block without a feed-forward
+                break
             m = P.rmsnorm(r, w[f"l{i}.n2"], 1e-6)
             h = r + P.linear(P.swiglu(P.linear(m, w[f"l{i}.g"]), P.linear(m, w[f"l{i}.u"])), w[f"l{i}.d"])
         return P.linear(P.rmsnorm(h, w["norm"], 1e-6), w["emb"]).numpy()

@@ -75,7 +75,7 @@ def test_cuts_match_plain(model_folders, oracle, name, dtype, cut):
     worst = _check(got, want, dtype, f"{name}/{dtype}/{cut}")
     print(f"{name} {dtype} {cut}: worst relative error {worst:.2e}")
     runner.cache.check()
-    assert all(f == runner.cache.num_pages for f in runner.cache.free_pages())
+    assert runner.cache.free_pages() == runner.cache.pages_per_group()
     if cut == "mixed":
         assert runner.cache.pages_taken_total > runner.cache.num_pages
 
@@ -196,6 +196,31 @@ def test_real_layer_sizes(tmp_path, sizes):
     runner = ModelRunner(model, model.env, page_size=16, num_pages=24, max_requests=4, max_batch_tokens=512)
     worst = _check(collect(steps, _replay(runner, steps)), want, "bfloat16", f"{sizes['hidden_size']} wide/library products")
     print(f"{sizes['hidden_size']} wide, library products of many rows: worst relative error {worst:.2e}")
+
+
+def test_three_layers_at_the_width_of_qwen3_8b(tmp_path):
+    """Three layers of the Qwen3-8B sizes against the plain implementation, requests mixed so
+    that pages are used again: which layer of the cache a page's keys belong to, at the true
+    strides of the pool (8 kv heads of 128, pages of 16), in float32 and in bfloat16."""
+    from tiny_llm_infer_amd.config import Qwen3Config
+    from tiny_llm_infer_amd.engine.loading import load_model, write_random_model
+    from tiny_llm_infer_amd.engine.runner import ModelRunner
+    cfg = Qwen3Config.from_dict(dict(
+        architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=3, head_dim=128, vocab_size=1024,
+        max_position_embeddings=4096, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False,
+        hidden_size=4096, intermediate_size=12288, num_attention_heads=32, num_key_value_heads=8))
+    folder = write_random_model(str(tmp_path / "three"), "Qwen3ForCausalLM", cfg, seed=8)
+    reqs = {f"r{i}": random_prompt(1024, n, 500 + i) for i, n in enumerate([120, 61, 40, 97])}
+    want = plain_logits(folder, reqs)
+    steps = trace_mixed(reqs, max_tokens=256, seed=4)
+    for dtype in ("float32", "bfloat16"):
+        model, _ = load_model(folder, dtype, "cuda:0")
+        runner = ModelRunner(model, model.env, page_size=16, num_pages=16, max_requests=4, max_batch_tokens=512)
+        got = collect(steps, _replay(runner, steps))
+        worst = _check(got, want, dtype, f"three layers/{dtype}")
+        print(f"three layers at 4096 wide, {dtype}, mixed: worst relative error {worst:.2e}")
+        runner.cache.check()
+        assert runner.cache.pages_taken_total > runner.cache.num_pages
 
 
 @pytest.mark.parametrize("name", ["B", "D"])

@@ -7,8 +7,10 @@ tensor for keys and one for values, and one block table per request, so layers
 that keep all keys and layers that keep a window of them do not share pages.
 A window group gives a page back as soon as every slot of it lies before the
 window of all tokens still to come; every group gives all of a request's pages
-back when the request ends.  (The reference has one group and no window:
-model/src/qwen3_kv_cache.cpp:14-44, engine/src/block_manager.cpp.)
+back when the request ends.  A group has as many pages as it can use: one that
+keeps all keys the number asked for, a window group no more than its requests
+can ever hold together (``window_group_pages``).  (The reference has one group
+and no window: model/src/qwen3_kv_cache.cpp:14-44, engine/src/block_manager.cpp.)
 
 Prefix caching (off unless asked for; the reference's block manager does the same,
 engine/src/block_manager.cpp:24-64, 184-224): every full page gets a hash chained
@@ -163,15 +165,47 @@ def page_hash(tokens: Sequence[int], prefix_hash: int) -> int:
     return h
 
 
+def window_group_pages(window: int, page_size: int, max_requests: int, max_step_tokens: int) -> int:
+    """The most pages that the live requests of a window group can hold together.  A request that
+    has s tokens in the cache and runs c more holds the blocks from the first one a query at s
+    reads to the one its last token is written to: at most (window - 1 + c) / page + 2, the
+    window and the portion each straddling a page's edge.  Over ``max_requests`` requests whose
+    portions of one step add up to ``max_step_tokens``."""
+    blocks = lambda n: (n + page_size - 1) // page_size
+    return max_requests * (blocks(window - 1) + 2) + blocks(max_step_tokens)
+
+
+def group_needs(needs: Sequence[Optional["CacheNeed"]]) -> List["CacheNeed"]:
+    """The distinct needs among ``needs`` in the order the groups are made."""
+    out: List[CacheNeed] = []
+    for need in needs:
+        if need is not None and need not in out:
+            out.append(need)
+    return out
+
+
 class CacheManager:
-    def __init__(self, needs: Sequence[Optional[CacheNeed]], page_size: int, num_pages: int,
-                 max_requests: int, prefix_caching: bool = False):
+    def __init__(self, needs: Sequence[Optional[CacheNeed]], page_size: int, num_pages,
+                 max_requests: int, prefix_caching: bool = False, max_step_tokens: Optional[int] = None):
         """``needs[i]`` is the need of cache layer i (None: that layer keeps nothing).
-        Every group gets ``num_pages`` pages of ``page_size`` slots."""
-        if page_size <= 0 or num_pages <= 0 or max_requests <= 0:
+        ``num_pages``: the pages (of ``page_size`` slots) of a group that keeps all keys, or a
+        list with one count for every group (``group_needs`` gives their order).  Given one
+        number and ``max_step_tokens`` (the most tokens that the requests of one step bring
+        together), a window group gets no more pages than ``window_group_pages`` says it can
+        use; without it every group gets ``num_pages``."""
+        per_group = None if isinstance(num_pages, int) else [int(n) for n in num_pages]
+        if page_size <= 0 or max_requests <= 0 or (per_group is None and num_pages <= 0) \
+                or (per_group is not None and any(n <= 0 for n in per_group)):
             raise ValueError("page_size, num_pages and max_requests must be positive")
+        distinct = group_needs(needs)
+        if per_group is None:
+            per_group = [num_pages if (n.window is None or max_step_tokens is None) else
+                         min(num_pages, window_group_pages(n.window, page_size, max_requests, max_step_tokens))
+                         for n in distinct]
+        if len(per_group) != len(distinct):
+            raise ValueError(f"{len(per_group)} page counts for {len(distinct)} groups of cache layers")
         self.page_size = page_size
-        self.num_pages = num_pages
+        self.num_pages = max(per_group, default=0)         # of the largest group
         self.max_requests = max_requests
         self.groups: List[GroupLayout] = []
         self.group_of_layer: Dict[int, int] = {}
@@ -181,7 +215,7 @@ class CacheManager:
                 continue
             g = by_need.get(need)
             if g is None:
-                g = GroupLayout(need, [], PagePool(num_pages), index=len(self.groups))
+                g = GroupLayout(need, [], PagePool(per_group[len(self.groups)]), index=len(self.groups))
                 by_need[need] = g
                 self.groups.append(g)
             g.cache_layers.append(layer)
@@ -328,6 +362,48 @@ class CacheManager:
     def can_reserve(self, key: Hashable, new_total: int) -> bool:
         return all(n <= g.pool.free_count
                    for n, g in zip(self.pages_needed(key, new_total), self.groups))
+
+    def most_pages_needed(self, total_tokens: int, portion: int) -> List[int]:
+        """Per group, the most pages one request of ``total_tokens`` tokens ever holds when it is
+        run in portions of at most ``portion`` tokens: all its blocks where all keys are kept, the
+        window's and a portion's where a window passes."""
+        whole = _blocks(total_tokens, self.page_size)
+        out = []
+        for g in self.groups:
+            if g.need.window is None:
+                out.append(whole)
+            else:
+                out.append(min(whole, _blocks(g.need.window - 1, self.page_size) + 2
+                               + _blocks(min(portion, total_tokens), self.page_size)))
+        return out
+
+    def pages_per_group(self) -> List[int]:
+        return [g.pool.num_pages for g in self.groups]
+
+    def _ahead_needed(self, rc: RequestCache, total: int) -> List[int]:
+        nb = _blocks(total, self.page_size)
+        return [max(0, nb - len(rc.tables[gi])) if g.need.window is None else 0
+                for gi, g in enumerate(self.groups)]
+
+    def can_hold_ahead(self, key: Hashable, total: int) -> bool:
+        return all(n <= g.pool.free_count
+                   for n, g in zip(self._ahead_needed(self._live[key], total), self.groups))
+
+    def hold_ahead(self, key: Hashable, total: int) -> None:
+        """Take now, in the groups that keep all keys, the pages for ``total`` tokens of the
+        request, so that once it is admitted no other request can take them from under it (the
+        reference allocates a whole prompt at admission, engine/src/block_manager.cpp:87-119).
+        Window groups take theirs portion by portion (``reserve``), since they give them back
+        the same way.  All or nothing."""
+        rc = self._live[key]
+        if not self.can_hold_ahead(key, total):
+            raise CacheFull(f"not enough free pages to hold {total} tokens of {key!r}")
+        nb = _blocks(total, self.page_size)
+        for gi, g in enumerate(self.groups):
+            if g.need.window is None:
+                table = rc.tables[gi]
+                while len(table) < nb:
+                    table.append(self._take(gi))
 
     def reserve(self, key: Hashable, new_total: int) -> None:
         """Take pages so that positions up to ``new_total`` can be written and

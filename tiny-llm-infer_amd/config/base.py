@@ -35,10 +35,11 @@ class PartSpec:
 @dataclass(frozen=True)
 class BlockSpec:
     """A residual block: which arrangement of norm/mixer/feed-forward it uses
-    and the parts themselves."""
+    and the parts themselves.  ``ffn`` None: a block of a mixer alone (its arrangement has
+    to know what to do without one; "prenorm" then is norm, mixer, sum)."""
     arrangement: str
     mixer: PartSpec
-    ffn: PartSpec
+    ffn: Optional[PartSpec]
     norms: Dict[str, PartSpec]
 
 

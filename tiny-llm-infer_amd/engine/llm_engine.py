@@ -105,6 +105,15 @@ class LLMEngine:
             raise ValueError(f"the prompt has {len(prompt)} tokens, this engine holds at most {self.max_model_len} a request (max_model_len)")
         if sampling.max_tokens > self.max_model_len - len(prompt) + 1:
             raise ValueError(f"{len(prompt)} prompt tokens and {sampling.max_tokens} new ones do not fit max_model_len = {self.max_model_len}")
+        # what the request holds at its longest (its last token is never run) must fit the pools
+        # even when it is the only one: else it would be preempted for ever
+        cache = self.runner.cache
+        longest = len(prompt) + sampling.max_tokens - 1
+        need = cache.most_pages_needed(longest, self.scheduler.config.max_num_batched_tokens)
+        for g, (n, have) in enumerate(zip(need, cache.pages_per_group())):
+            if n > have:
+                raise ValueError(f"{len(prompt)} prompt tokens and {sampling.max_tokens} new ones need {n} cache pages "
+                                 f"of {cache.page_size} tokens, the cache has {have} (group {g} of its layers)")
         vocab = self.runner.model.spec.vocab_size
         for t in prompt:
             if not 0 <= int(t) < vocab:
@@ -139,7 +148,8 @@ class LLMEngine:
                 "preemptions": self.scheduler.num_preemptions,
                 "waiting": len(self.scheduler.waiting),
                 "running": len(self.scheduler.running),
-                "pages": cache.num_pages,
+                "pages": cache.num_pages,                  # of the largest group
+                "pages_per_group": cache.pages_per_group(),
                 "pages_free": cache.free_pages(),          # one count per group of layers
                 "pages_taken_total": cache.pages_taken_total,
                 "prefix_pages_reused": cache.prefix_hits,

@@ -19,7 +19,7 @@ class Model:
         self.blocks = []
         for b in spec.blocks:
             mixer = build_part("mixer", b.mixer)
-            ffn = build_part("ffn", b.ffn)
+            ffn = build_part("ffn", b.ffn) if b.ffn is not None else None
             norms = {role: build_part("norm", s) for role, s in b.norms.items()}
             self.blocks.append(build_part("block", PartSpec(b.arrangement), mixer, ffn, norms))
         self.final_norm = build_part("norm", spec.final_norm)

@@ -114,18 +114,20 @@ class ModelRunner:
         env.ops.check_page_size(page_size)
         if prefix_caching and any(n is not None for n in model.state_needs()):
             raise ValueError("prefix caching cannot take over per-request state of a mixer")
-        self.cache = CacheManager(model.cache_needs(), page_size, num_pages, max_requests, prefix_caching)
+        self.cache = CacheManager(model.cache_needs(), page_size, num_pages, max_requests, prefix_caching,
+                                  max_step_tokens=max_batch_tokens)
         # The pages' contents: for every group the records its mixers declared, one tensor each,
-        # [layers in group, pages, *the record's page shape], zeroed.  (One page and one state
-        # slot more than the manager hands out: what the padding rows of a recorded decode
-        # step write to.)
+        # [layers in group, pages, *the record's page shape], zeroed.  A group that keeps all keys has
+        # ``num_pages`` pages, a window group no more than its requests can hold together.  (One page
+        # and one state slot more than the manager hands out: what the padding rows of a recorded
+        # decode step write to.)
         self.group_tensors: List[Dict[str, torch.Tensor]] = []
         for g in self.cache.groups:
             self.group_tensors.append({
-                rec.name: torch.zeros((len(g.cache_layers), num_pages + 1) + rec.page_shape(page_size),
+                rec.name: torch.zeros((len(g.cache_layers), g.pool.num_pages + 1) + rec.page_shape(page_size),
                                       dtype=rec.dtype or env.dtype, device=env.device)
                 for rec in g.need.records})
-        self.pad_page, self.pad_slot = num_pages, max_requests
+        self.pad_pages, self.pad_slot = [g.pool.num_pages for g in self.cache.groups], max_requests
         self.states: List[Optional[torch.Tensor]] = []
         for need in model.state_needs():
             self.states.append(None if need is None else torch.zeros(
@@ -249,7 +251,7 @@ class ModelRunner:
                 if len(tab):
                     rows_of[i, :len(tab)] = np.frombuffer(tab, dtype=np.int32)
             if pads:
-                rows_of[seqs:, 0] = self.pad_page
+                rows_of[seqs:, 0] = self.pad_pages[g]
         self.inputs.upload(lay["_end"].stop)
         dev = self.inputs.dev
         rows, seqs = rows + pads, seqs + pads

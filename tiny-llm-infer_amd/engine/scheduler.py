@@ -10,7 +10,9 @@ The policy is the reference's (engine/src/scheduler.cpp:40-121):
 2. Then prompts.  Waiting requests, in order, each get at most one portion per
    step, cut to the budget that is left.  A request is admitted only when the
    pages for all its current tokens are free (and a state slot); otherwise it
-   goes to the back of the queue.  With prefix caching, leading full pages that
+   goes to the back of the queue.  (Layers that keep a window of keys have pages
+   of their own, which a request takes portion by portion and gives back as the
+   window passes; an admitted request whose portion finds none waits a step.)  With prefix caching, leading full pages that
    the cache knows are taken over and not computed again.  A prompt that needs more pages than the pool
    owns is an error.
 3. If nothing could be scheduled while work remains, that is an error.
@@ -122,8 +124,8 @@ class Scheduler:
         self.waiting.appendleft(seq)
 
     def _pages_for_whole_pool(self, size: int) -> bool:
-        page = self.cache.page_size
-        return (size + page - 1) // page <= self.cache.num_pages
+        need = self.cache.most_pages_needed(size, self.config.max_num_batched_tokens)
+        return all(n <= have for n, have in zip(need, self.cache.pages_per_group()))
 
     def _admit(self, seq: Sequence) -> bool:
         if self.cache.free_slots() == 0:
@@ -131,10 +133,10 @@ class Scheduler:
         self.cache.admit(seq.request_id)
         # with prefix caching the leading full pages that are known are taken over
         cached = self.cache.adopt_prefix(seq.request_id, seq.token_ids) if self.cache.prefix_caching else 0
-        if not self.cache.can_reserve(seq.request_id, seq.size):
+        if not self.cache.can_hold_ahead(seq.request_id, seq.size):
             self.cache.release(seq.request_id)
             return False
-        self.cache.reserve(seq.request_id, seq.size)
+        self.cache.hold_ahead(seq.request_id, seq.size)
         seq.admitted = True
         seq.tokens_in_cache = cached
         return True
@@ -169,6 +171,10 @@ class Scheduler:
             if remaining <= 0:
                 raise SchedulerError(f"request {seq.request_id} waits although all its {seq.size} tokens are in the cache")
             count = min(remaining, budget - tokens)
+            if not self.cache.can_reserve(seq.request_id, seq.tokens_in_cache + count):
+                self.waiting.append(seq)          # (a window group has no pages for this portion yet)
+                continue
+            self.cache.reserve(seq.request_id, seq.tokens_in_cache + count)
             plan.items.append(PlanItem(seq, seq.tokens_in_cache, count, True))
             tokens += count
             if seq.tokens_in_cache + count == seq.size:

@@ -525,17 +525,13 @@ class HipOps:
         cos = sin = None
         rd = npos = 0
         if rotary is not None:
-            cos, sin, rd = rotary
+            cos, sin, rd = self._rotary(rotary, step)
             npos = cos.shape[0]
-            self._want(cos, "cos table", torch.float32, (npos, rd // 2))
-            self._want(sin, "sin table", torch.float32, (npos, rd // 2))
-            if step.max_seq_len > npos:
-                raise KernelError(f"a position reaches {step.max_seq_len}, the rotation table has {npos}")
         write = 1 if (cache is not None and cache.writes) else 0
         k_ptr = v_ptr = tab_ptr = None
         width = page = pages = 0
         if write:
-            kc, vc = cache.k, cache.v
+            kc, vc = cache.record("k"), cache.record("v")
             g = cache.group
             self._check_cache(kc, vc, g, kv_heads, head_dim, qkv.dtype, step)
             k_ptr, v_ptr, tab_ptr = kc.data_ptr(), vc.data_ptr(), g.tables.data_ptr()
@@ -551,6 +547,20 @@ class HipOps:
                        kv_heads, head_dim, self._stream())
         return q
 
+    def _rotary(self, rotary, step):
+        """(cos, sin, rotary_dim) of what a mixer passes as ``rotary``, checked.  The kernels turn
+        the pairs (i, i + rotary_dim/2); a fourth element that names another pairing is refused."""
+        cos, sin, rd = rotary[0], rotary[1], int(rotary[2])
+        if len(rotary) > 3 and rotary[3] != "half":
+            raise KernelError(f"the kernels rotate the pairs (i, i + rotary_dim/2) of a head, not the pairing "
+                              f"'{rotary[3]}'; the attention part reorders a head's elements for that")
+        npos = cos.shape[0]
+        self._want(cos, "cos table", torch.float32, (npos, rd // 2))
+        self._want(sin, "sin table", torch.float32, (npos, rd // 2))
+        if step.max_seq_len > npos:
+            raise KernelError(f"a position reaches {step.max_seq_len}, the rotation table has {npos}")
+        return cos, sin, rd
+
     def _check_cache(self, kc, vc, g, kv_heads, head_dim, dtype, step):
         pages = kc.shape[0]
         self._want(kc, "key cache", dtype, (pages, kv_heads, g.page_size, head_dim))
@@ -564,7 +574,7 @@ class HipOps:
         self._want(q, "queries", None, (T, heads * head_dim))
         if cache is None:
             raise KernelError("attention needs a cache layer")
-        kc, vc, g = cache.k, cache.v, cache.group
+        kc, vc, g = cache.record("k"), cache.record("v"), cache.group
         self._check_cache(kc, vc, g, kv_heads, head_dim, q.dtype, step)
         out = torch.empty_like(q)
         if q.dtype == torch.bfloat16 and head_dim <= 256 and g.page_size >= 4 and not self.force_plain:
@@ -594,7 +604,7 @@ class HipOps:
             if not (step.max_rows_per_seq == 1 and qkv.dtype == torch.bfloat16 and cache is not None
                     and head_dim % 64 == 0 and head_dim <= 256 and heads // kv_heads <= 16
                     and cache.group.page_size >= 8 and not self.force_plain and not self.unfused_decode
-                    and (rotary is None or rotary[2] == head_dim)):
+                     and (rotary is None or rotary[2] == head_dim)):
                 qkv, sums = self.resolve(qkv), None
         fusable = (qkv.dtype == torch.bfloat16 and cache is not None and head_dim % 64 == 0
                    and head_dim <= 256 and not self.force_plain and not self.unfused_decode
@@ -614,7 +624,7 @@ class HipOps:
                        (sums.parts.shape[0], T, (heads + 2 * kv_heads) * head_dim))
         else:
             self._want(qkv, "qkv", None, (T, (heads + 2 * kv_heads) * head_dim))
-        kc, vc, g = cache.k, cache.v, cache.group
+        kc, vc, g = cache.record("k"), cache.record("v"), cache.group
         self._check_cache(kc, vc, g, kv_heads, head_dim, qkv.dtype, step)
         qw, qe = q_norm if q_norm is not None else (None, 0.0)
         kw, ke = k_norm if k_norm is not None else (None, 0.0)
@@ -623,12 +633,7 @@ class HipOps:
                 self._want(w, "head norm weight", torch.float32, (head_dim,))
         cos = sin = None
         if rotary is not None:
-            cos, sin, rd = rotary
-            npos = cos.shape[0]
-            self._want(cos, "cos table", torch.float32, (npos, rd // 2))
-            self._want(sin, "sin table", torch.float32, (npos, rd // 2))
-            if step.max_seq_len > npos:
-                raise KernelError(f"a position reaches {step.max_seq_len}, the rotation table has {npos}")
+            cos, sin, rd = self._rotary(rotary, step)
         out = torch.empty((T, heads * head_dim), dtype=qkv.dtype, device=self.device)
         splits, per_split, partial = self._decode_splits(step.num_rows, step.reach, g, heads, kv_heads, head_dim, window)
         self._call(self.lib.tli_qkv_attention_decode_bf16, None if sums is not None else qkv.data_ptr(),
@@ -648,7 +653,7 @@ class HipOps:
         one wave only, so nothing is done twice and q is never written)."""
         T = step.num_rows
         self.qkv_to_cache(qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary, queries=False)
-        kc, vc, g = cache.k, cache.v, cache.group
+        kc, vc, g = cache.record("k"), cache.record("v"), cache.group
         self._check_cache(kc, vc, g, kv_heads, head_dim, qkv.dtype, step)
         qw, qe = q_norm if q_norm is not None else (None, 0.0)
         cos, sin = (rotary[0], rotary[1]) if rotary is not None else (None, None)

@@ -1,7 +1,8 @@
 """Attention over the paged cache with grouped heads.
 
 Order (model/src/qwen3_paged_batch.cpp:147-271): q, k, v projections (no
-bias) -> optional per-head norm of q and of k -> optional rotation of q and k
+bias) -> optional per-head norm of q and of k -> optional rotation of q and k (pairs (i, i + d/2) as the reference turns them,
+kernels/src/rope_kernel_cpu.cpp:156-179, or neighbours for an encoding that says so)
 -> k and v into the cache at (table[pos // page], pos % page) -> for the row at
 position p and head h, kv head h // (heads / kv_heads), scores (q.k) * scale
 over the keys 0..p (kernels/src/paged_attention_cpu.cpp:16-69), or over
@@ -18,7 +19,7 @@ import torch
 
 from ..cache.manager import CacheNeed
 from ..weights.loader import TensorDecl
-from .base import BuildEnv, Mixer, StepView, build_part, register_part
+from .base import ROTARY_PAIRINGS, BuildEnv, Mixer, RotaryTables, StepView, build_part, register_part
 from .linear import as_matrix, fuse_rows
 
 
@@ -58,12 +59,49 @@ class PagedAttention(Mixer):
     def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
         super().load(weights, env)
         n = self.spec.names
-        self.w_qkv = fuse_rows([weights[n["q"]], weights[n["k"]], weights[n["v"]]], env)
-        self.w_o = as_matrix(weights[n["o"]], env)
         for part in (self.q_norm, self.k_norm, self.position):
             if part is not None:
                 part.load(weights, env)
         env.ops.check_attention_sizes(self.heads, self.kv_heads, self.head_dim)
+        # The kernels turn the pairs (i, i + rotary_dim/2) of a head.  An encoding that pairs
+        # neighbours (2i, 2i + 1) is served by the same kernels: a head's scores q.k do not change
+        # when q and k are permuted alike, so the rows of the q and k projections (and the weights
+        # of their norms) are put in the order 0, 2, 4, .., 1, 3, 5, .. once, here.
+        self.rotary, order = None, None
+        tables = self.position.rotary() if self.position is not None else None
+        if tables is not None:
+            tables = RotaryTables(*tables)
+            if tables.pairing not in ROTARY_PAIRINGS:
+                raise ValueError(f"rotary pairing '{tables.pairing}' is not known; known: {', '.join(ROTARY_PAIRINGS)}")
+            rd = int(tables.rotary_dim)
+            if rd <= 0 or rd % 2 or rd > self.head_dim:
+                raise ValueError(f"rotary_dim {rd} must be even and at most head_dim {self.head_dim}")
+            if tables.pairing == "interleaved":
+                order = torch.cat([torch.arange(0, rd, 2), torch.arange(1, rd, 2), torch.arange(rd, self.head_dim)])
+            self.rotary = (tables.cos, tables.sin, rd)
+        # The norms of q and k per head are applied inside the kernels, which have the RMS norm
+        # built in: any other kind of norm there is refused, not taken for one.
+        self.head_norms = []
+        for role, norm in (("q", self.q_norm), ("k", self.k_norm)):
+            rms = None
+            if norm is not None:
+                rms = norm.as_rms()
+                if rms is None:
+                    raise ValueError(f"the {role} norm of an attention layer is '{norm.spec.kind}': the attention "
+                                     f"kernels apply it per head themselves and have the RMS norm only")
+                weight, eps = rms
+                if tuple(weight.shape) != (self.head_dim,):
+                    raise ValueError(f"the {role} norm has {tuple(weight.shape)} weights, a head has {self.head_dim} elements")
+                rms = (weight[order.to(weight.device)].contiguous() if order is not None else weight, float(eps))
+            self.head_norms.append(rms)
+
+        def heads_in_order(w: torch.Tensor, heads: int) -> torch.Tensor:
+            if order is None:
+                return w
+            return w.view(heads, self.head_dim, self.hidden)[:, order.to(w.device)].reshape(heads * self.head_dim, self.hidden)
+        self.w_qkv = fuse_rows([heads_in_order(weights[n["q"]], self.heads),
+                                heads_in_order(weights[n["k"]], self.kv_heads), weights[n["v"]]], env)
+        self.w_o = as_matrix(weights[n["o"]], env)
 
     def cache_need(self) -> Optional[CacheNeed]:
         return CacheNeed.keys_and_values(self.kv_heads, self.head_dim, self.window)
@@ -79,12 +117,8 @@ class PagedAttention(Mixer):
     def forward(self, x: torch.Tensor, step: StepView) -> torch.Tensor:
         ops = self.env.ops
         qkv = ops.linear(x, self.w_qkv, sums_only=True)      # partial sums, if k was split, are the attention's to add
-        rot = self.position.rotary() if self.position is not None else None
-        o = ops.qkv_attention(
-            qkv, step, step.cache, self.heads, self.kv_heads, self.head_dim,
-            None if self.q_norm is None else (self.q_norm.weight, self.q_norm.eps),
-            None if self.k_norm is None else (self.k_norm.weight, self.k_norm.eps),
-            rot, self.scale, self.window)
+        o = ops.qkv_attention(qkv, step, step.cache, self.heads, self.kv_heads, self.head_dim,
+                              self.head_norms[0], self.head_norms[1], self.rotary, self.scale, self.window)
         return ops.linear(o, self.w_o, deferred=True)       # goes to the next norm as the residual delta
 
 

@@ -15,7 +15,7 @@ No part knows which architecture it is in.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Callable, Dict, List, Optional
+from typing import Any, Callable, Dict, List, NamedTuple, Optional
 
 import torch
 
@@ -44,14 +44,6 @@ class GroupView:
     page_size: int
     window: Optional[int]
 
-    @property
-    def k(self) -> torch.Tensor:       # the attention part's records:
-        return self.tensors["k"]       # [layers in group, pages, kv heads, page_size, head_dim]
-
-    @property
-    def v(self) -> torch.Tensor:
-        return self.tensors["v"]       # [layers in group, pages, kv heads, head_dim, page_size]
-
 
 @dataclass
 class LayerCache:
@@ -63,14 +55,6 @@ class LayerCache:
     def record(self, name: str) -> torch.Tensor:
         """This layer's tensor of the record ``name``: [pages, *page shape]."""
         return self.group.tensors[name][self.layer]
-
-    @property
-    def k(self) -> torch.Tensor:
-        return self.group.tensors["k"][self.layer]
-
-    @property
-    def v(self) -> torch.Tensor:
-        return self.group.tensors["v"][self.layer]
 
 
 @dataclass
@@ -124,11 +108,25 @@ class Part:
         return 0
 
 
-class PositionEncoding(Part):
-    """Rotary encodings expose ``rotary()``: cos and sin tables
-    [positions, rotary_dim/2] in float32 and the pairing of elements."""
+class RotaryTables(NamedTuple):
+    """What a rotary encoding hands to the mixer that applies it.  Pair i of a head, i <
+    rotary_dim/2, is turned by the angle whose cosine and sine are ``cos[position, i]`` and
+    ``sin[position, i]``; ``pairing`` says which two elements pair i is: "half" = (i, i +
+    rotary_dim/2), "interleaved" = (2i, 2i + 1).  Elements from ``rotary_dim`` on are left alone."""
+    cos: torch.Tensor             # float32 [positions, rotary_dim / 2]
+    sin: torch.Tensor
+    rotary_dim: int
+    pairing: str = "half"
 
-    def rotary(self):
+
+ROTARY_PAIRINGS = ("half", "interleaved")
+
+
+class PositionEncoding(Part):
+    """Rotary encodings expose ``rotary()``: a ``RotaryTables`` (None for an encoding that
+    is not rotary and acts elsewhere)."""
+
+    def rotary(self) -> Optional[RotaryTables]:
         return None
 
 
@@ -142,6 +140,12 @@ class Norm(Part):
     # returned (a product not run yet, or partial sums).  For a norm without it the caller
     # makes a tensor of the delta first.
     takes_unfinished_products = False
+
+    def as_rms(self):
+        """(weight float32 [size], eps) if this norm is y = weight * x / sqrt(mean(x^2) + eps) and
+        nothing else, so that a kernel which has that formula built in (the attention kernels, for
+        the norms of q and k per head) can apply it; None for every other kind of norm."""
+        return None
 
     def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor],
                 rows: Optional[torch.Tensor] = None, num_rows: Optional[int] = None) -> torch.Tensor:

@@ -32,6 +32,9 @@ class RMSNorm(Norm):
         # vectors are held in float32: exact for 16-bit storage, unchanged for 32-bit
         self.weight = weights[self.weight_name].to(torch.float32).contiguous()
 
+    def as_rms(self):
+        return self.weight, self.eps
+
     def forward(self, resid, delta, rows=None, num_rows=None, lazy=False):
         """``lazy``: the rows go to matrix products only, which may then apply the rows'
         scalar factor themselves (the kernel library decides; see its ``add_rmsnorm``)."""

@@ -13,7 +13,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from .base import BuildEnv, PositionEncoding, register_part
+from .base import BuildEnv, PositionEncoding, RotaryTables, register_part
 
 
 class NeoxRope(PositionEncoding):
@@ -48,8 +48,8 @@ class NeoxRope(PositionEncoding):
         self.sin = torch.from_numpy(np.sin(a64).astype(np.float32)).to(env.device).contiguous()
         env.shared[key] = (self.cos, self.sin)
 
-    def rotary(self):
-        return self.cos, self.sin, self.rotary_dim
+    def rotary(self) -> RotaryTables:
+        return RotaryTables(self.cos, self.sin, self.rotary_dim, "half")
 
 
 register_part("position", "rope_neox", NeoxRope)
