@@ -116,6 +116,31 @@ def test_random_weights_folder_round_trip(model_folders):
     assert torch.equal(again.read("lm_head.weight"), ck.read("lm_head.weight"))
 
 
+def test_random_weights_are_a_function_of_seed_tensor_and_element(model_folders):
+    """The file of a random model against the rule written out again in numpy (tests/plain_random.py,
+    its quantiles from the standard library): every tensor bit for bit.  An element does not
+    depend on the tensor's shape or on what else is drawn."""
+    import numpy as np
+    import plain_random
+    from tiny_llm_infer_amd.weights.random_init import draw_normal
+    for name in ("A", "C"):
+        decls = _decls(name)
+        want = plain_random.model_weights([(d.name, d.shape, d.init) for d in decls], TINY[name]["seed"])
+        ck = Checkpoint(model_folders[name])
+        for d in decls:
+            got = ck.read(d.name)
+            assert got.dtype == torch.bfloat16
+            assert np.array_equal(got.double().numpy(), want[d.name]), d.name
+        ck.close()
+    a = draw_normal((7, 1000), 5, 3, 0.02)
+    b = draw_normal((7000,), 5, 3, 0.02)
+    assert torch.equal(a.reshape(-1), b) and torch.equal(draw_normal((10,), 5, 3, 0.02), b[:10])
+    assert not torch.equal(draw_normal((7000,), 5, 4, 0.02), b) and not torch.equal(draw_normal((7000,), 6, 3, 0.02), b)
+    big = draw_normal((2000000,), 1, 0, 1.0).double()
+    assert abs(float(big.mean())) < 3e-3 and abs(float(big.std()) - 1) < 3e-3
+    assert abs(float((big ** 4).mean()) - 3) < 0.03 and 4.2 < float(big.abs().max()) < 4.5       # normal, cut at 4.5 sigma
+
+
 def test_storage_rule(tmp_path):
     """16-bit floats -> bfloat16 (or widened for a float32 run); 32-bit stays;
     integer tables -> int32."""

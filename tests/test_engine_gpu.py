@@ -337,6 +337,35 @@ def test_decode_steps_are_padded_to_few_sizes(model_folders):
     assert eng.runner.cache.free_pages() == eng.runner.cache.pages_per_group()
 
 
+def test_a_default_run_never_asks_for_the_row_major_form_of_a_matrix(tmp_path):
+    """bfloat16 matrices are held once, in the decode layout.  Prefill of more than 128 rows,
+    portions, recorded decode steps: nothing puts the row-major form together again.  The plain
+    kernels do ask for it, and then it is made once for every matrix and kept."""
+    from tiny_llm_infer_amd.config import Qwen3Config
+    from tiny_llm_infer_amd.engine.llm_engine import LLMEngine
+    from tiny_llm_infer_amd.engine.loading import write_random_model
+    from tiny_llm_infer_amd.parts.linear import Matrix
+    from tiny_llm_infer_amd.sampling.params import SamplingParams
+    cfg = Qwen3Config.from_dict(dict(
+        architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2, head_dim=64, vocab_size=512,
+        hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+        max_position_embeddings=1024, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False))
+    folder = write_random_model(str(tmp_path / "m"), "Qwen3ForCausalLM", cfg, seed=2)
+    eng = LLMEngine.from_folder(folder, dtype="bfloat16", device="cuda:0", max_model_len=512, page_size=16,
+                                num_kv_blocks=128, max_num_seqs=4, max_num_batched_tokens=256)
+    before = Matrix.rebuilt
+    prompts = [random_prompt(512, n, n) for n in (300, 40, 7, 150)]
+    first = eng.generate(prompts, SamplingParams(max_tokens=6, ignore_eos=True))
+    assert Matrix.rebuilt == before and eng.runner.graph_replays > 0
+    eng.runner.env.ops.use_plain_kernels()
+    eng.generate(prompts, SamplingParams(max_tokens=6, ignore_eos=True))
+    made = Matrix.rebuilt - before
+    assert made == 2 * 4 + 1                      # q/k/v, o, gate/up, down of two layers, and the head
+    eng.generate(prompts, SamplingParams(max_tokens=6, ignore_eos=True))
+    assert Matrix.rebuilt - before == made        # kept, not made again
+    assert all(len(r.token_ids) == 6 for r in first)
+
+
 def test_prefix_caching_on_the_gpu(model_folders):
     """Requests that share a prompt prefix take its pages over instead of computing
     them; the tokens are those of an engine without the cache."""

@@ -618,6 +618,23 @@ RAW_CASES = [
 ]
 
 
+def test_the_prefill_kernel_is_told_of_keys_before_its_own_rows_only(ops):
+    """The launch rule of the prefill kernel is told whether its rows have many keys before them.
+    When the sequences that decode have gone to the decode kernel, the lengths that count are
+    those of the portions that are left, not the longest sequence of the step."""
+    class Step:
+        num_seqs, h_seq_len, max_seq_len = 3, [6000, 90, 300], 6000
+    assert ops._prefill_mode(Step, 302) == 13                  # all three in the prefill kernel: one has 5,999 keys before its row
+    assert ops._prefill_mode(Step, 300, first=2) == 0          # the portion alone starts at position 0
+    Step.h_seq_len = [6000, 90, 2300]
+    assert ops._prefill_mode(Step, 300, first=2) == 13         # 300 rows behind 2,000 keys
+    ops.prefill_direct = 3
+    try:
+        assert ops._prefill_mode(Step, 300, first=2) == 3      # a form forced by a test stays
+    finally:
+        ops.prefill_direct = 0
+
+
 @pytest.mark.parametrize("mode", [0, 3])
 @pytest.mark.parametrize("case", RAW_CASES)
 def test_attention_from_raw_projections(ops, case, mode):

@@ -20,7 +20,7 @@ def _library():
     lib.tli_sample_no_alloc.argtypes = [P, I, I, P, P, P, P, P]
     lib.tli_sample_scratch_bytes.argtypes = [I]
     for fn in (lib.tli_sample, lib.tli_sample_no_alloc, lib.tli_sample_scratch_bytes,
-               lib.tli_sample_no_alloc_max_rows):
+               lib.tli_sample_no_alloc_max_rows, lib.tli_sample_no_alloc_prepare):
         fn.restype = I
     return lib
 
@@ -67,3 +67,37 @@ def test_sampling_without_allocation_matches_sampling_with_a_callers_scratch():
     assert b"rows" in lib.tli_last_error()
     torch.cuda.synchronize()
     assert out.tolist() == [7, 7, 7, 7]
+
+
+def test_sampling_without_allocation_recorded_into_a_graph():
+    """What the entry point is for: after the address of the array has been looked up outside
+    any capture, the call is recorded into a HIP graph, which is replayed several times on new
+    logits, with eager work and synchronisation between the replays; every replay gives what
+    tli_sample gives for the same logits."""
+    lib = _library()
+    assert lib.tli_sample_no_alloc_prepare() == 0, lib.tli_last_error()
+    rows, vocab = 9, 40007
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    logits = torch.randn((rows, vocab), generator=gen, device="cuda", dtype=torch.float32)
+    temps = torch.full((rows,), 0.9, device="cuda", dtype=torch.float32)
+    temps[3] = 0.0
+    seeds = torch.arange(7, 7 + rows, device="cuda", dtype=torch.int64)
+    out = torch.full((rows,), -2, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        code = lib.tli_sample_no_alloc(logits.data_ptr(), rows, vocab, temps.data_ptr(), seeds.data_ptr(), None,
+                                       out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert code == 0, lib.tli_last_error()
+    for replay in range(4):
+        logits.copy_(torch.randn((rows, vocab), generator=gen, device="cuda"))          # eager work between replays
+        seeds += 1000
+        graph.replay()
+        torch.cuda.synchronize()
+        want = torch.full((rows,), -1, dtype=torch.int32, device="cuda")
+        scratch = torch.empty(lib.tli_sample_scratch_bytes(rows), dtype=torch.uint8, device="cuda")
+        assert lib.tli_sample(logits.data_ptr(), rows, vocab, temps.data_ptr(), seeds.data_ptr(), None,
+                              want.data_ptr(), scratch.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {replay}"
+        assert int(out[3]) == int(logits[3].argmax())

@@ -256,6 +256,7 @@ REPLAY_HELP = """Trace replay: feed given token ids through a model step by step
 the logits at the wanted places.  Nothing is sampled.
 
     trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
+    trace_run --config FILE --random-weights [--seed S] --dtype ... (weights drawn, no folder)
 
 Steps are read from standard input, one JSON object a line:
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
@@ -270,7 +271,11 @@ def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
     kernels that generation uses, driven by a trace instead of a scheduler."""
     ap = argparse.ArgumentParser(prog=prog, description=REPLAY_HELP,
                                  formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--model", help="folder with config.json and model.safetensors")
+    ap.add_argument("--config", help="a config.json, with --random-weights, instead of --model")
+    ap.add_argument("--random-weights", action="store_true",
+                    help="draw the weights from --seed (the same ones a model folder written with that seed holds)")
+    ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
@@ -287,15 +292,18 @@ def run_replay(argv: List[str], prog: str = "model_main --replay") -> int:
     args = ap.parse_args(argv)
     if 64 % args.page_size:
         ap.error("--page-size must divide 64")
+    if bool(args.model) == bool(args.random_weights):
+        ap.error("give --model DIR, or --config FILE with --random-weights")
     print("[trace_run] loading the kernel library (compiled at the first call)", file=sys.stderr, flush=True)
-    from .engine.loading import load_model
     from .engine.replay import Replayer
     from .engine.runner import ModelRunner
-    model, cfg = load_model(args.model, args.dtype, _device(args.device), ops=_ops(_device(args.device), args.kernels))
+    args.quantization = "none"
+    model = _load(args, None)
+    cfg = model.spec.architecture
     pages = max(1, (args.max_tokens + args.page_size - 1) // args.page_size)
     runner = ModelRunner(model, model.env, page_size=args.page_size, num_pages=pages,
                          max_requests=args.max_live, max_batch_tokens=args.max_step_tokens)
-    print(f"[trace_run] ready: {type(cfg).__name__}, {args.dtype}, {pages} pages of {args.page_size}, "
+    print(f"[trace_run] ready: {cfg}, {args.dtype}, {pages} pages of {args.page_size}, "
           f"kernels: {args.kernels}", file=sys.stderr, flush=True)
     Replayer(runner, args.out).run_stream(sys.stdin, ack=sys.stdout)
     return 0

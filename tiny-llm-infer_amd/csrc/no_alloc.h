@@ -12,6 +12,9 @@
 // Arguments and result are those of tli_sample without `scratch`.  The caller still passes
 // inputs and outputs.  It calls no hipMalloc, hipFree or allocating library routine; at its
 // first call on a device it asks once for the address of that device's copy of the array.
+// That first query must not fall inside a stream capture: before recording the entry point
+// into a HIP graph, call tli_sample_no_alloc_prepare() (or the entry point itself, eagerly)
+// once on that device, with that device current.
 //
 // Limit: rows <= TLI_SAMPLE_NO_ALLOC_MAX_ROWS (more is refused with an error, nothing
 // launched).  The array takes 256 KiB on every GPU the library runs on until the process ends.
@@ -28,3 +31,4 @@
 extern "C" int tli_sample_no_alloc(const float* logits, int rows, int vocab, const float* temperatures,
                                    const uint32_t* seeds, const float* top_p, int* out, void* stream);
 extern "C" int tli_sample_no_alloc_max_rows();
+extern "C" int tli_sample_no_alloc_prepare();

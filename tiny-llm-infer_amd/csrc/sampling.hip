@@ -215,6 +215,15 @@ extern "C" int tli_sample_no_alloc(const float* logits, int rows, int vocab, con
 
 extern "C" int tli_sample_no_alloc_max_rows() { return TLI_SAMPLE_NO_ALLOC_MAX_ROWS; }
 
+// Looks up the current device's copy of the array and launches nothing: for callers that
+// record tli_sample_no_alloc into a HIP graph, so that the one query of the runtime (and the
+// loading of this library's code on the device that may come with it) happens before the
+// capture begins and not inside it.
+extern "C" int tli_sample_no_alloc_prepare() {
+    void* ptr = nullptr;
+    return scratch_of_current_device(&ptr);
+}
+
 // the same draw on the host, for tests and for callers that hold logits there
 
 extern "C" float tli_sample_uniform(uint32_t seed_lo, uint32_t seed_hi, uint32_t token) {

@@ -20,7 +20,8 @@ and of ``want``), and ``index.jsonl``, one JSON object a step:
 
 ``rows`` names the request and the position in it of every row of the file;
 ``block_tables`` holds, for every request of the step and every group of cache
-layers, the pages the request held when the step ran (-1: given back).
+layers, the pages the step ran with: taken after the step's pages were reserved
+and before a window gave any back (-1: given back by an earlier step).
 """
 from __future__ import annotations
 
@@ -43,6 +44,12 @@ class Replayer:
         if out_dir is not None:
             os.makedirs(out_dir, exist_ok=True)
             self.index = open(os.path.join(out_dir, "index.jsonl"), "w", encoding="utf-8")
+            runner.keep_tables = True
+
+    def close(self) -> None:
+        if self.index is not None:
+            self.index.close()
+            self.index = None
 
     def run_step(self, record: dict) -> Optional[np.ndarray]:
         """Run one trace step; returns float32 [wanted, vocab] or None."""
@@ -63,7 +70,7 @@ class Replayer:
                 if self.out_dir is not None:
                     out.astype("<f4").tofile(os.path.join(self.out_dir, f"{record['step']}.f32"))
         if self.index is not None:
-            tables = {str(e.key): [list(t) for t in self.runner.cache.get(e.key).tables] for e in entries}
+            tables = {str(e.key): self.runner.tables_run[e.key] for e in entries}
             self.index.write(json.dumps({"step": record.get("step"), "file": f"{record['step']}.f32" if rows else None,
                                          "rows": rows, "block_tables": tables}) + "\n")
             self.index.flush()
@@ -73,12 +80,15 @@ class Replayer:
         return out
 
     def run_stream(self, lines: Iterable[str], ack: Optional[IO[str]] = None) -> None:
-        for line in lines:
-            line = line.strip()
-            if not line:
-                continue
-            record = json.loads(line)
-            self.run_step(record)
-            if ack is not None:
-                ack.write(f"done {record['step']}\n")
-                ack.flush()
+        try:
+            for line in lines:
+                line = line.strip()
+                if not line:
+                    continue
+                record = json.loads(line)
+                self.run_step(record)
+                if ack is not None:
+                    ack.write(f"done {record['step']}\n")
+                    ack.flush()
+        finally:
+            self.close()

@@ -145,6 +145,11 @@ class ModelRunner:
         self.graphs = {}
         self.graph_pool = None
         self.graph_replays = 0
+        # for the replay tool's index: with ``keep_tables`` set, the block tables that the last step
+        # ran with (request -> per group a list of pages), taken after its pages were reserved and
+        # before a window gave any back
+        self.keep_tables = False
+        self.tables_run: Dict[Hashable, List[List[int]]] = {}
 
     # ---- requests ---------------------------------------------------------
     def admit(self, key: Hashable):
@@ -338,6 +343,8 @@ class ModelRunner:
             self.cache.reserve(e.key, self.cache.get(e.key).num_tokens + len(e.tokens))
         if feed is None and any(e.token_from is not None for e in entries):
             raise StepError("an entry takes its token from the device but no tensor was given")
+        if self.keep_tables:
+            self.tables_run = {e.key: [list(t) for t in self.cache.get(e.key).tables] for e in entries}
         wanted = sum(len(e.want) for e in entries)
         if self.use_graphs and wanted == len(entries) and all(len(e.tokens) == 1 for e in entries):
             view = self._pack(entries, feed, pad_to=_decode_bucket(len(entries)))

@@ -92,6 +92,7 @@ def load_library():
         "tli_qkv_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, P, F, P, P, F, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
         "tli_sample_scratch_bytes": [I],
+        "tli_random_normal": [P, ctypes.c_longlong, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, P, F, F, I, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -682,7 +683,7 @@ class HipOps:
                        0, float(scale), int(window or 0), splits, per_split, None, 0, self._stream())
         else:
             first = 0
-        direct = self._prefill_mode(step, T - first)
+        direct = self._prefill_mode(step, T - first, first)
         self._call(self.lib.tli_qkv_attention_prefill_bf16, qkv.data_ptr(), out.data_ptr(), kc.data_ptr(),
                    vc.data_ptr(), step.row_start.data_ptr() + 4 * first, step.seq_start.data_ptr() + 4 * first,
                    step.num_seqs - first, T - first, g.tables.data_ptr() + 4 * first * g.table_width, g.table_width,
@@ -691,11 +692,13 @@ class HipOps:
                    direct, self._stream())
         return out
 
-    def _prefill_mode(self, step, rows):
-        """The mode argument of the prefill attention kernels.  Their launch rule wants to know
-        whether the rows have many keys before them, and the lengths themselves are on the
-        device: 13 says that they have (the longest sequence is a quarter longer than all rows)."""
-        if not self.prefill_direct and step.max_seq_len > rows + rows // 4:
+    def _prefill_mode(self, step, rows, first=0):
+        """The mode argument of the prefill attention kernels for the sequences from ``first`` on
+        (``rows`` rows in all).  Their launch rule wants to know whether the rows have many keys
+        before them, and the lengths themselves are on the device: 13 says that they have (the
+        longest of those sequences is a quarter longer than all the rows)."""
+        longest = max(step.h_seq_len[first:step.num_seqs]) if step.h_seq_len else step.max_seq_len
+        if not self.prefill_direct and longest > rows + rows // 4:
             return 13
         return int(self.prefill_direct)
 

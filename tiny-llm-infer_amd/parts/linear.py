@@ -15,8 +15,12 @@ class Matrix:
     stream in a row; the row-major form ``w`` [out, in] is held beside it only where the
     kernel library says it multiplies with it (products of many rows given to the BLAS
     library) or where there is no decode layout (a float32 run, a width the layout does not
-    take).  Asked for all the same (the plain kernels), ``w`` is put together again from the
-    decode layout, a copy made on the spot."""
+    take).  Asked for all the same (the plain kernels, a product too large for the offsets of
+    the kernel for many rows), ``w`` is put together from the decode layout once and kept from
+    then on (``rebuilt`` counts how often that happened in the process): a default run never
+    asks for it, and one that does pays the second copy once, not at every product."""
+
+    rebuilt = 0
 
     def __init__(self, w: torch.Tensor, env: BuildEnv, decode_layout: bool = True):
         w = w.to(env.dtype).contiguous()
@@ -32,8 +36,12 @@ class Matrix:
 
     @property
     def w(self) -> torch.Tensor:
-        if self._w is not None:
-            return self._w
+        if self._w is None:
+            self._w = self._rebuild()
+            Matrix.rebuilt += 1
+        return self._w
+
+    def _rebuild(self) -> torch.Tensor:
         return self.ops.untile_matrix(self.tiled, self.shape)
 
     def nbytes(self) -> int:
@@ -63,12 +71,9 @@ class GatedMatrix(Matrix):
         if self.gated is not None and not self._keeps_row_major():
             self._w = None
 
-    @property
-    def w(self) -> torch.Tensor:
-        if self._w is not None:
-            return self._w
+    def _rebuild(self) -> torch.Tensor:
         if self.gated is None:
-            return super().w
+            return super()._rebuild()
         rows, k = self.shape
         pairs = self.ops.untile_matrix(self.gated, (rows, k)).view(-1, 2, 16, k)      # [block, gate/up, 16, k]
         return torch.cat([pairs[:, 0].reshape(self.inter, k), pairs[:, 1].reshape(self.inter, k)], dim=0)

@@ -119,18 +119,15 @@ def load_tensors(model_path: str, decls: Sequence[TensorDecl], run_dtype: torch.
 
 def random_tensor(decl: TensorDecl, seed: int, index: int, dtype: torch.dtype,
                   device="cpu", std: float = 0.02) -> torch.Tensor:
-    """The ``index``-th tensor of a random model: drawn in float32 from a
-    generator seeded by (seed, index), then rounded to ``dtype``."""
+    """The ``index``-th tensor of a random model: N(0, std^2) ("normal") or N(1, std^2)
+    ("ones_normal") in float32, every element a function of (seed, index, its place) alone and
+    the same bits wherever it is drawn (``random_init.draw_normal``), then rounded to ``dtype``."""
     if decl.init == "int":
         return torch.zeros(decl.shape, dtype=torch.int32, device=device)
-    gen = torch.Generator(device=device)
-    gen.manual_seed((int(seed) * 1000003 + index * 7919 + 12345) & 0x7FFFFFFFFFFFFFFF)
-    t = torch.empty(decl.shape, dtype=torch.float32, device=device)
-    t.normal_(0.0, std, generator=gen)
-    if decl.init == "ones_normal":
-        t += 1.0
-    elif decl.init != "normal":
+    if decl.init not in ("normal", "ones_normal"):
         raise ValueError(f"unknown initialisation '{decl.init}' for {decl.name}")
+    from .random_init import draw_normal
+    t = draw_normal(tuple(decl.shape), seed, index, std, 1.0 if decl.init == "ones_normal" else 0.0, device)
     return t.to(dtype)
 
 
