@@ -5,7 +5,14 @@ of one 2,048-token prompt and decode at batch 1 and 64.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
 
 A step is one decode step of the engine (schedule, run the batch, sample,
-post-process).  One JSON line is printed.
+post-process).  One JSON line is printed.  Beside the headline, ``points`` holds (all
+with 128-token prompts unless the name says otherwise, tokens a second and the fraction of
+the HBM peak that the bytes a step has to read make of its time):
+  decode_b1, decode_b64                      a few steps at batch 1 and 64
+  decode_b{1,8,64}_128out                    all 128 output tokens of 128-token prompts
+  decode_b{8,64}_ctx4096                     contexts that end at 4,096 tokens
+  qwen3_14b_*, qwen3_32b_*                   decode at batch 8 and the prefill of 2,048 tokens at
+                                             the layer sizes of the larger models (configs/)
 """
 import argparse
 import json
@@ -57,7 +64,8 @@ def main():
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-points", action="store_true", help="skip every point beside the headline")
+    ap.add_argument("--no-other-shapes", action="store_true", help="skip the points at the layer sizes of the larger models")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiles)")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement (for profiles)")
     ap.add_argument("--own-products", action="store_true",
@@ -74,6 +82,7 @@ def main():
         print(f"bench.py runs on one GPU only; --gpus {args.gpus} is not supported (single-GPU engine)")
         return 2
 
+    import gc
     import random
 
     import torch
@@ -95,40 +104,46 @@ def main():
     cfg = Qwen3Config.from_dict(cfg_json)
     elem = 2 if args.dtype == "bfloat16" else 4
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
-    t0 = time.time()
     from tiny_llm_infer_amd.kernels.ops import HipOps
-    ops = HipOps("cuda:0")
-    # which kernel multiplies more than 128 rows is settled before the weights are loaded: a matrix
-    # keeps its row-major form only where the library (or the plain kernels of the untimed check) reads it
-    ops.many_rows = "library" if args.library_products else ("measure" if args.measured_products else "own")
-    ops.rows_cfg = args.rows_cfg
-    before = torch.cuda.memory_allocated()
-    model = random_model("Qwen3ForCausalLM", cfg, args.seed, args.dtype, "cuda:0", args.context, ops=ops)
-    weight_gb = (torch.cuda.memory_allocated() - before) / 1e9
-    torch.cuda.synchronize()
-    print(f"[bench] model with {layers} layers on the device in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
-
     page = 16
-    max_batch = args.batch if args.no_points else max(64, args.batch)      # the points run 64 requests
     budget = max(args.prefill_tokens, 2048)
-
-    def prefill_steps(batch):
-        """Steps in which the prompts are taken in; those taken in first decode meanwhile."""
-        return (batch * args.prompt_len + budget - 1) // budget + 1
-    pages = max_batch * ((args.prompt_len + args.steps + args.warmup + prefill_steps(max_batch) + 64 + page - 1)
-                         // page) + (args.prefill_tokens + page - 1) // page + 8
-    engine = LLMEngine.from_model(model, max_model_len=args.context, page_size=page, num_kv_blocks=pages,
-                                  max_num_seqs=max_batch, max_num_batched_tokens=budget)
     rng = random.Random(args.seed)
-    vocab = cfg.vocab_size
 
-    def decode_run(batch, steps, warmup):
-        """Prefill ``batch`` prompts, then time ``steps`` decode steps."""
+    def make_engine(conf, max_batch, longest, outputs):
+        """A model of ``conf`` with random weights and an engine whose cache holds ``max_batch``
+        requests of ``longest`` prompt tokens and ``outputs`` new ones beside one prompt of
+        --prefill-tokens."""
+        t0 = time.time()
+        ops = HipOps("cuda:0")
+        # which kernel multiplies more than 128 rows is settled before the weights are loaded: a matrix
+        # keeps its row-major form only where the library (or the plain kernels of the untimed check) reads it
+        ops.many_rows = "library" if args.library_products else ("measure" if args.measured_products else "own")
+        ops.rows_cfg = args.rows_cfg
+        before = torch.cuda.memory_allocated()
+        m = random_model("Qwen3ForCausalLM", Qwen3Config.from_dict(conf), args.seed, args.dtype, "cuda:0",
+                         args.context, ops=ops)
+        gb = (torch.cuda.memory_allocated() - before) / 1e9
+        torch.cuda.synchronize()
+        print(f"[bench] model with {conf['num_hidden_layers']} layers of {conf['hidden_size']} on the device in "
+              f"{time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+        pages = max_batch * ((longest + outputs + 64 + page - 1) // page) + (args.prefill_tokens + page - 1) // page + 8
+        e = LLMEngine.from_model(m, max_model_len=args.context, page_size=page, num_kv_blocks=pages,
+                                 max_num_seqs=max_batch, max_num_batched_tokens=budget)
+        return m, e, gb
+
+    def prefill_steps(batch, prompt_len):
+        """Steps in which the prompts are taken in; those taken in first decode meanwhile."""
+        return (batch * prompt_len + budget - 1) // budget + 1
+
+    def decode_run(engine, conf, batch, steps, warmup, prompt_len):
+        """Prefill ``batch`` prompts, then time ``steps`` decode steps after ``warmup`` untimed ones.
+        Returns (seconds, tokens of context a step reads on average, fraction of the HBM peak)."""
+        vocab = conf["vocab_size"]
         # (the margin keeps every request alive through the timed steps)
-        params = SamplingParams(max_tokens=steps + warmup + prefill_steps(batch) + 16, temperature=0.0,
+        params = SamplingParams(max_tokens=steps + warmup + prefill_steps(batch, prompt_len) + 16, temperature=0.0,
                                 ignore_eos=True)
         for _ in range(batch):
-            engine.add_request([rng.randrange(vocab) for _ in range(args.prompt_len)], params)
+            engine.add_request([rng.randrange(vocab) for _ in range(prompt_len)], params)
         while engine.scheduler.waiting:
             engine.step()
         for _ in range(warmup):
@@ -145,45 +160,72 @@ def main():
         assert len(engine.scheduler.running) == batch, "a request ended inside the timed steps"
         while not engine.is_finished():
             engine.step()
-        return dt, (ctx0 + ctx1) / 2.0
+        ctx = (ctx0 + ctx1) / 2.0
+        n_layers = conf["num_hidden_layers"]
+        nbytes = weight_bytes(conf, n_layers, elem) + ctx * kv_bytes_per_token(conf, n_layers, elem)
+        return dt, ctx, nbytes / (dt / steps) / HBM_PEAK
 
-    if args.no_decode:
-        dt, ctx_tokens = float("nan"), 0.0
-    else:
-        dt, ctx_tokens = decode_run(args.batch, args.steps, args.warmup)
-    ms_step = dt / args.steps * 1e3
-    value = args.batch * args.steps / dt
-    step_bytes = weight_bytes(cfg_json, layers, elem) + ctx_tokens * kv_bytes_per_token(cfg_json, layers, elem)
-    achieved = step_bytes / (dt / args.steps)
+    def prefill_run(engine, conf, tokens):
+        """One prompt of ``tokens`` tokens in one step: (median of five, best) in seconds, after one
+        untimed run, and the fraction of the matrix cores' peak that the median makes."""
+        vocab = conf["vocab_size"]
 
-    # prefill of one prompt in one step
-    def prefill_once():
-        engine.add_request([rng.randrange(vocab) for _ in range(args.prefill_tokens)],
-                           SamplingParams(max_tokens=1, ignore_eos=True))
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        engine.step()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t
-        assert engine.is_finished()
-        return dt
-    if args.no_prefill:
-        pre = pre_best = float("nan")
-    else:
-        prefill_once()
-        runs = sorted(prefill_once() for _ in range(5))
-        pre, pre_best = runs[2], runs[0]          # the median is what is reported, the best beside it
-    T = args.prefill_tokens
-    pre_flops = step_flops(cfg_json, layers, T, T * (T + 1) / 2.0, 1)
+        def once():
+            engine.add_request([rng.randrange(vocab) for _ in range(tokens)], SamplingParams(max_tokens=1, ignore_eos=True))
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            engine.step()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            assert engine.is_finished()
+            return dt
+        once()
+        runs = sorted(once() for _ in range(5))
+        flops = step_flops(conf, conf["num_hidden_layers"], tokens, tokens * (tokens + 1) / 2.0, 1)
+        return runs[2], runs[0], flops / runs[2] / MFMA_PEAK[dkey]
 
     points = {}
+    most = args.batch if args.no_points else max(64, args.batch)
+    model, engine, weight_gb = make_engine(cfg_json, most, args.prompt_len if args.no_points else args.context - 192,
+                                           max(args.steps + args.warmup, 128) + 64)
+    vocab = cfg.vocab_size
+
+    if args.no_decode:
+        dt, ctx_tokens, frac = float("nan"), 0.0, float("nan")
+    else:
+        dt, ctx_tokens, frac = decode_run(engine, cfg_json, args.batch, args.steps, args.warmup, args.prompt_len)
+    ms_step = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    achieved = frac * HBM_PEAK
+
+    # prefill of one prompt in one step
+    T = args.prefill_tokens
+    if args.no_prefill:
+        pre = pre_best = pre_frac = float("nan")
+    else:
+        pre, pre_best, pre_frac = prefill_run(engine, cfg_json, T)
+
     if not args.no_points:
+        n = min(args.steps, 32)
         for b in (1, 64):
-            n = min(args.steps, 32)
-            d, ctx = decode_run(b, n, 4)
+            d, _, f = decode_run(engine, cfg_json, b, n, 4, args.prompt_len)
             points[f"decode_b{b}"] = round(b * n / d, 2)
-            nbytes = weight_bytes(cfg_json, layers, elem) + ctx * kv_bytes_per_token(cfg_json, layers, elem)
-            points[f"decode_b{b}_hbm_frac"] = round(nbytes / (d / n) / HBM_PEAK, 4)
+            points[f"decode_b{b}_hbm_frac"] = round(f, 4)
+        # every one of the 128 output tokens of 128-token prompts (the first token comes with the
+        # prompt's last step); once untimed before, because the steps past 256 tokens are recorded anew
+        for b in (1, 8, 64):
+            decode_run(engine, cfg_json, b, 127, 0, 128)
+            d, _, f = decode_run(engine, cfg_json, b, 127, 0, 128)
+            points[f"decode_b{b}_128out"] = round(b * 127 / d, 2)
+            points[f"decode_b{b}_128out_hbm_frac"] = round(f, 4)
+        # contexts that end at the limit (4,096 tokens unless --context says otherwise): prompts as
+        # long as leaves every request room for the steps it takes while the others' prompts come in
+        for b in (8, 64):
+            long_prompt = args.context - (n + 4 + prefill_steps(b, args.context) + 16)
+            d, ctx, f = decode_run(engine, cfg_json, b, n, 4, long_prompt)
+            points[f"decode_b{b}_ctx{args.context}"] = round(b * n / d, 2)
+            points[f"decode_b{b}_ctx{args.context}_hbm_frac"] = round(f, 4)
+            points[f"decode_b{b}_ctx{args.context}_mean_context"] = round(ctx / b, 1)
 
     def logit_check():
         """Outside every timed region: the logits of the last prompt token and of a few decoded
@@ -226,6 +268,24 @@ def main():
                 "argmax_same_as_fp32": same, "rows": int(tuned.shape[0])}
     check = logit_check() if (args.dtype == "bfloat16" and not args.no_check) else {}
 
+    # the layer sizes of the larger models of the family: decode at batch 8 and the prefill of 2,048 tokens
+    if not args.no_points and not args.no_other_shapes and not args.shape and not args.layers:
+        del model, engine
+        for tag in ("14b", "32b"):
+            gc.collect()
+            torch.cuda.empty_cache()
+            with open(os.path.join(ROOT, "configs", f"qwen3_{tag}_shape.json")) as fh:
+                conf = json.load(fh)
+            m2, e2, _ = make_engine(conf, 8, args.prompt_len, 128)
+            n = min(args.steps, 32)
+            d, _, f = decode_run(e2, conf, 8, n, 4, args.prompt_len)
+            points[f"qwen3_{tag}_decode_b8"] = round(8 * n / d, 2)
+            points[f"qwen3_{tag}_decode_b8_hbm_frac"] = round(f, 4)
+            p_med, _, p_frac = prefill_run(e2, conf, T)
+            points[f"qwen3_{tag}_prefill_{T}"] = round(T / p_med, 1)
+            points[f"qwen3_{tag}_prefill_{T}_mfma_frac"] = round(p_frac, 4)
+            del m2, e2
+
     out = {
         "metric": f"decode tok/s @ batch {args.batch} ({shape_name}, {dkey}, random weights)",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
@@ -239,7 +299,7 @@ def main():
                    "vocab_size": cfg.vocab_size, "prompt_len": args.prompt_len,
                    "page_size": page, "prefill_tokens": T, "weights_gb_on_device": round(weight_gb, 2)},
         "prefill": {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
-                    "frac": round(pre_flops / pre / MFMA_PEAK[dkey], 4), "of": "median of 5",
+                    "frac": round(pre_frac, 4), "of": "median of 5",
                     "best_ms": round(pre_best * 1e3, 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4)},
