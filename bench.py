@@ -12,7 +12,11 @@ the HBM peak that the bytes a step has to read make of its time):
   decode_b{1,8,64}_128out                    all 128 output tokens of 128-token prompts
   decode_b{8,64}_ctx4096                     contexts that end at 4,096 tokens
   qwen3_14b_*, qwen3_32b_*                   decode at batch 8 and the prefill of 2,048 tokens at
-                                             the layer sizes of the larger models (configs/)
+                                             the layer sizes of the larger models (configs/), and
+                                             one serving workload each through the scheduler: 32
+                                             requests with prompts of 64 to 2,048 tokens in portions
+                                             beside decoding (14B), 64 requests that join while the
+                                             others are served (32B)
 """
 import argparse
 import json
@@ -66,6 +70,7 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip every point beside the headline")
     ap.add_argument("--no-other-shapes", action="store_true", help="skip the points at the layer sizes of the larger models")
+    ap.add_argument("--no-workloads", action="store_true", help="skip the two serving workloads at those sizes")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiles)")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement (for profiles)")
     ap.add_argument("--own-products", action="store_true",
@@ -109,10 +114,11 @@ def main():
     budget = max(args.prefill_tokens, 2048)
     rng = random.Random(args.seed)
 
-    def make_engine(conf, max_batch, longest, outputs):
-        """A model of ``conf`` with random weights and an engine whose cache holds ``max_batch``
-        requests of ``longest`` prompt tokens and ``outputs`` new ones beside one prompt of
-        --prefill-tokens."""
+    def make_engine(conf, max_batch, longest, outputs, context=None):
+        """A model of ``conf`` with random weights (for up to ``context`` positions) and an engine
+        whose cache holds ``max_batch`` requests of ``longest`` prompt tokens and ``outputs`` new
+        ones beside one prompt of --prefill-tokens."""
+        context = context or args.context
         t0 = time.time()
         ops = HipOps("cuda:0")
         # which kernel multiplies more than 128 rows is settled before the weights are loaded: a matrix
@@ -121,13 +127,13 @@ def main():
         ops.rows_cfg = args.rows_cfg
         before = torch.cuda.memory_allocated()
         m = random_model("Qwen3ForCausalLM", Qwen3Config.from_dict(conf), args.seed, args.dtype, "cuda:0",
-                         args.context, ops=ops)
+                         context, ops=ops)
         gb = (torch.cuda.memory_allocated() - before) / 1e9
         torch.cuda.synchronize()
         print(f"[bench] model with {conf['num_hidden_layers']} layers of {conf['hidden_size']} on the device in "
               f"{time.time() - t0:.1f} s", file=sys.stderr, flush=True)
         pages = max_batch * ((longest + outputs + 64 + page - 1) // page) + (args.prefill_tokens + page - 1) // page + 8
-        e = LLMEngine.from_model(m, max_model_len=args.context, page_size=page, num_kv_blocks=pages,
+        e = LLMEngine.from_model(m, max_model_len=context, page_size=page, num_kv_blocks=pages,
                                  max_num_seqs=max_batch, max_num_batched_tokens=budget)
         return m, e, gb
 
@@ -268,6 +274,39 @@ def main():
                 "argmax_same_as_fp32": same, "rows": int(tuned.shape[0])}
     check = logit_check() if (args.dtype == "bfloat16" and not args.no_check) else {}
 
+    def serving_workload(tag, m):
+        """The two serving workloads that go with the larger shapes, through the scheduler (output
+        tokens a second over the whole run, prompts included in the time).  14B: 32 requests at
+        once, prompts of 64 to 2,048 tokens taken in in portions under a budget of 2,048 tokens
+        a step beside the decoding of the others, 256 new tokens each, up to 8,192 positions.
+        32B: 64 requests of 512 prompt tokens and 512 new ones that join eight steps apart while
+        the earlier ones are served, up to 16,384 positions, the cache sized from the memory that
+        the weights leave.  Every request has to come back with its full length and the cache
+        whole."""
+        from tiny_llm_infer_amd.cli import _generate_arriving, make_benchmark_requests
+        if tag == "14b":
+            name, reqs = "mixed_32_requests", make_benchmark_requests(32, 64, 2048, 256, 256, 10000, m.spec.vocab_size, 7)
+            e = LLMEngine.from_model(m, max_model_len=8192, page_size=page, max_num_seqs=32, max_num_batched_tokens=2048,
+                                     num_kv_blocks=32 * ((2048 + 256 + page - 1) // page) + 8)
+            run = lambda: e.generate([q for q, _ in reqs], [sp for _, sp in reqs])
+        else:
+            name, reqs = "continuous_64_requests", make_benchmark_requests(64, 512, 512, 512, 512, 10000, m.spec.vocab_size, 9)
+            e = LLMEngine.from_model(m, max_model_len=16384, page_size=page, max_num_seqs=64, max_num_batched_tokens=2048,
+                                     num_kv_blocks=0, gpu_memory_utilization=0.9)
+            run = lambda: _generate_arriving(e, reqs, 8)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        results = run()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        assert [len(r.token_ids) for r in results] == [sp.max_tokens for _, sp in reqs], "a request came back short"
+        e.runner.cache.check()
+        assert e.runner.cache.free_pages() == e.runner.cache.pages_per_group() and e.is_finished()
+        st = e.stats()
+        out = sum(len(r.token_ids) for r in results)
+        return {f"qwen3_{tag}_{name}_tok_s": round(out / dt, 1), f"qwen3_{tag}_{name}_steps": st["steps"],
+                f"qwen3_{tag}_{name}_preemptions": st["preemptions"], f"qwen3_{tag}_{name}_cache_pages": st["pages"]}
+
     # the layer sizes of the larger models of the family: decode at batch 8 and the prefill of 2,048 tokens
     if not args.no_points and not args.no_other_shapes and not args.shape and not args.layers:
         del model, engine
@@ -276,7 +315,7 @@ def main():
             torch.cuda.empty_cache()
             with open(os.path.join(ROOT, "configs", f"qwen3_{tag}_shape.json")) as fh:
                 conf = json.load(fh)
-            m2, e2, _ = make_engine(conf, 8, args.prompt_len, 128)
+            m2, e2, _ = make_engine(conf, 8, args.prompt_len, 128, context=16384)
             n = min(args.steps, 32)
             d, _, f = decode_run(e2, conf, 8, n, 4, args.prompt_len)
             points[f"qwen3_{tag}_decode_b8"] = round(8 * n / d, 2)
@@ -284,7 +323,12 @@ def main():
             p_med, _, p_frac = prefill_run(e2, conf, T)
             points[f"qwen3_{tag}_prefill_{T}"] = round(T / p_med, 1)
             points[f"qwen3_{tag}_prefill_{T}_mfma_frac"] = round(p_frac, 4)
-            del m2, e2
+            del e2
+            if not args.no_workloads:
+                gc.collect()
+                torch.cuda.empty_cache()
+                points.update(serving_workload(tag, m2))
+            del m2
 
     out = {
         "metric": f"decode tok/s @ batch {args.batch} ({shape_name}, {dkey}, random weights)",

@@ -879,6 +879,11 @@ def test_products_that_take_the_norm_in(ops, M, hidden):
     assert torch.equal(nc, na) and torch.equal(rc, ra)
 
 
+def test_launch_rules_know_the_chip(ops):
+    assert ops.lib.tli_device_compute_units() == torch.cuda.get_device_properties(0).multi_processor_count
+    assert ops.DECODE_WORKGROUPS == ops.lib.tli_device_compute_units()
+
+
 # ------------------------------------------------------------------ sampling --
 def test_greedy_takes_the_lowest_index_on_ties(ops):
     logits = torch.zeros(3, 5000)

@@ -1674,7 +1674,8 @@ static int launch_prefill(
         // compute unit (long row blocks then come first); else one tile a wave.
         const long blocks1 = (rows + 4 * rq - 1) / (4 * rq) + num_seqs;
         const long blocks2 = (rows + 8 * rq - 1) / (8 * rq) + num_seqs;
-        bool two = head_dim <= 128 && blocks2 * kv_heads * head_tiles >= 512;
+        const long units = tli_compute_units();                   // 256 on MI355X
+        bool two = head_dim <= 128 && blocks2 * kv_heads * head_tiles >= 2 * units;
         // Heads of 64 and 128, while the chip has room for every workgroup at once: the longest
         // workgroups decide the time, and two sets of waves a workgroup walk a workgroup's keys in
         // half the rounds (one workgroup a compute unit then: two tiles a wave where one tile would
@@ -1685,12 +1686,12 @@ static int launch_prefill(
         // so: the lengths are on the device) and slower beyond.
         const bool dma = head_dim == 64 || head_dim == 128;
         const long groups2 = (blocks2 - num_seqs) * kv_heads * head_tiles;
-        bool sets = dma && groups2 <= (direct == 13 ? 256 : 512);
-        if (sets) two = (blocks1 - num_seqs) * kv_heads * head_tiles > 256;
+        bool sets = dma && groups2 <= (direct == 13 ? units : 2 * units);
+        if (sets) two = (blocks1 - num_seqs) * kv_heads * head_tiles > units;
         // rows with keys before them are all about as long: two tiles a wave, which read the keys
         // once for both, already pay when one round of them fills the chip (1,536 rows behind
         // 6,656 keys: a fifth faster than one tile a wave)
-        else if (dma && direct == 13 && groups2 > 256) two = true;
+        else if (dma && direct == 13 && groups2 > units) two = true;
         if (direct == 2) two = false;
         if (direct == 3 || (direct >= 4 && direct <= 7)) two = head_dim <= 128;
         if (direct == 8) two = false;
@@ -1701,7 +1702,7 @@ static int launch_prefill(
         const int rows_per_block = 4 * rq * (two ? 2 : 1);
         const long blocks = (rows + rows_per_block - 1) / rows_per_block + num_seqs;   // upper bound
         if (blocks > 2147483647L) return tli_fail("attention_prefill: too many rows");
-        int pair = two ? 3 : (blocks * kv_heads * head_tiles >= 1024 ? 1 : 2);
+        int pair = two ? 3 : (blocks * kv_heads * head_tiles >= 4 * units ? 1 : 2);
         if (direct >= 4 && direct <= 7) pair = direct - 4;        // measurements: 4..7 force the pairing mode, two tiles
         if (direct == 8) pair = 3;                                // one tile, long blocks first
         if (sets && !(direct >= 4 && direct <= 7)) pair = 3;      // (one workgroup a compute unit: long blocks first)

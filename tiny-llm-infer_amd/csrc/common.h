@@ -12,6 +12,13 @@ typedef uint16_t bf16_t;   // bfloat16 storage: the upper 16 bits of a float
 #define TLI_F32 0
 #define TLI_BF16 1
 
+// The chip that the launch rules deal work out to.  Workgroups go round the dies in turn, and
+// every die has an L2 cache of its own.  The runtime reports the compute units of a device but
+// not its dies, so their number is the one constant: 8 on MI355X, of 32 compute units each.
+#define TLI_DIES 8
+int tli_compute_units();                     // of the current device, asked once (256 on MI355X)
+static inline int tli_units_a_die() { return tli_compute_units() / TLI_DIES; }
+
 extern "C" const char* tli_last_error();
 int tli_fail(const char* fmt, ...);          // records a message, returns 1
 int tli_check_launch(const char* what);      // hipGetLastError -> message

@@ -67,7 +67,7 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
     // slice of x is rows a power of two apart, which all lie in one channel of the L2
     // cache, and workgroups in step would all wait for that one channel.  (Workgroups go
     // round the eight dies in turn, so neighbours on a die are blockIdx.x / 8 apart.)
-    const int rot = step_begin < step_end ? (blockIdx.x / 8) % (step_end - step_begin) : 0;
+    const int rot = step_begin < step_end ? (blockIdx.x / TLI_DIES) % (step_end - step_begin) : 0;
     auto at = [&](int step) { return step + rot < step_end ? step + rot : step + rot - (step_end - step_begin); };
 
     f32x4 acc[RT][MT];
@@ -301,7 +301,7 @@ static int launch_mid(const bf16_t* x, const bf16_t* w, void* y, float* part, in
 // column tiles a wave once that still leaves about 192 workgroups, else one; k is cut into
 // ranges until there are about 192 workgroups (tli_gemm_mid_bf16 then keeps the workgroups
 // at no more than one a compute unit where it can).
-static int mid_tiles_per_wave(int N, int gated) { return gated || (N + 15) / 16 >= 8 * 192 ? 2 : 1; }
+static int mid_tiles_per_wave(int N, int gated) { return gated || (N + 15) / 16 >= 8 * (3 * tli_compute_units() / 4) ? 2 : 1; }
 
 // How a product of this shape is dealt out: column tiles a wave and ranges of k.  As many
 // workgroups as fit the 256 compute units once (more cost more than they bring, measured at
@@ -312,7 +312,8 @@ static int mid_tiles_per_wave(int N, int gated) { return gated || (N + 15) / 16 
 // groups in 3 ranges).  A range keeps at least two slices of 128.  Gated products: see below.
 static void mid_plan(int N, int K, int gated, int* tiles_a_wave, int* waves_a_group, int* ranges) {
     const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
-    auto ranges_for = [&](int groups) { return max(1, min(min(256 / max(groups, 1), k_steps / 2), 16)); };
+    const int units = tli_compute_units(), most = 3 * units / 4;      // 256 and 192 on MI355X
+    auto ranges_for = [&](int groups) { return max(1, min(min(units / max(groups, 1), k_steps / 2), 16)); };
     int rt = mid_tiles_per_wave(N, gated), waves = 4;
     if (gated) {
         // a wave takes one pair of gate and up tiles; three to eight waves a workgroup, whichever
@@ -324,15 +325,15 @@ static void mid_plan(int N, int K, int gated, int* tiles_a_wave, int* waves_a_gr
         waves = 8;
         for (int w = 3; w <= 8; ++w) {
             const int groups = (pairs + w - 1) / w;
-            if (groups <= 256 && groups > best) {
+            if (groups <= units && groups > best) {
                 best = groups;
                 waves = w;
             }
         }
     }
     int groups = (n_tiles + waves * rt - 1) / (waves * rt);
-    int splits = groups >= 192 ? 1 : ranges_for(groups);
-    if (!gated && rt == 1 && groups * splits < 192) {
+    int splits = groups >= most ? 1 : ranges_for(groups);
+    if (!gated && rt == 1 && groups * splits < most) {
         const int groups2 = (n_tiles + 7) / 8, splits2 = ranges_for(groups2);
         if (groups2 * splits2 > groups * splits) {
             rt = 2;
@@ -381,7 +382,7 @@ extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* p
         if (splits != planned) {                                      // (ranges forced by the caller)
             rt = mid_tiles_per_wave(N, gated);
             const int groups = ((N + 15) / 16 + waves * rt - 1) / (waves * rt);
-            if (!gated && rt == 1 && (long)groups * splits > 256) rt = 2;
+            if (!gated && rt == 1 && (long)groups * splits > tli_compute_units()) rt = 2;
         }
         cfg = 200 + 10 * rt + waves;
     }

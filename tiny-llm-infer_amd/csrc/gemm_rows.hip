@@ -94,32 +94,32 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
     bf16_t* xs = reinterpret_cast<bf16_t*>(xs_raw) + (size_t)kg * 2 * SLICE;     // [2][ROWS][128] for this set, rows swizzled
     const int k_steps = (K + 127) / 128;
     const int n_tiles = (N + 15) / 16;
-    // Workgroup i runs on die i % 8.  A die takes the row blocks in chunks of 2,048 rows: all
+    // Workgroup i runs on die i % TLI_DIES.  A die takes the row blocks in chunks of 2,048 rows: all
     // row blocks of a chunk for one column group, then for the next column group of the die, and
     // so on; then the next chunk (the x rows of a chunk and a W panel stay in its L2 meanwhile).
     constexpr int CHUNK = 2048 / ROWS;
     const int row_blocks = (M + ROWS - 1) / ROWS;
     const int col_groups = (n_tiles + RT * WAVES - 1) / (RT * WAVES);
-    const int groups_a_die = (col_groups + 7) / 8;
-    const int die = blockIdx.x % 8, turn = blockIdx.x / 8;
+    const int groups_a_die = (col_groups + TLI_DIES - 1) / TLI_DIES;
+    const int die = blockIdx.x % TLI_DIES, turn = blockIdx.x / TLI_DIES;
     const int chunk = turn / (CHUNK * groups_a_die), in_chunk = turn % (CHUNK * groups_a_die);
     const int chunk_rows = min(CHUNK, row_blocks - chunk * CHUNK);      // row blocks of this chunk (the last may be short)
     // The column groups that do not make a whole round of the eight dies are dealt out by row
     // blocks instead, so that every die gets as many workgroups as the others (5,120 columns are
     // 20 groups of 256: two for every die, and of the other four each die takes half the row
     // blocks of one).
-    const int whole = col_groups / 8, left = col_groups % 8;
+    const int whole = col_groups / TLI_DIES, left = col_groups % TLI_DIES;
     int row_block, col_group;
     if (in_chunk < whole * chunk_rows) {
         row_block = chunk * CHUNK + in_chunk % chunk_rows;
-        col_group = (in_chunk / chunk_rows) * 8 + die;
+        col_group = (in_chunk / chunk_rows) * TLI_DIES + die;
     } else {
-        const int share = (left * chunk_rows + 7) / 8;                   // workgroups of the left-over groups a die takes
+        const int share = (left * chunk_rows + TLI_DIES - 1) / TLI_DIES; // workgroups of the left-over groups a die takes
         const int j = in_chunk - whole * chunk_rows;
         const int at = die * share + j;                                   // index among the left-over groups' workgroups
         if (j >= share || at >= left * chunk_rows) return;                // (the grid is rounded up)
         row_block = chunk * CHUNK + at % chunk_rows;
-        col_group = whole * 8 + at / chunk_rows;
+        col_group = whole * TLI_DIES + at / chunk_rows;
     }
     x += (size_t)row_block * ROWS * K;
     const int n_out = GATED ? N / 2 : N;
@@ -352,7 +352,7 @@ static int launch_rows(const bf16_t* x, const bf16_t* w, bf16_t* y, float* part,
     const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
     const long col_groups = (n_tiles + RT * WAVES - 1) / (RT * WAVES), row_blocks = (M + MT * 16 - 1) / (MT * 16);
     const long chunk = 2048 / (MT * 16);                     // as the kernel deals the row blocks out
-    const long blocks = (col_groups + 7) / 8 * 8 * ((row_blocks + chunk - 1) / chunk * chunk);
+    const long blocks = (col_groups + TLI_DIES - 1) / TLI_DIES * TLI_DIES * ((row_blocks + chunk - 1) / chunk * chunk);
     if (blocks > 2147483647L) return tli_fail("gemm_rows: too many workgroups");
     const int slices_per_split = (k_steps + splits - 1) / splits;
     if (KG == 2 && (slices_per_split % 2 || k_steps % slices_per_split))
@@ -391,7 +391,8 @@ extern "C" int tli_gemm_rows_splits(int M, int N, int K) {
     const long col_groups = ((N + 15) / 16 + 15) / 16, row_blocks = (M + 127) / 128;
     const int k_steps = (K + 127) / 128;
     int splits = 1;
-    while (col_groups * row_blocks * splits < 192 && splits * 2 * 4 <= k_steps && splits < 16) splits *= 2;
+    const long enough = 3L * tli_compute_units() / 4;
+    while (col_groups * row_blocks * splits < enough && splits * 2 * 4 <= k_steps && splits < 16) splits *= 2;
     return splits;
 }
 
@@ -411,13 +412,14 @@ static int rows_pick(int M, int N, int K, int splits, int gated) {
     const long n_tiles = (N + 15) / 16, row_blocks = (M + 127) / 128;
     // workgroups of the busiest of the eight dies (each has 32 compute units), in units of one
     // workgroup alone on its compute unit
-    auto a_die = [&](long tiles_a_group) { return ((n_tiles + tiles_a_group - 1) / tiles_a_group * row_blocks * splits + 7) / 8; };
+    const long units = tli_units_a_die();          // compute units of a die (32)
+    auto a_die = [&](long tiles_a_group) { return ((n_tiles + tiles_a_group - 1) / tiles_a_group * row_blocks * splits + TLI_DIES - 1) / TLI_DIES; };
     auto shared = [&](long wgs) {                  // four waves a workgroup: two workgroups share a compute unit
-        if (wgs <= 32) return 1.0;
-        const long full = wgs / 64, rem = wgs % 64;
-        return 1.75 * (double)full + (rem == 0 ? 0.0 : rem <= 32 ? 1.0 : 1.75);
+        if (wgs <= units) return 1.0;
+        const long full = wgs / (2 * units), rem = wgs % (2 * units);
+        return 1.75 * (double)full + (rem == 0 ? 0.0 : rem <= units ? 1.0 : 1.75);
     };
-    auto alone = [&](long wgs) { return (double)((wgs + 31) / 32); };     // eight waves: one workgroup a compute unit
+    auto alone = [&](long wgs) { return (double)((wgs + units - 1) / units); };     // eight waves: one workgroup a compute unit
     const long k_steps = (K + 127) / 128, per = (k_steps + splits - 1) / splits;
     const double cost2 = shared(a_die(16)) * 256.0, cost4 = shared(a_die(12)) * 192.0 * 1.06;
     const double cost3 = alone(a_die(32)) * 512.0 * 0.84, cost6 = alone(a_die(16)) * 256.0 * 0.88;

@@ -350,7 +350,7 @@ static int pick_skinny(const bf16_t* x, const bf16_t* w, void* y, int M, int N, 
     // cfg 0: by shape.  Narrow outputs get one 16-column tile per workgroup so that
     // even N = 4096 gives 256 workgroups; wide outputs share x over two tiles.
     const long tiles = (N + 15) / 16;
-    if (cfg == 0) cfg = tiles <= 256 ? 18 : (tiles < 1024 ? 28 : 24);
+    if (cfg == 0) cfg = tiles <= tli_compute_units() ? 18 : (tiles < 4 * tli_compute_units() ? 28 : 24);
     if (tiled == 2 && cfg < 20) cfg = 24;          // gated needs pairs of row tiles
     switch (cfg) {
         case 14: return launch_skinny<1, MT, 4>(x, w, y, M, N, K, y_dtype, tiled, s);
@@ -426,7 +426,7 @@ extern "C" int tli_gemm_skinny_fused_bf16(const void* x, const void* w, void* y,
     const bf16_t* xp = (const bf16_t*)x;
     const bf16_t* wp = (const bf16_t*)w;
     const long tiles = (N + 15) / 16;
-    if (cfg == 0) cfg = tiles <= 256 ? 18 : (tiles < 1024 ? 28 : 24);
+    if (cfg == 0) cfg = tiles <= tli_compute_units() ? 18 : (tiles < 4 * tli_compute_units() ? 28 : 24);
     if (gated && cfg < 20) cfg = 24;
     switch (cfg) {
         case 14: return launch_skinny_fused<1, 4>(xp, wp, (bf16_t*)y, M, N, K, gated, f, s);

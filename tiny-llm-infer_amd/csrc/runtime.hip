@@ -22,3 +22,19 @@ int tli_check_launch(const char* what) {
 }
 
 extern "C" int tli_abi_version() { return 1; }
+
+int tli_compute_units() {
+    static int units = 0;
+    if (units == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n >= TLI_DIES)
+            units = n;
+        else
+            units = 256;                     // (no device to ask: the chip this library is written for)
+        (void)hipGetLastError();
+    }
+    return units;
+}
+
+extern "C" int tli_device_compute_units() { return tli_compute_units(); }

@@ -70,6 +70,7 @@ def load_library():
     P, I, F = c_void_p, c_int, c_float
     sigs = {
         "tli_abi_version": [],
+        "tli_device_compute_units": [],
         "tli_embed": [P, P, P, I, I, I, I, P],
         "tli_feed_tokens": [P, P, P, I, I, P],
         "tli_add_rmsnorm": [P, P, P, P, P, I, I, I, F, I, I, P],
@@ -135,7 +136,8 @@ class HipOps:
     MID_ROWS_FROM = 17           # from this many rows the x-sharing kernel multiplies,
     MID_ROWS_TO = 128            # up to this many
     DECODE_WORKGROUPS = 256      # aim of the decode attention's key splitting: one workgroup a compute unit (measured
-                                 # against 128, 192 and 512 at batch 1 to 64 and 128 to 30,000 keys: up to 10% over 512)
+                                 # against 128, 192 and 512 at batch 1 to 64 and 128 to 30,000 keys: up to 10% over 512);
+                                 # set to what the device reports when the library is loaded
     DECODE_SPLIT_KEYS = 512      # a split walks at least this many keys (128, 256 and 1024 measured: no better)
     # A step of prompt portions whose first sequences decode: those go to the decode kernel when the
     # longest of them has this many times the keys of the longest portion, or as many keys when they
@@ -151,6 +153,8 @@ class HipOps:
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible to torch; this engine has no CPU path")
         self.lib = load_library()
+        with torch.cuda.device(self.device):
+            self.DECODE_WORKGROUPS = int(self.lib.tli_device_compute_units())
         self.force_plain = False     # tests: run the plain attention kernel for bfloat16 too
         self.plain_products = False  # every matrix product through the plain kernel
         self.separate_norms = False  # tests: decode steps run their norms as kernels of their own
