@@ -134,5 +134,46 @@ def build_library(force: bool = False, verbose: bool = True) -> str:
     return lib
 
 
+# ---- the C ABI of the engine (capi/): host code only, a Python interpreter embedded ----------
+CAPI = os.path.join(os.path.dirname(CSRC), "capi")
+ENGINE_LIB = "libtli_engine.so"
+
+
+def find_engine_api() -> Optional[str]:
+    lib = os.path.join(CAPI, ENGINE_LIB)
+    srcs = [os.path.join(CAPI, f) for f in ("tli_engine.cpp", "tli_engine.h")]
+    if os.path.exists(lib) and all(os.path.getmtime(s) <= os.path.getmtime(lib) for s in srcs):
+        return lib
+    return None
+
+
+def build_engine_api(force: bool = False, verbose: bool = True) -> str:
+    """Compile ``capi/tli_engine.cpp`` (the engine for C and C++ programs) against this
+    interpreter's headers and library; returns the path of ``libtli_engine.so``."""
+    import sysconfig
+    if not force:
+        lib = find_engine_api()
+        if lib:
+            return lib
+    cxx = shutil.which("g++") or shutil.which("c++") or shutil.which("clang++")
+    if not cxx:
+        raise BuildError("no C++ compiler was found for the engine's C ABI (g++, c++ or clang++)")
+    include = sysconfig.get_paths()["include"]
+    libdir = sysconfig.get_config_var("LIBDIR") or ""
+    version = sysconfig.get_config_var("LDVERSION") or sysconfig.get_python_version()
+    lib = os.path.join(CAPI, ENGINE_LIB)
+    tmp = lib + f".tmp{os.getpid()}"
+    cmd = [cxx, "-O2", "-std=c++17", "-shared", "-fPIC", f"-I{include}", os.path.join(CAPI, "tli_engine.cpp"),
+           "-o", tmp, f"-L{libdir}", f"-lpython{version}", "-ldl", f"-Wl,-rpath,{libdir}"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise BuildError(f"building {lib} failed:\n{proc.stdout}")
+    os.replace(tmp, lib)
+    if verbose:
+        print(f"[tli build] built {lib}", file=sys.stderr, flush=True)
+    return lib
+
+
 if __name__ == "__main__":
     print(build_library(force="--force" in sys.argv))
+    print(build_engine_api(force="--force" in sys.argv))
