@@ -754,6 +754,48 @@ def _raw_projections_case(ops, case):
     close(out2, want, dtype, "attention through two kernels")
 
 
+@pytest.mark.parametrize("hd,page,rotation,norms", [(128, 16, True, True), (64, 8, True, True), (256, 32, False, True),
+                                                    (128, 64, True, False), (64, 16, False, False)])
+def test_keys_and_values_of_portions_in_one_pass(ops, hd, page, rotation, norms):
+    """Prompt portions write their keys (normed, rotated) and values into the pages with one
+    kernel: the cache it leaves is bit for bit what the two kernels (keys; values) leave, for
+    portions that start and end inside a page, single rows among them, and nothing else in the
+    cache is touched."""
+    heads, kv_heads = 4, 2
+    seq_lens, new_counts = [137, 40, 9, 70, 300], [130, 40, 1, 3, 77]
+    dtype = torch.bfloat16
+    num_pages = sum((n + page - 1) // page for n in seq_lens) + 3
+    step, tables, pos, seq = make_step(seq_lens, new_counts, page, num_pages, 13, kv_heads, hd, dtype)
+    T = len(pos)
+    qkv = rnd((T, (heads + 2 * kv_heads) * hd), dtype, 31).to(DEV)
+    qkv[5, (heads + kv_heads) * hd + 7] = float("inf")                  # made finite on its way in
+    kn = ((1 + rnd((hd,), torch.float32, 23, 0.2)).to(DEV), 3e-6) if norms else None
+    rotary = None
+    if rotation:
+        ang = torch.arange(512, dtype=torch.float64)[:, None] * (10000.0 ** (-2.0 * torch.arange(hd // 2, dtype=torch.float64) / hd))[None, :]
+        rotary = (torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV), hd)
+    k0, v0 = step.cache.k.clone(), step.cache.v.clone()
+    assert ops.qkv_to_cache(qkv, step, step.cache, heads, kv_heads, hd, None, kn, rotary, queries=False) is None
+    k1, v1 = step.cache.k.clone(), step.cache.v.clone()
+    step.cache.k.copy_(k0)
+    step.cache.v.copy_(v0)
+    ops.separate_cache_writes = True
+    try:
+        ops.qkv_to_cache(qkv, step, step.cache, heads, kv_heads, hd, None, kn, rotary, queries=False)
+    finally:
+        ops.separate_cache_writes = False
+    assert torch.equal(k1, step.cache.k) and torch.equal(v1, step.cache.v)
+    written = torch.zeros((num_pages, page), dtype=torch.bool)
+    for r in range(T):
+        written[int(tables[seq[r], pos[r] // page]), pos[r] % page] = True
+    untouched = ~written[:, None, :, None].expand_as(k0.cpu())
+    assert torch.equal(k1.cpu()[untouched], k0.cpu()[untouched]) and not torch.equal(k1, k0)
+    untouched_v = ~written[:, None, None, :].expand_as(v0.cpu())
+    assert torch.equal(v1.cpu()[untouched_v], v0.cpu()[untouched_v])
+    p5 = int(tables[seq[5], pos[5] // page])
+    assert float(v1[p5, 0, 7, pos[5] % page]) == 0.0
+
+
 @pytest.mark.parametrize("hd,counts", [(128, [1, 1]), (128, [20, 1]), (48, [5, 1])])
 def test_values_enter_the_cache_finite(ops, hd, counts):
     """Infinities and NaNs among the values become 0 on their way into the cache (every

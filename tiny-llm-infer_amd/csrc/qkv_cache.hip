@@ -238,6 +238,145 @@ __global__ void values_to_cache_kernel(
     }
 }
 
+// Keys and values of a step's rows into the cache in one pass, for steps that bring many rows a
+// sequence and heads of 64, 128 or 256 (EPL = head_dim / 64 elements a lane): a workgroup takes
+// up to G consecutive positions of one sequence that share a page, and one kv head.  Its four
+// waves norm and rotate the keys of those positions, a row a wave at a time (as
+// qkv_to_cache_wide_kernel does), and its threads then write the values as runs of slots (as
+// values_to_cache_kernel does).  One launch instead of two: a kernel that follows another costs
+// some 4 us on this chip however little it does.  grid (groups upper bound, kv_heads).
+template <int EPL, int G>
+__global__ void __launch_bounds__(QKV_WAVES * TLI_WAVE)
+keys_values_to_cache_kernel(
+    const bf16_t* __restrict__ qkv, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
+    const int* __restrict__ row_start, const int* __restrict__ seq_start, int num_seqs,
+    const int* __restrict__ tables, int table_width, int page_size, int num_pages, int heads, int kv_heads,
+    const float* __restrict__ k_norm_w, float k_eps, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, int table_positions) {
+    constexpr int HD = 64 * EPL;
+    int grp = blockIdx.x, seq = 0, start = 0, first_row = 0, n_rows = 0;
+    for (; seq < num_seqs; ++seq) {
+        first_row = row_start[seq];
+        n_rows = row_start[seq + 1] - first_row;
+        start = seq_start[seq];
+        const int groups = n_rows > 0 ? (start + n_rows - 1) / G - start / G + 1 : 0;
+        if (grp < groups) break;
+        grp -= groups;
+    }
+    if (seq >= num_seqs) return;
+    const int g0 = start / G + grp;
+    const int p_lo = max(start, g0 * G), p_hi = min(start + n_rows, (g0 + 1) * G);
+    const int n = p_hi - p_lo;
+    const int page = tables[(size_t)seq * table_width + p_lo / page_size];
+    if (page < 0 || page >= num_pages) return;
+    const int slot0 = p_lo % page_size, kvh = blockIdx.y;
+    const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE;
+    const size_t stride = (size_t)(heads + 2 * kv_heads) * HD;
+    const bf16_t* rows = qkv + (size_t)(first_row + p_lo - start) * stride;
+
+    // keys: position p_lo + j by wave j % 4
+    const bf16_t* ksrc = rows + (size_t)(heads + kvh) * HD + lane * EPL;
+    bf16_t* kdst = k_cache + (((size_t)page * kv_heads + kvh) * page_size + slot0) * HD + lane * EPL;
+    for (int j = wave; j < n; j += QKV_WAVES) {
+        const int pos = p_lo + j;
+        const bf16_t* src = ksrc + (size_t)j * stride;
+        float x[EPL];
+        if (EPL == 1) {
+            x[0] = bf16_to_f32(src[0]);
+        } else if (EPL == 2) {
+            const uint32_t u = *reinterpret_cast<const uint32_t*>(src);
+            x[0] = bf16_to_f32((bf16_t)(u & 0xffffu));
+            x[1 % EPL] = bf16_to_f32((bf16_t)(u >> 16));
+        } else {
+            const uint2 u = *reinterpret_cast<const uint2*>(src);
+            x[0] = bf16_to_f32((bf16_t)(u.x & 0xffffu));
+            x[1 % EPL] = bf16_to_f32((bf16_t)(u.x >> 16));
+            x[2 % EPL] = bf16_to_f32((bf16_t)(u.y & 0xffffu));
+            x[3 % EPL] = bf16_to_f32((bf16_t)(u.y >> 16));
+        }
+        if (k_norm_w) {
+            float ss = 0.f;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) ss += x[e] * x[e];
+            ss = wave_sum(ss);
+            const float scale = 1.0f / sqrtf(ss / (float)HD + k_eps);
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) x[e] = k_norm_w[lane * EPL + e] * x[e] * scale;
+        }
+        if (cos_table && pos >= 0 && pos < table_positions) {
+            const float* cr = cos_table + (size_t)pos * (HD / 2) + (lane % 32) * EPL;
+            const float* sr = sin_table + (size_t)pos * (HD / 2) + (lane % 32) * EPL;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                const float partner = __shfl_xor(x[e], 32, TLI_WAVE);
+                x[e] = lane < 32 ? x[e] * cr[e] - partner * sr[e] : partner * sr[e] + x[e] * cr[e];
+            }
+        }
+        bf16_t* dst = kdst + (size_t)j * HD;
+        if (EPL == 1) {
+            dst[0] = f32_to_bf16(x[0]);
+        } else if (EPL == 2) {
+            *reinterpret_cast<uint32_t*>(dst) = pack_bf16x2(x[0], x[1 % EPL]);
+        } else {
+            *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(x[0], x[1 % EPL]), pack_bf16x2(x[2 % EPL], x[3 % EPL]));
+        }
+    }
+
+    // values: one dim a thread, the positions as one run of slots
+    const bf16_t* vsrc = rows + (size_t)(heads + kv_heads + kvh) * HD;
+    for (int d = threadIdx.x; d < HD; d += QKV_WAVES * TLI_WAVE) {
+        bf16_t vals[G];
+#pragma unroll
+        for (int j = 0; j < G; ++j) vals[j] = j < n ? cache_value(vsrc[(size_t)j * stride + d]) : (bf16_t)0;
+        bf16_t* dst = v_cache + (((size_t)page * kv_heads + kvh) * HD + d) * page_size + slot0;
+        if (n == G) {               // a whole group: its slots start at a multiple of G
+            uint32_t w[G / 2];
+#pragma unroll
+            for (int j = 0; j < G / 2; ++j) w[j] = (uint32_t)vals[2 * j] | ((uint32_t)vals[2 * j + 1] << 16);
+            if (G == 16) {
+                reinterpret_cast<uint4*>(dst)[0] = make_uint4(w[0], w[1], w[2], w[3]);
+                reinterpret_cast<uint4*>(dst)[1] = make_uint4(w[4 % (G / 2)], w[5 % (G / 2)], w[6 % (G / 2)], w[7 % (G / 2)]);
+            } else {
+                reinterpret_cast<uint4*>(dst)[0] = make_uint4(w[0], w[1], w[2 % (G / 2)], w[3 % (G / 2)]);
+            }
+        } else {
+            for (int j = 0; j < n; ++j) dst[j] = vals[j];
+        }
+    }
+}
+
+// Keys (normed, rotated) and values of the step's rows into the cache; q is left to the attention
+// kernel that takes it from qkv itself.  bfloat16, head_dim 64, 128 or 256, the whole head rotated
+// (or none of it), pages of 8 or more.
+extern "C" int tli_keys_values_to_cache(
+    const void* qkv, void* k_cache, void* v_cache, const int* row_start, const int* seq_start, int num_seqs,
+    int rows, const int* tables, int table_width, int page_size, int num_pages, int heads, int kv_heads,
+    int head_dim, const float* k_norm_w, float k_eps, const float* cos_table, const float* sin_table,
+    int table_positions, void* stream) {
+    if (rows <= 0 || num_seqs <= 0) return 0;
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+        return tli_fail("keys_values_to_cache: head_dim %d, the kernel takes 64, 128 and 256", head_dim);
+    if (heads <= 0 || kv_heads <= 0 || kv_heads > 65535) return tli_fail("keys_values_to_cache: bad head counts");
+    if (page_size < 8 || (page_size & (page_size - 1)) || table_width <= 0 || num_pages <= 0)
+        return tli_fail("keys_values_to_cache: bad cache geometry (pages of a power of two, at least 8)");
+    if ((cos_table == nullptr) != (sin_table == nullptr)) return tli_fail("keys_values_to_cache: cos without sin");
+    hipStream_t s = (hipStream_t)stream;
+    const int G = page_size >= 16 ? 16 : 8;
+    const long groups = (long)rows / G + 2L * num_seqs;           // upper bound
+    if (groups > 2147483647L) return tli_fail("keys_values_to_cache: too many rows");
+    dim3 grid((unsigned)groups, kv_heads);
+#define KV(EPL, GG)                                                                                       \
+    keys_values_to_cache_kernel<EPL, GG><<<grid, QKV_WAVES * TLI_WAVE, 0, s>>>(                           \
+        (const bf16_t*)qkv, (bf16_t*)k_cache, (bf16_t*)v_cache, row_start, seq_start, num_seqs, tables,   \
+        table_width, page_size, num_pages, heads, kv_heads, k_norm_w, k_eps, cos_table, sin_table,        \
+        table_positions)
+    if (head_dim == 64) { if (G == 16) KV(1, 16); else KV(1, 8); }
+    else if (head_dim == 128) { if (G == 16) KV(2, 16); else KV(2, 8); }
+    else { if (G == 16) KV(4, 16); else KV(4, 8); }
+#undef KV
+    return tli_check_launch("keys_values_to_cache");
+}
+
 // rows: the step's rows; row_start/seq_start as the prefill attention takes them.  bfloat16.
 extern "C" int tli_values_to_cache(
     const void* qkv, void* v_cache, const int* row_start, const int* seq_start, int num_seqs, int rows,

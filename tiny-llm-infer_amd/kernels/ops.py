@@ -77,6 +77,7 @@ def load_library():
         "tli_swiglu": [P, P, I, I, I, P],
         "tli_qkv_to_cache": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I, I, I, I, I, P],
         "tli_values_to_cache": [P, P, P, P, I, I, P, I, I, I, I, I, I, P],
+        "tli_keys_values_to_cache": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, P, F, P, P, I, P],
         "tli_attention_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
         "tli_gemm_plain": [P, P, P, I, I, I, I, I, I, P],
         "tli_gemm_skinny_bf16": [P, P, P, I, I, I, I, I, I, P],
@@ -159,6 +160,7 @@ class HipOps:
         self.plain_products = False  # every matrix product through the plain kernel
         self.separate_norms = False  # tests: decode steps run their norms as kernels of their own
         self.unfused_decode = False  # tests: decode steps through qkv_to_cache and paged_attention too
+        self.separate_cache_writes = False   # tests: the keys and the values of prompt portions by a kernel each
         self.prefill_direct = 0      # tests: 1 = the prefill attention kernel without LDS staging; 2, 3 = with, 1 or 2 tiles a wave; 4..8 = a forced order of row blocks; 10, 11 = heads of 64 and 128 with two sets of waves a workgroup, with one; 13 = as 0 for rows with many keys before them
         self.mid_cfg = 0             # measurements: launch shape and k ranges of the 17..128-row kernel
         self.mid_splits = 0
@@ -541,6 +543,13 @@ class HipOps:
             self._check_cache(kc, vc, g, kv_heads, head_dim, qkv.dtype, step)
             k_ptr, v_ptr, tab_ptr = kc.data_ptr(), vc.data_ptr(), g.tables.data_ptr()
             width, page, pages = g.table_width, g.page_size, kc.shape[0]
+        if (not queries and write and qkv.dtype == torch.bfloat16 and head_dim in (64, 128, 256) and page >= 8
+                and (rotary is None or rd == head_dim) and not self.separate_cache_writes):
+            # keys and values in one pass (prompt portions: the attention kernel takes q from qkv itself)
+            self._call(self.lib.tli_keys_values_to_cache, qkv.data_ptr(), k_ptr, v_ptr, step.row_start.data_ptr(),
+                       step.seq_start.data_ptr(), step.num_seqs, T, tab_ptr, width, page, pages, heads, kv_heads,
+                       head_dim, _ptr(kw), float(ke), _ptr(cos), _ptr(sin), npos, self._stream())
+            return None
         self._call(self.lib.tli_qkv_to_cache, qkv.data_ptr(), _ptr(q), k_ptr, v_ptr,
                    step.positions.data_ptr(), step.seq_of_row.data_ptr(), tab_ptr, width, page, pages,
                    T, heads, kv_heads, head_dim, _ptr(qw), float(qe), _ptr(kw), float(ke),
