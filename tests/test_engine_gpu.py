@@ -108,10 +108,12 @@ def test_greedy_generation_bfloat16_follows_plain(model_folders, name):
     for p, r in zip(prompts, got):
         logits = plain_qwen3.forward(cfg, w, p + r.token_ids[:-1])[len(p) - 1:]
         for t, row in zip(r.token_ids, logits):
-            margin = 2.5e-2 * float(row.abs().max())
+            # (bfloat16 logits of these configurations are within 1.2e-2 of the largest logit of the plain
+            # ones, so a token the engine prefers is at most twice that below the plain best)
+            margin = 1.2e-2 * float(row.abs().max())
             assert float(row.max() - row[t]) <= 2 * margin
             same += int(t == int(row.argmax()))
-    assert same >= 30          # of 36
+    assert same >= 32          # of 36
 
 
 def test_temperature_workload_of_configuration_b(model_folders):

@@ -58,6 +58,32 @@ def test_sampling_without_allocation_matches_sampling_with_a_callers_scratch():
         assert torch.equal(got, want)
         assert int(got[0]) == int(logits[0].argmax())
         assert not torch.equal(got.long(), logits.argmax(dim=1).cpu())   # the draws are draws
+    # the drawn rows of the last (small) call against the rule itself, written out in numpy: token =
+    # argmax(logit + T * Gumbel(u)), u the hash of (seed, token) that tli_sample_uniform gives
+    import numpy as np
+
+    def uniforms(seed, n):
+        def mix(h):
+            h = h.copy()
+            h ^= h >> np.uint32(16); h *= np.uint32(0x85EBCA6B); h ^= h >> np.uint32(13)
+            h *= np.uint32(0xC2B2AE35); h ^= h >> np.uint32(16)
+            return h
+        lo, hi = np.uint32(seed & 0xFFFFFFFF), np.uint32(seed >> 32)
+        with np.errstate(over="ignore"):
+            h = mix(np.arange(n, dtype=np.uint32) ^ np.uint32(0x9E3779B9))
+            h = mix(h ^ lo)
+            h = mix(h + hi * np.uint32(0x85EBCA6B) + np.uint32(0x27D4EB2F))
+        # (in float32, as the kernel computes it: above 2^23 the half is rounded away)
+        return (((h >> np.uint32(8)).astype(np.float32) + np.float32(0.5)) * np.float32(1.0 / 16777216.0)).astype(np.float64)
+
+    lib.tli_sample_uniform.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32]
+    lib.tli_sample_uniform.restype = ctypes.c_float
+    assert all(uniforms(104, 50)[t] == lib.tli_sample_uniform(104, 0, t) for t in range(50))
+    host = logits.double().cpu().numpy()
+    for r in range(1, rows):
+        score = host[r] + float(temps[r]) * -np.log(-np.log(uniforms(int(seeds[r]), vocab)))
+        order = np.argsort(-score)
+        assert int(got[r]) == int(order[0]) or score[order[0]] - score[int(got[r])] < 1e-5     # float32 noise on a near-tie
     # beyond the array's size: refused, nothing launched, the output untouched
     limit = lib.tli_sample_no_alloc_max_rows()
     out = torch.full((4,), 7, dtype=torch.int32, device="cuda")

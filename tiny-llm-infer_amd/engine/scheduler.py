@@ -172,7 +172,11 @@ class Scheduler:
                 raise SchedulerError(f"request {seq.request_id} waits although all its {seq.size} tokens are in the cache")
             count = min(remaining, budget - tokens)
             if not self.cache.can_reserve(seq.request_id, seq.tokens_in_cache + count):
-                self.waiting.append(seq)          # (a window group has no pages for this portion yet)
+                # a window group has no pages for this portion yet: the request waits for others to give
+                # theirs back, unless no pool could ever hold it
+                if not self._pages_for_whole_pool(seq.size):
+                    raise SchedulerError(f"request {seq.request_id} holds {seq.size} tokens, more than all {self.cache.num_pages} pages of {self.cache.page_size} can take")
+                self.waiting.append(seq)
                 continue
             self.cache.reserve(seq.request_id, seq.tokens_in_cache + count)
             plan.items.append(PlanItem(seq, seq.tokens_in_cache, count, True))
