@@ -796,6 +796,39 @@ def test_keys_and_values_of_portions_in_one_pass(ops, hd, page, rotation, norms)
     assert float(v1[p5, 0, 7, pos[5] % page]) == 0.0
 
 
+@pytest.mark.parametrize("separate", [False, True])
+def test_cache_writes_of_a_step_with_hundreds_of_sequences(ops, separate):
+    """300 sequences in one step (more than a workgroup has threads), single rows and short
+    portions mixed, some with no rows before them: every key and value lands in its slot."""
+    heads, kv_heads, hd, page = 2, 2, 64, 16
+    rng = np.random.default_rng(3)
+    new_counts = [int(c) for c in rng.choice([1, 1, 1, 2, 5, 17, 33], 300)]
+    seq_lens = [c + int(rng.integers(0, 40)) for c in new_counts]
+    dtype = torch.bfloat16
+    num_pages = sum((n + page - 1) // page for n in seq_lens) + 3
+    step, tables, pos, seq = make_step(seq_lens, new_counts, page, num_pages, 17, kv_heads, hd, dtype)
+    T = len(pos)
+    qkv = rnd((T, (heads + 2 * kv_heads) * hd), dtype, 33).to(DEV)
+    k0 = step.cache.k.clone()
+    ops.separate_cache_writes = separate
+    try:
+        ops.qkv_to_cache(qkv, step, step.cache, heads, kv_heads, hd, None, None, None, queries=False)
+    finally:
+        ops.separate_cache_writes = False
+    kd = (heads) * hd
+    rows = torch.arange(T)
+    pages = torch.as_tensor(tables)[torch.as_tensor(seq), torch.as_tensor(pos) // page].long()
+    slots = torch.as_tensor(pos) % page
+    want_k = qkv[:, kd:kd + kv_heads * hd].reshape(T, kv_heads, hd).cpu()
+    want_v = qkv[:, kd + kv_heads * hd:].reshape(T, kv_heads, hd).cpu()
+    assert torch.equal(step.cache.k.cpu()[pages, :, slots], want_k)
+    assert torch.equal(step.cache.v.cpu()[pages, :, :, slots], want_v)
+    written = torch.zeros((num_pages, page), dtype=torch.bool)
+    written[pages, slots] = True
+    untouched = ~written[:, None, :, None].expand_as(k0.cpu())
+    assert torch.equal(step.cache.k.cpu()[untouched], k0.cpu()[untouched])
+
+
 @pytest.mark.parametrize("hd,counts", [(128, [1, 1]), (128, [20, 1]), (48, [5, 1])])
 def test_values_enter_the_cache_finite(ops, hd, counts):
     """Infinities and NaNs among the values become 0 on their way into the cache (every

@@ -186,6 +186,62 @@ qkv_to_cache_wide_kernel(
     }
 }
 
+// Which sequence and which of its groups a workgroup has: group `grp` of the step, where sequence
+// s has the positions seq_start[s] .. + its rows, cut at multiples of G.  Every thread of the
+// workgroup looks at one sequence (at a stride of the workgroup's size), the numbers of groups are
+// summed up to each thread through LDS, and the thread whose sequence holds `grp` says so: a
+// step of hundreds of sequences costs a workgroup a few rounds, not hundreds of dependent loads.
+// Returns false if the step has fewer groups (the grid is an upper bound).  `found` is 4 ints of LDS.
+template <int G>
+__device__ __forceinline__ bool find_group(int grp, const int* __restrict__ row_start,
+                                           const int* __restrict__ seq_start, int num_seqs, int* found,
+                                           int* wave_totals, int& seq, int& start, int& first_row, int& n_rows,
+                                           int& in_seq) {
+    const int tid = threadIdx.x, lane = tid % TLI_WAVE, wave = tid / TLI_WAVE;
+    const int waves = (blockDim.x + TLI_WAVE - 1) / TLI_WAVE;
+    if (tid == 0) found[0] = -1;
+    int base = 0;
+    for (int s0 = 0; s0 < num_seqs; s0 += blockDim.x) {
+        const int s = s0 + tid;
+        int fr = 0, nr = 0, st = 0, g = 0;
+        if (s < num_seqs) {
+            fr = row_start[s];
+            nr = row_start[s + 1] - fr;
+            st = seq_start[s];
+            g = nr > 0 ? (st + nr - 1) / G - st / G + 1 : 0;
+        }
+        int incl = g;                               // sum over the lanes up to this one
+#pragma unroll
+        for (int off = 1; off < TLI_WAVE; off <<= 1) {
+            const int up = __shfl_up(incl, off, TLI_WAVE);
+            if (lane >= off) incl += up;
+        }
+        __syncthreads();                            // (the totals of the round before have been read)
+        if (lane == TLI_WAVE - 1) wave_totals[wave] = incl;
+        __syncthreads();
+        int before = base, total = 0;
+        for (int w = 0; w < waves; ++w) {
+            if (w < wave) before += wave_totals[w];
+            total += wave_totals[w];
+        }
+        const int excl = before + incl - g;
+        if (g > 0 && grp >= excl && grp < excl + g) {
+            found[0] = s;
+            found[1] = grp - excl;
+        }
+        base += total;
+        __syncthreads();
+        if (found[0] >= 0 || grp < base) break;     // (uniform: every thread reads the same words)
+    }
+    seq = found[0];
+    if (seq < 0) return false;
+    in_seq = found[1];
+    first_row = row_start[seq];
+    n_rows = row_start[seq + 1] - first_row;
+    start = seq_start[seq];
+    return true;
+}
+
 // The values of a step's rows into the cache, for steps that bring many rows a sequence: a
 // workgroup takes up to G consecutive positions of one sequence that share a page and one kv
 // head; a thread reads one dim of each of them (a wave reads whole rows) and writes them as one
@@ -196,16 +252,10 @@ __global__ void values_to_cache_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* __restrict__ v_cache, const int* __restrict__ row_start,
     const int* __restrict__ seq_start, int num_seqs, const int* __restrict__ tables, int table_width,
     int page_size, int num_pages, int heads, int kv_heads, int head_dim) {
-    int grp = blockIdx.x, seq = 0, start = 0, first_row = 0, n_rows = 0;
-    for (; seq < num_seqs; ++seq) {
-        first_row = row_start[seq];
-        n_rows = row_start[seq + 1] - first_row;
-        start = seq_start[seq];
-        const int groups = n_rows > 0 ? (start + n_rows - 1) / G - start / G + 1 : 0;
-        if (grp < groups) break;
-        grp -= groups;
-    }
-    if (seq >= num_seqs) return;
+    __shared__ int found[4], wave_totals[16];
+    int seq, start, first_row, n_rows, grp;
+    if (!find_group<G>(blockIdx.x, row_start, seq_start, num_seqs, found, wave_totals, seq, start, first_row, n_rows, grp))
+        return;
     const int g0 = start / G + grp;
     const int p_lo = max(start, g0 * G), p_hi = min(start + n_rows, (g0 + 1) * G);
     const int n = p_hi - p_lo;
@@ -254,16 +304,10 @@ keys_values_to_cache_kernel(
     const float* __restrict__ k_norm_w, float k_eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int table_positions) {
     constexpr int HD = 64 * EPL;
-    int grp = blockIdx.x, seq = 0, start = 0, first_row = 0, n_rows = 0;
-    for (; seq < num_seqs; ++seq) {
-        first_row = row_start[seq];
-        n_rows = row_start[seq + 1] - first_row;
-        start = seq_start[seq];
-        const int groups = n_rows > 0 ? (start + n_rows - 1) / G - start / G + 1 : 0;
-        if (grp < groups) break;
-        grp -= groups;
-    }
-    if (seq >= num_seqs) return;
+    __shared__ int found[4], wave_totals[16];
+    int seq, start, first_row, n_rows, grp;
+    if (!find_group<G>(blockIdx.x, row_start, seq_start, num_seqs, found, wave_totals, seq, start, first_row, n_rows, grp))
+        return;
     const int g0 = start / G + grp;
     const int p_lo = max(start, g0 * G), p_hi = min(start + n_rows, (g0 + 1) * G);
     const int n = p_hi - p_lo;
