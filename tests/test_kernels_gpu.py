@@ -618,6 +618,70 @@ RAW_CASES = [
 ]
 
 
+def _solo_cases():
+    rng = np.random.default_rng(11)
+    many = [int(n) for n in rng.integers(1, 500, 70)]
+    many[3], many[17], many[40] = 1, 512, 33
+    return [
+        # heads, kv_heads, head_dim, norms, rotation, page, seq_lens, new rows, window, writes
+        (32, 8, 128, True, True, 16, many, [1] * 70, None, True),
+        (8, 8, 64, True, True, 8, [int(n) for n in rng.integers(1, 400, 41)], [1] * 41, 100, True),
+        (4, 1, 256, True, False, 32, [1500, 31, 32, 33, 700, 1, 64, 65, 999], [1] * 9, 700, True),
+        (16, 1, 64, False, True, 16, [48, 1, 300, 17, 16], [1] * 5, None, False),      # reads another layer's cache
+        (5, 5, 128, False, False, 64, [3000, 129, 64], [1] * 3, 900, True),             # a window that begins inside a page
+    ] + [c for c in RAW_CASES if max(c[7]) == 1 and c[2] in (64, 128, 256)]
+
+
+@pytest.mark.parametrize("case", _solo_cases())
+def test_decode_attention_with_a_wave_to_a_row(ops, case):
+    """The decode kernel for steps of many rows with short contexts (a wave does a row's kv head on
+    its own: norm and rotation, the row's key and value into the cache, all the row's keys, the
+    output) wherever its limits allow it, against float64 and against the two-kernel path, with the
+    cache it leaves; and given partial sums of the projections, bit for bit what their rounded sum
+    gives."""
+    from tiny_llm_infer_amd.kernels.ops import DeferredSum
+    heads, kv_heads, hd, norms, rotation, page, seq_lens, new_counts, window, writes = case
+    reach = max(128, 1 << (max(seq_lens) - 1).bit_length())
+
+    class G:
+        page_size = page
+    _, keys, _ = ops._decode_splits(len(seq_lens), reach, G, heads, kv_heads, hd, window)
+    ops.decode_solo = "always"
+    try:
+        takes = ops._decode_splits(len(seq_lens), reach, G, heads, kv_heads, hd, window)[0] == 1 and \
+            ops._a_wave_a_row(len(seq_lens), keys, G, heads, kv_heads, hd)
+        if not takes:
+            pytest.skip("the keys are split over workgroups, or lie in more pages than a wave keeps entries of")
+        _raw_projections_case(ops, case)
+        # partial sums of the projections
+        dtype = torch.bfloat16
+        num_pages = sum((n + page - 1) // page for n in seq_lens) + 3
+        step, tables, pos, seq = make_step(seq_lens, new_counts, page, num_pages, 7, kv_heads, hd, dtype, window)
+        fill_cache(step, tables, seq_lens, kv_heads, hd, dtype, 300)
+        step.cache.writes = writes
+        T, width = len(pos), (heads + 2 * kv_heads) * hd
+        planes = torch.stack([rnd((T, width), torch.float32, 60 + p) for p in range(3)]).to(DEV)
+        total = planes[0].clone()
+        for p in range(1, 3):
+            total += planes[p]
+        qn = ((1 + rnd((hd,), torch.float32, 22, 0.2)).to(DEV), 1e-5) if norms else None
+        kn = ((1 + rnd((hd,), torch.float32, 23, 0.2)).to(DEV), 3e-6) if norms else None
+        rotary = None
+        if rotation:
+            ang = torch.arange(4096, dtype=torch.float64)[:, None] * (10000.0 ** (-2.0 * torch.arange(hd // 2, dtype=torch.float64) / hd))[None, :]
+            rotary = (torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV), hd)
+        k0, v0 = step.cache.k.clone(), step.cache.v.clone()
+        want = ops.qkv_attention(total.to(dtype), step, step.cache, heads, kv_heads, hd, qn, kn, rotary, hd ** -0.5, window)
+        k1, v1 = step.cache.k.clone(), step.cache.v.clone()
+        step.cache.k.copy_(k0)
+        step.cache.v.copy_(v0)
+        got = ops.qkv_attention(DeferredSum(planes, dtype), step, step.cache, heads, kv_heads, hd, qn, kn, rotary,
+                                hd ** -0.5, window)
+        assert torch.equal(got, want) and torch.equal(step.cache.k, k1) and torch.equal(step.cache.v, v1)
+    finally:
+        ops.decode_solo = "auto"
+
+
 def test_the_prefill_kernel_is_told_of_keys_before_its_own_rows_only(ops):
     """The launch rule of the prefill kernel is told whether its rows have many keys before them.
     When the sequences that decode have gone to the decode kernel, the lengths that count are

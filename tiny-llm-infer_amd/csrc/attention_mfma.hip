@@ -816,6 +816,155 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     }
 }
 
+// Decode attention from the raw projections for steps of many rows with short contexts, a wave
+// to itself: wave w of a workgroup has row 4 blockIdx.y + w and the kv head of blockIdx.x, norms
+// and rotates the row's queries (its 16 columns are the heads of the kv group) and its key,
+// writes key and value into the cache, walks all the row's keys in blocks of 32 (the next block
+// asked for before this one is multiplied) and writes the output.  No LDS, no barrier, nothing
+// merged: where every row has few keys and there are rows enough to fill the chip, four waves
+// sharing out one row's prologue and merging their sums spend most of their instructions on
+// each other (the kernel above is bound by the issue of its instructions).  The row's block
+// table entries are held by the lanes (entry first_entry + lane) and looked up by a shuffle, so
+// a row sees at most 64 pages: the caller checks it.  head_dim == 32 NJ, at most 16 heads a kv
+// head.  grid (kv_heads * head_tiles, ceil(rows / 4)).
+template <int NJ, int ND>
+__global__ void __launch_bounds__(256)
+attention_decode_solo_kernel(bf16_t* __restrict__ out, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
+                             const int* __restrict__ positions, const int* __restrict__ seq_of_row,
+                             const int* __restrict__ tables, int table_width, int page_size, int page_shift,
+                             int num_pages, int rows, int heads, int kv_heads, int head_dim, float scale,
+                             int window, RawQkv raw) {
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, c = lane / 16;
+    const int row = blockIdx.y * 4 + wave;
+    if (row >= rows) return;                               // (no barrier anywhere: a wave may leave)
+    const int group = heads / kv_heads, head_tiles = (group + 15) / 16;
+    const int kv_head = blockIdx.x / head_tiles, head_tile = blockIdx.x % head_tiles;
+    const int col_head = head_tile * 16 + r;
+    const bool live = col_head < group;
+    const int head = kv_head * group + (live ? col_head : 0);
+    const int pos = positions[row];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int begin = lo / 32 * 32;
+    const int* table = tables + (size_t)seq_of_row[row] * table_width;
+    const int first_entry = begin >> page_shift;
+    // this lane's table entry, asked for before anything waits
+    const int entry_at = min(first_entry + lane, table_width - 1);
+    const int my_entry = table[entry_at];
+    CacheView cv{k_cache, v_cache, table, table_width, page_size, page_shift, num_pages, kv_heads, head_dim, kv_head};
+
+    const size_t width = (size_t)(heads + 2 * kv_heads) * head_dim;
+    const bf16_t* raw_row = raw.qkv ? raw.qkv + (size_t)row * width : nullptr;
+    const float* sums_row = raw.partial_sums ? raw.partial_sums + (size_t)row * width : nullptr;
+    const float* cos_row = raw.cos ? raw.cos + (size_t)pos * (head_dim / 2) : nullptr;
+    const float* sin_row = raw.cos ? raw.sin + (size_t)pos * (head_dim / 2) : nullptr;
+    Tile<NJ, ND> t;
+    tile_init(t);
+    t.pos = live ? pos : -1;
+    t.lo = live ? lo : 0;
+    const size_t q_off = (size_t)head * head_dim, k_off = (size_t)(heads + kv_head) * head_dim;
+    head_from_raw<NJ>(t.q, raw_row ? raw_row + q_off : nullptr, raw.q_norm_w, raw.q_eps, cos_row, sin_row,
+                      sums_row ? sums_row + q_off : nullptr, raw.parts, raw.part_stride);
+    auto page_of_key = [&](int key) {
+        const int page = __shfl(my_entry, (key >> page_shift) - first_entry, 64);
+        return (unsigned)page < (unsigned)num_pages ? page : 0;
+    };
+    if (raw.write_cache) {
+        // the row's own key (every lane column computes the same one; column 0 writes it) and value
+        Frag kf[NJ];
+        head_from_raw<NJ>(kf, raw_row ? raw_row + k_off : nullptr, raw.k_norm_w, raw.k_eps, cos_row, sin_row,
+                          sums_row ? sums_row + k_off : nullptr, raw.parts, raw.part_stride);
+        const int own_raw = __shfl(my_entry, (pos >> page_shift) - first_entry, 64);
+        const bool store = (unsigned)own_raw < (unsigned)num_pages;
+        const int slot = pos & (page_size - 1);
+        if (store && r == 0) {
+            bf16_t* kd = k_cache + (((size_t)own_raw * kv_heads + kv_head) * page_size + slot) * head_dim + c * 8 * NJ;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) *reinterpret_cast<uint4*>(kd + j * 8) = kf[j].u;
+        }
+        if (store) {
+            const size_t v_off = (size_t)(heads + kv_heads + kv_head) * head_dim;
+            bf16_t* vd = v_cache + ((size_t)own_raw * kv_heads + kv_head) * head_dim * page_size + slot;
+            for (int d = lane; d < head_dim; d += 64) {
+                bf16_t v;
+                if (sums_row) {
+                    float a = 0.f;
+                    for (int p = 0; p < raw.parts; p += 2) {
+                        const bool pair = p + 1 < raw.parts;
+                        const float x0 = sums_row[v_off + (size_t)p * raw.part_stride + d];
+                        const float x1 = sums_row[v_off + (size_t)(pair ? p + 1 : p) * raw.part_stride + d];
+                        a += x0;
+                        a += pair ? x1 : 0.f;
+                    }
+                    v = f32_to_bf16(a);
+                } else {
+                    v = raw_row[v_off + d];
+                }
+                vd[(size_t)d * page_size] = cache_value(v);
+            }
+        }
+        // the wave reads its own key and value back with the last block: its stores have to be done
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    }
+
+    // the blocks of 32 keys begin, begin + 32, .. up to the one that holds pos, two sets of
+    // registers taking turns (see the kernel above: dealt from the end, nothing asked for twice)
+    auto fetch = [&](KeyBlock<NJ, ND>& b, int t0) {
+        const int in_page = page_size - 1;
+        const int key_k = t0 + 8 * (r / 4) + (r % 4);
+        const bf16_t* kp = k_cache + (((size_t)page_of_key(key_k) * kv_heads + kv_head) * page_size + (key_k & in_page)) * head_dim;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                b.ka[u][j].u = *reinterpret_cast<const uint4*>(kp + (size_t)u * 4 * head_dim + c * 8 * NJ + j * 8);
+        const int key_v = t0 + 8 * c;
+        const bf16_t* vp = v_cache + ((size_t)page_of_key(key_v) * kv_heads + kv_head) * ((size_t)head_dim * page_size) + (key_v & in_page);
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt)
+            b.vt[dt].u = *reinterpret_cast<const uint4*>(vp + (size_t)(dt * 16 + r) * page_size);
+    };
+    int t0 = begin;
+    const int last = pos / 32 * 32;
+    {
+        KeyBlock<NJ, ND> b0, b1;
+        if (((last - t0) / 32) & 1) {                       // an even number of blocks
+            fetch(b1, t0);
+            fetch(b0, t0 + 32);
+            __builtin_amdgcn_sched_barrier(0);
+            tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, t0 + 8 * c, 4, scale);
+            __builtin_amdgcn_sched_barrier(0);
+            t0 += 32;
+        } else {
+            fetch(b0, t0);
+        }
+        while (t0 != last) {
+            fetch(b1, t0 + 32);
+            __builtin_amdgcn_sched_barrier(0);
+            tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 8 * c, 4, scale);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(b0, t0 + 64);
+            __builtin_amdgcn_sched_barrier(0);
+            tile_consume<NJ, ND, true>(t, b1.ka, b1.vt, t0 + 32 + 8 * c, 4, scale);
+            __builtin_amdgcn_sched_barrier(0);
+            t0 += 64;
+        }
+        tile_consume<NJ, ND, true>(t, b0.ka, b0.vt, t0 + 8 * c, 4, scale);
+    }
+    if (!live) return;
+    const float l = tile_sum(t);
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    bf16_t* o = out + ((size_t)row * heads + head) * head_dim;
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) {
+        uint2 packed;
+        packed.x = (uint32_t)f32_to_bf16(t.acc[dt][0] * inv) | ((uint32_t)f32_to_bf16(t.acc[dt][1] * inv) << 16);
+        packed.y = (uint32_t)f32_to_bf16(t.acc[dt][2] * inv) | ((uint32_t)f32_to_bf16(t.acc[dt][3] * inv) << 16);
+        *reinterpret_cast<uint2*>(o + dt * 16 + 4 * c) = packed;
+    }
+}
+
 // grid (heads, rows); one thread per output element
 __global__ void attention_merge_splits_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
                                               int heads, int head_dim, int splits) {
@@ -1564,6 +1713,32 @@ static int launch_decode(const void* q, void* out, float* partial, void* k_cache
                          void* stream) {
     if (rows <= 0) return 0;
     if (check_common("attention_decode", heads, kv_heads, head_dim, page_size, table_width, num_pages)) return 1;
+    if (splits == 0) {
+        // a wave a row: from the raw projections only, heads of 64, 128 or 256, the keys that a row
+        // sees within 64 pages
+        const int group0 = heads / kv_heads, tiles0 = (group0 + 15) / 16;
+        if (!raw || head_dim % 64 || head_dim == 192 || group0 > 16 || page_size < 8)
+            return tli_fail("attention_decode, a wave a row: from raw projections with heads of 64, 128 or 256, at "
+                            "most 16 heads a kv head, pages of at least 8");
+        // (a wave keeps 64 table entries; a window that begins inside a page and the rounding to blocks
+        // of 32 keys take up to two more than the keys themselves)
+        if (keys_per_split <= 0 || keys_per_split > 60 * page_size)
+            return tli_fail("attention_decode, a wave a row: %d keys in pages of %d are more than the 60 pages a wave "
+                            "keeps the table entries of", keys_per_split, page_size);
+        if ((rows + 3) / 4 > 65535) return tli_fail("attention_decode: %d rows exceed the grid limit", rows);
+        dim3 grid0(kv_heads * tiles0, (rows + 3) / 4);
+        hipStream_t s0 = (hipStream_t)stream;
+        const int shift0 = log2_exact(page_size);
+#define SOLO(NJ, ND)                                                                                              \
+    attention_decode_solo_kernel<NJ, ND><<<grid0, 256, 0, s0>>>((bf16_t*)out, (bf16_t*)k_cache, (bf16_t*)v_cache,   \
+        positions, seq_of_row, tables, table_width, page_size, shift0, num_pages, rows, heads, kv_heads, head_dim, \
+        scale * LOG2E, window, *raw)
+        if (head_dim == 64) SOLO(2, 4);
+        else if (head_dim == 128) SOLO(4, 8);
+        else SOLO(8, 16);
+#undef SOLO
+        return tli_check_launch("attention_decode_solo");
+    }
     if (splits < 1 || splits > 65535 || keys_per_split <= 0 || keys_per_split % 128)
         return tli_fail("attention_decode: %d splits of %d keys (keys per split must be a multiple of 128)",
                         splits, keys_per_split);

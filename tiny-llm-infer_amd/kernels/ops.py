@@ -161,6 +161,8 @@ class HipOps:
         self.separate_norms = False  # tests: decode steps run their norms as kernels of their own
         self.unfused_decode = False  # tests: decode steps through qkv_to_cache and paged_attention too
         self.separate_cache_writes = False   # tests: the keys and the values of prompt portions by a kernel each
+        self.decode_solo = "auto"    # the decode attention that gives a row's kv head a wave to itself: "auto" (where
+                                     # the rows fill the chip), "always" (wherever its limits allow), "never"
         self.prefill_direct = 0      # tests: 1 = the prefill attention kernel without LDS staging; 2, 3 = with, 1 or 2 tiles a wave; 4..8 = a forced order of row blocks; 10, 11 = heads of 64 and 128 with two sets of waves a workgroup, with one; 13 = as 0 for rows with many keys before them
         self.mid_cfg = 0             # measurements: launch shape and k ranges of the 17..128-row kernel
         self.mid_splits = 0
@@ -650,6 +652,8 @@ class HipOps:
             cos, sin, rd = self._rotary(rotary, step)
         out = torch.empty((T, heads * head_dim), dtype=qkv.dtype, device=self.device)
         splits, per_split, partial = self._decode_splits(step.num_rows, step.reach, g, heads, kv_heads, head_dim, window)
+        if splits == 1 and self._a_wave_a_row(T, per_split, g, heads, kv_heads, head_dim):
+            splits = 0
         self._call(self.lib.tli_qkv_attention_decode_bf16, None if sums is not None else qkv.data_ptr(),
                    out.data_ptr(), _ptr(partial),
                    kc.data_ptr(), vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
@@ -732,6 +736,19 @@ class HipOps:
             partial = torch.empty((T * heads * splits * (head_dim + 2),), dtype=torch.float32,
                                   device=self.device)
         return splits, per_split, partial
+
+    def _a_wave_a_row(self, T, keys, g, heads, kv_heads, head_dim) -> bool:
+        """Whether a decode step of ``T`` rows that see at most ``keys`` keys each goes to the kernel that
+        gives every (row, kv head) one wave to itself: when there are four such pairs for every compute
+        unit (a wave on its own waits for every block of its keys, so it takes many waves a SIMD to keep
+        the chip busy; then it wins because four waves that share out one row's work and merge their sums
+        spend most of their instructions on each other.  Measured at Qwen3-8B sizes, 160 keys a row, a whole
+        decode step: 32 rows 3.74 -> 3.93 ms, 64 rows 4.09 -> 4.18, 128 rows 5.38 -> 5.28, 256 rows 10.11 ->
+        9.73), and a row's keys lie within the 60 pages whose table entries a wave keeps in its lanes."""
+        if self.decode_solo == "never" or head_dim not in (64, 128, 256) or keys > 60 * g.page_size:
+            return False
+        groups = T * kv_heads * ((heads // kv_heads + 15) // 16)
+        return self.decode_solo == "always" or groups >= 4 * self.DECODE_WORKGROUPS
 
     def _attention_decode(self, q, out, step, kc, vc, g, heads, kv_heads, head_dim, scale, window):
         """One row per sequence."""
