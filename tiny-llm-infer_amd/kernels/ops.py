@@ -136,10 +136,9 @@ class HipOps:
     SKINNY_ROWS = 64
     MID_ROWS_FROM = 17           # from this many rows the x-sharing kernel multiplies,
     MID_ROWS_TO = 128            # up to this many
-    DECODE_WORKGROUPS = 256      # aim of the decode attention's key splitting: one workgroup a compute unit (measured
-                                 # against 128, 192 and 512 at batch 1 to 64 and 128 to 30,000 keys: up to 10% over 512);
-                                 # set to what the device reports when the library is loaded
-    DECODE_SPLIT_KEYS = 512      # a split walks at least this many keys (128, 256 and 1024 measured: no better)
+    DECODE_WORKGROUPS = 256      # the device's compute units (set to what the device reports when the library is loaded):
+                                 # the decode attention splits a row's keys to come near one workgroup for each
+    DECODE_SPLIT_KEYS = 1024     # a split walks at least this many keys
     # A step of prompt portions whose first sequences decode: those go to the decode kernel when the
     # longest of them has this many times the keys of the longest portion, or as many keys when they
     # are this many rows (measured at 2 to 63 rows of 200 to 6,000 keys beside portions of 300 to
@@ -722,11 +721,25 @@ class HipOps:
     def _decode_splits(self, T, reach, g, heads, kv_heads, head_dim, window):
         """How the keys of ``T`` rows that decode (``reach``: a power of two that the longest
         of their sequences fits) are split over workgroups: they are when the batch alone
-        would leave most of the 256 compute units idle."""
+        would leave most of the compute units idle and the rows are long enough for the split
+        to pay for its merge."""
         reach = reach if not window else min(reach, (window + 31) // 32 * 32 + 32)
         groups = T * kv_heads * ((heads // kv_heads + 15) // 16)
-        # a split costs a merge pass: only worth it when a workgroup would walk many keys
-        splits = max(1, min((self.DECODE_WORKGROUPS + groups - 1) // groups, reach // self.DECODE_SPLIT_KEYS, 64))
+        # A split costs a pass that merges the parts (4 to 5 us) and a workgroup that walks no more than
+        # 1,500 keys is done in the time of the shortest split run (13 to 17 us against 17.5), so: no split
+        # up to a reach of 2,048 keys; beyond, towards one workgroup a compute unit, half of that for 16
+        # (row, kv head) pairs and fewer (more parts than that cost more in the merge than they save in the
+        # walk), and splits of at least 1,024 keys, of 4,096 from a quarter of the compute units on (there
+        # the workgroups already share the memory's rate between them).  Measured at heads of 128, 1 to 64
+        # rows of 600 to 32,768 keys, every power of two of splits: this rule is within 8% of the best
+        # everywhere; the one before (256 workgroups, 512 keys) was up to 45% over it at 1,024 keys and 20%
+        # over it at 1 and 2 rows of 16,384 keys and more.
+        units = self.DECODE_WORKGROUPS
+        splits = 1
+        if reach > 2 * self.DECODE_SPLIT_KEYS and groups < units:
+            aim = units // 2 if groups <= units // 16 else units
+            least = self.DECODE_SPLIT_KEYS if groups <= units // 4 else 4 * self.DECODE_SPLIT_KEYS
+            splits = max(1, min((aim + groups - 1) // groups, reach // least, 64))
         # (a split's block table entries are kept in LDS: at most 2046 pages a split)
         splits = max(splits, -(-reach // (2046 * g.page_size // 128 * 128)))
         per_split = ((reach + splits - 1) // splits + 127) // 128 * 128

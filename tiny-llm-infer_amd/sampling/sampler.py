@@ -53,12 +53,18 @@ class Sampler:
         assert rows == len(params) == len(request_seeds) == len(sample_indices)
         if all(p.greedy for p in params):
             return self.ops.sample(logits)
-        temps = torch.tensor([0.0 if p.greedy else p.temperature for p in params],
-                             dtype=torch.float32)
         seeds = [draw_seed(s, i) for s, i in zip(request_seeds, sample_indices)]
-        seeds_t = torch.tensor([s - (1 << 64) if s >= (1 << 63) else s for s in seeds],
-                               dtype=torch.int64)
-        top_p = None
-        if any(p.top_p < 1.0 and not p.greedy for p in params):
-            top_p = torch.tensor([p.top_p for p in params], dtype=torch.float32).to(self.device)
-        return self.ops.sample(logits, temps.to(self.device), seeds_t.to(self.device), top_p=top_p)
+        with_top_p = any(p.top_p < 1.0 and not p.greedy for p in params)
+        # One staging buffer for the step's seeds, temperatures and top_p, in page-locked memory where the
+        # device is a GPU: its copy is queued behind the step's kernels and does not wait for them, which a
+        # copy from ordinary memory does (and with it the host, which then plans the next step beside an
+        # idle device).
+        staged = torch.empty(rows * 16, dtype=torch.uint8, pin_memory=self.device.type == "cuda")
+        staged[:rows * 8].view(torch.int64).copy_(
+            torch.tensor([s - (1 << 64) if s >= (1 << 63) else s for s in seeds], dtype=torch.int64))
+        staged[rows * 8:rows * 12].view(torch.float32).copy_(
+            torch.tensor([0.0 if p.greedy else p.temperature for p in params], dtype=torch.float32))
+        staged[rows * 12:].view(torch.float32).copy_(torch.tensor([p.top_p for p in params], dtype=torch.float32))
+        dev = staged.to(self.device, non_blocking=True)
+        return self.ops.sample(logits, dev[rows * 8:rows * 12].view(torch.float32), dev[:rows * 8].view(torch.int64),
+                               top_p=dev[rows * 12:].view(torch.float32) if with_top_p else None)
