@@ -279,6 +279,13 @@ class ModelRunner:
 
     def forward(self, step: StepView, num_wanted: int) -> Optional[torch.Tensor]:
         """Run the model over a packed step; float32 logits [wanted, vocab] or None."""
+        hold = getattr(self.env.ops, "hold_stream", None)
+        if hold is None:
+            return self._forward(step, num_wanted)
+        with hold():
+            return self._forward(step, num_wanted)
+
+    def _forward(self, step: StepView, num_wanted: int) -> Optional[torch.Tensor]:
         model = self.model
         resid = model.embedding.forward(step.token_ids, step.num_rows)
         pending = None

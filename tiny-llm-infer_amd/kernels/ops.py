@@ -7,6 +7,7 @@ kernel and its grid assume before anything is launched.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from ctypes import c_float, c_int, c_void_p
 from typing import Optional, Tuple
@@ -155,6 +156,7 @@ class HipOps:
         self.lib = load_library()
         with torch.cuda.device(self.device):
             self.DECODE_WORKGROUPS = int(self.lib.tli_device_compute_units())
+        self._held_stream = None
         self.force_plain = False     # tests: run the plain attention kernel for bfloat16 too
         self.plain_products = False  # every matrix product through the plain kernel
         self.separate_norms = False  # tests: decode steps run their norms as kernels of their own
@@ -188,7 +190,21 @@ class HipOps:
 
     # ---- helpers ----------------------------------------------------------
     def _stream(self):
+        if self._held_stream is not None:
+            return self._held_stream
         return torch.cuda.current_stream(self.device).cuda_stream
+
+    @contextlib.contextmanager
+    def hold_stream(self):
+        """Inside, every kernel goes to the stream that was current on entry: one look-up for the
+        hundreds of launches of a step instead of one each (a quarter of the host's time in a step
+        that is not replayed from a recording)."""
+        before = self._held_stream
+        self._held_stream = torch.cuda.current_stream(self.device).cuda_stream
+        try:
+            yield
+        finally:
+            self._held_stream = before
 
     def _call(self, fn, *args):
         if fn(*args) != 0:
