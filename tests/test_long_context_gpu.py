@@ -190,6 +190,40 @@ def test_decode_rows_with_long_contexts(ops, name):
         assert torch.equal(step.cache.v[p, :, :, pos[r] % page], vv[r].to(BF))
 
 
+def test_decode_rows_of_unequal_lengths_are_split_by_their_skew(ops):
+    """One long sequence among many short ones: told of the skew (the runner sets it from the lengths),
+    the launch rule splits the keys although the rows alone fill the chip, and not otherwise; both
+    launches against float64, and the planted key of the long row found in every split."""
+    heads, kv_heads, hd, page = 32, 8, 128, 16
+    seq_lens = [4000] + [300] * 31
+    num_pages = sum((n + page - 1) // page for n in seq_lens) + 5
+    step, tables, pos, seq = make_step(seq_lens, [1] * len(seq_lens), page, num_pages, 5, kv_heads, hd, BF, None)
+    g = step.cache.group
+    assert ops._decode_splits(len(seq_lens), step.reach, g, heads, kv_heads, hd, None)[0] == 1
+    splits, per_split, _ = ops._decode_splits(len(seq_lens), step.reach, g, heads, kv_heads, hd, None, skew=8)
+    assert splits > 1
+    assert ops._decode_splits(len(seq_lens), step.reach, g, heads, kv_heads, hd, 1024, skew=8)[0] == 1     # a window evens the rows out
+    ks, vs = fill(step, tables, seq_lens, kv_heads, hd, 100)
+    scale = 1.0 / math.sqrt(hd)
+    q = rnd_dev((len(pos), heads * hd), 50)
+    want = ref_attention_dev(q, ks, vs, pos, seq, heads, kv_heads, scale, None)
+    close(ops.paged_attention(q, step, step.cache, heads, kv_heads, hd, scale, None), want, "unsplit")
+    step.skew = 8
+    close(ops.paged_attention(q, step, step.cache, heads, kv_heads, hd, scale, None), want, "split by the skew")
+    # a key that takes all the weight, in each split of the long row in turn
+    table0 = torch.as_tensor(tables[0], device=DEV).long()
+    q[0, :] = 2.0
+    for spot in [per_split * i + d for i in range(splits) for d in (0, per_split // 2) if per_split * i + d < seq_lens[0]]:
+        k, v = step.cache.k, step.cache.v
+        p, slot = int(table0[spot // page]), spot % page
+        old_k, old_v = k[p, :, slot].clone(), v[p, :, :, slot].clone()
+        k[p, :, slot] = 4.0
+        v[p, :, :, slot] = 3.0
+        out = ops.paged_attention(q, step, step.cache, heads, kv_heads, hd, scale, None)
+        assert (out[0].float() - 3.0).abs().max() < 0.05, f"key {spot}"
+        k[p, :, slot], v[p, :, :, slot] = old_k, old_v
+
+
 @pytest.mark.parametrize("name,stride", [("one-row-32000", 37), ("cap-of-64-splits", 41),
                                          ("table-entries-a-split", 53), ("window-4096", 7)])
 def test_decode_finds_a_planted_key_wherever_it_lies(ops, name, stride):
@@ -416,3 +450,46 @@ def test_a_request_of_9000_tokens_through_the_engine(long_request, dtype):
         assert err <= tol * scale, f"{dtype}/{cut}: error {err:.3e} at token {row} (logit scale {scale:.3e})"
         runner.cache.check()
         assert runner.cache.free_pages() == runner.cache.pages_per_group()
+
+
+def test_a_long_request_decodes_beside_short_ones(long_request):
+    """The 9,000-token request's last 24 tokens one by one in steps that five short requests share
+    (bfloat16, recorded steps): the lengths are so unequal that the decode attention's keys are split
+    by the skew, and every request's logits still are the plain implementation's."""
+    from helpers import TINY, collect, max_error, plain_logits, random_prompt
+    from tiny_llm_infer_amd.engine.loading import load_model
+    from tiny_llm_infer_amd.engine.replay import Replayer
+    from tiny_llm_infer_amd.engine.runner import ModelRunner
+    folder, reqs, want = long_request
+    n, tail = LONG, 24
+    short = {f"s{i}": random_prompt(TINY["D"]["vocab_size"], 40 + 31 * i + tail, 50 + i) for i in range(5)}
+    want = dict(want, **plain_logits(folder, short))
+    steps = [{"step": 0, "entries": [{"id": "r0", "tokens": reqs["r0"][:n - tail], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": rid, "tokens": toks[:-tail], "want": []} for rid, toks in short.items()], "end": []}]
+    for j in range(tail):
+        entries = [{"id": "r0", "tokens": [reqs["r0"][n - tail + j]], "want": [0]}]
+        entries += [{"id": rid, "tokens": [toks[len(toks) - tail + j]], "want": [0]} for rid, toks in short.items()]
+        steps.append({"step": len(steps), "entries": entries, "end": list(short) + ["r0"] if j == tail - 1 else []})
+    model, _ = load_model(folder, "bfloat16", "cuda:0")
+    runner = ModelRunner(model, model.env, page_size=8, num_pages=(n + 7) // 8 + 5 * 40 + 8, max_requests=6,
+                         max_batch_tokens=n)
+    seen = []
+    rule = type(model.env.ops)._decode_splits
+
+    def spy(self, T, reach, g, heads, kv_heads, head_dim, window, skew=1):
+        out = rule(self, T, reach, g, heads, kv_heads, head_dim, window, skew)
+        seen.append((skew, window, out[0]))
+        return out
+    type(model.env.ops)._decode_splits = spy
+    try:
+        rp = Replayer(runner)
+        got = collect(steps, {st["step"]: rp.run_step(st) for st in steps})
+    finally:
+        type(model.env.ops)._decode_splits = rule
+    assert any(skew > 1 and not window and splits > 1 for skew, window, splits in seen), seen[:8]
+    assert runner.graph_replays >= tail - 2
+    for rid, toks in dict(short, r0=reqs["r0"]).items():
+        err, row, scale = max_error(got[rid], want[rid][len(toks) - tail:])
+        assert err <= 2.5e-2 * scale, f"{rid}: error {err:.3e} at decoded token {row} (logit scale {scale:.3e})"
+    runner.cache.check()
+    assert runner.cache.free_pages() == runner.cache.pages_per_group()

@@ -579,7 +579,10 @@ __device__ __forceinline__ uint4 slice_finish(float (&x)[8], bool normed, const 
     return make_uint4(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]), pack_bf16x2(x[4], x[5]), pack_bf16x2(x[6], x[7]));
 }
 
-// grid (splits, kv_heads * head_tiles, rows); 256 threads.  FUSED: queries come from the
+// grid (kv_heads * head_tiles, rows, splits); 256 threads.  (Workgroups go to the eight dies in turn,
+// in the order of the grid with x fastest: with the splits in x, split s of every row would run on the
+// dies s, s + splits, .., and the dies of a row's last splits, which are short or empty, would idle
+// while the others walk the whole ones.)  FUSED: queries come from the
 // raw projections `raw` (q is not read), and the workgroup whose keys include the row's
 // own position writes that key and value into the cache first; needs head_dim == 32*NJ
 // and at most 16 heads a kv head (one workgroup per kv head and split).
@@ -593,10 +596,10 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
                         int splits, int keys_per_split, RawQkv raw) {
     extern __shared__ float lds[];       // 4 waves x 64 lanes x (ND*4 + 2), then this split's table entries, FUSED: the prologue's sums of squares and slices of q
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, c = lane / 16;
-    const int split = blockIdx.x, row = blockIdx.z;
+    const int split = blockIdx.z, row = blockIdx.y;
     const int group = heads / kv_heads;
     const int head_tiles = (group + 15) / 16;
-    const int kv_head = blockIdx.y / head_tiles, head_tile = blockIdx.y % head_tiles;
+    const int kv_head = blockIdx.x / head_tiles, head_tile = blockIdx.x % head_tiles;
     const int col_head = head_tile * 16 + r;                  // head inside the kv group
     const bool live = col_head < group;
     const int head = kv_head * group + col_head;
@@ -1750,7 +1753,7 @@ static int launch_decode(const void* q, void* out, float* partial, void* k_cache
     if (raw && (head_dim % 64 || group > 16))
         return tli_fail("attention_decode from raw projections: head_dim %d must be a multiple of 64 and "
                         "heads per kv head (%d) at most 16", head_dim, group);
-    dim3 grid(splits, kv_heads * head_tiles, rows);
+    dim3 grid(kv_heads * head_tiles, rows, splits);
     const int shift = log2_exact(page_size);
     // the table entries of one split are kept in LDS
     const size_t seg_bytes = ((((size_t)(keys_per_split >> shift) + 2) + 3) & ~(size_t)3) * sizeof(int);      // (16-byte aligned: the prologue's exchange comes behind it)

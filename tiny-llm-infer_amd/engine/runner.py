@@ -137,7 +137,7 @@ class ModelRunner:
                                  _decode_bucket(max_requests), len(self.cache.groups), max_width)
         self.steps_run = 0
         # Decode steps (one token for every request, every logit wanted) launch the same
-        # kernels with the same arguments whenever (requests, table width, reach) agree:
+        # kernels with the same arguments whenever (requests, table width, reach, skew) agree:
         # their launch sequence is recorded once as a HIP graph and replayed.
         parts = [model.embedding, model.final_norm, model.head] + list(model.blocks)
         self.use_graphs = (env.device.type == "cuda" and env.dtype == torch.bfloat16
@@ -275,6 +275,7 @@ class ModelRunner:
             h_row_start=row_start, h_seq_start=starts, h_seq_len=totals,
             h_slots=slots, max_rows_per_seq=max(counts),
             max_seq_len=max(totals), reach=max(128, 1 << (max(totals) - 1).bit_length()),
+            skew=min(16, 1 << ((max(totals) * len(totals)) // max(sum(totals), 1)).bit_length() - 1),
             groups=groups)
 
     def forward(self, step: StepView, num_wanted: int) -> Optional[torch.Tensor]:
@@ -309,7 +310,7 @@ class ModelRunner:
     def _replay(self, view: StepView, wanted: int) -> torch.Tensor:
         """A decode step through its recorded launch sequence.  The step's inputs
         already lie in the device buffer whose layout depends on the key alone."""
-        key = (view.num_seqs, view.groups[0].table_width if view.groups else 0, view.reach)
+        key = (view.num_seqs, view.groups[0].table_width if view.groups else 0, view.reach, view.skew)
         entry = self.graphs.get(key)
         if entry is None:
             self.forward(view, wanted)                 # once eagerly: anything lazy happens now

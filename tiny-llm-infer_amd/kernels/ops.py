@@ -666,7 +666,8 @@ class HipOps:
         if rotary is not None:
             cos, sin, rd = self._rotary(rotary, step)
         out = torch.empty((T, heads * head_dim), dtype=qkv.dtype, device=self.device)
-        splits, per_split, partial = self._decode_splits(step.num_rows, step.reach, g, heads, kv_heads, head_dim, window)
+        splits, per_split, partial = self._decode_splits(step.num_rows, step.reach, g, heads, kv_heads, head_dim, window,
+                                                         getattr(step, "skew", 1))
         if splits == 1 and self._a_wave_a_row(T, per_split, g, heads, kv_heads, head_dim):
             splits = 0
         self._call(self.lib.tli_qkv_attention_decode_bf16, None if sums is not None else qkv.data_ptr(),
@@ -734,11 +735,12 @@ class HipOps:
             return 13
         return int(self.prefill_direct)
 
-    def _decode_splits(self, T, reach, g, heads, kv_heads, head_dim, window):
+    def _decode_splits(self, T, reach, g, heads, kv_heads, head_dim, window, skew=1):
         """How the keys of ``T`` rows that decode (``reach``: a power of two that the longest
         of their sequences fits) are split over workgroups: they are when the batch alone
         would leave most of the compute units idle and the rows are long enough for the split
-        to pay for its merge."""
+        to pay for its merge.  ``skew``: the longest sequence has at least this many times the
+        keys of the average one."""
         reach = reach if not window else min(reach, (window + 31) // 32 * 32 + 32)
         groups = T * kv_heads * ((heads // kv_heads + 15) // 16)
         # A split costs a pass that merges the parts (4 to 5 us) and a workgroup that walks no more than
@@ -750,6 +752,12 @@ class HipOps:
         # rows of 600 to 32,768 keys, every power of two of splits: this rule is within 8% of the best
         # everywhere; the one before (256 workgroups, 512 keys) was up to 45% over it at 1,024 keys and 20%
         # over it at 1 and 2 rows of 16,384 keys and more.
+        # Sequences of unequal lengths: the workgroups of the short ones are done early, so the step's
+        # rows count as that many fewer of the longest one's length (32 rows, one of 4,000 keys and 31 of
+        # 300: 40 us unsplit, 30 us in four splits; 16 rows of 64 to 2,304 keys: 24.3 and 22.5 us).  With a
+        # window every row walks about as many keys.
+        if skew > 1 and not window:
+            groups = max(1, groups // skew)
         units = self.DECODE_WORKGROUPS
         splits = 1
         if reach > 2 * self.DECODE_SPLIT_KEYS and groups < units:
@@ -782,7 +790,8 @@ class HipOps:
     def _attention_decode(self, q, out, step, kc, vc, g, heads, kv_heads, head_dim, scale, window):
         """One row per sequence."""
         T = step.num_rows
-        splits, per_split, partial = self._decode_splits(step.num_rows, step.reach, g, heads, kv_heads, head_dim, window)
+        splits, per_split, partial = self._decode_splits(step.num_rows, step.reach, g, heads, kv_heads, head_dim, window,
+                                                         getattr(step, "skew", 1))
         self._call(self.lib.tli_attention_decode_bf16, q.data_ptr(), out.data_ptr(), _ptr(partial),
                    kc.data_ptr(), vc.data_ptr(), step.positions.data_ptr(), step.seq_of_row.data_ptr(),
                    g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], T, heads, kv_heads,

@@ -80,6 +80,8 @@ class StepView:
     max_seq_len: int = 1
     reach: int = 1                # max_seq_len rounded up to a power of two: launches are shaped by
                                   # this, so that steps of like shape launch alike (and can be replayed)
+    skew: int = 1                 # the longest sequence has at least this many times the tokens of the average
+                                  # one (a power of two, at most 16): launches may split the long ones' work by it
     groups: List[GroupView] = field(default_factory=list)
     # filled by the runner for the layer call that is running
     cache: Optional[LayerCache] = None
@@ -88,7 +90,7 @@ class StepView:
 
 class Part:
     # True if forward() looks at nothing on the host but the step's shape (rows,
-    # sequences, table width, reach): then a recorded launch sequence can be replayed
+    # sequences, table width, reach, skew): then a recorded launch sequence can be replayed
     replayable = False
 
     def __init__(self, spec: PartSpec):
