@@ -215,3 +215,24 @@ def test_a_window_group_has_the_smaller_pool(model_folders):
     assert eng.scheduler.num_preemptions == 0
     cache.check()
     assert cache.free_pages() == [160, 22]
+
+
+def test_a_step_is_told_how_unequal_its_sequences_are(model_folders):
+    """``StepView.skew``: the largest power of two (at most 16) that the longest sequence of a step
+    has times the average length; rows that only fill a decode step up count as sequences of one
+    token.  Launch rules may split the long sequences' work by it."""
+    from tiny_llm_infer_amd.engine.runner import StepEntry
+    eng = _engine(model_folders["A"], "A", max_model_len=128, num_kv_blocks=64, max_num_seqs=8, max_num_batched_tokens=128)
+    runner = eng.runner
+    lengths = {"long": 100, "a": 5, "b": 5, "c": 6}
+    for key in lengths:
+        runner.admit(key)
+    view = runner._pack([StepEntry(k, [1] * n, []) for k, n in lengths.items()])
+    assert view.max_seq_len == 100 and view.skew == 2                 # 100 against an average of 29
+    for k, n in lengths.items():
+        runner.cache.reserve(k, n)
+        runner.cache.advance(k, n)
+    view = runner._pack([StepEntry(k, [1], [0]) for k in lengths], pad_to=8)
+    assert view.num_seqs == 8 and view.skew == 4                      # 101 against (101 + 6 + 6 + 7 + 4) / 8
+    view = runner._pack([StepEntry(k, [1], [0]) for k in ("a", "b", "c")])
+    assert view.skew == 1
