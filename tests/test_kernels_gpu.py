@@ -451,6 +451,11 @@ ATT_CASES = [
     (8, 2, 128, 64, [700], [650], None),
     (4, 2, 128, 128, [700, 130], [333, 2], 100),
     (4, 1, 64, 256, [600], [600], None),
+    # many sequences in a step: beyond 16 the workgroups of the prefill kernels look their sequence up
+    # together (one sequence a thread, sums by shuffles and through LDS), in rounds when there are more
+    # sequences than threads
+    (8, 2, 128, 16, [13 + 7 * (i % 9) for i in range(40)], [2 + i % 5 for i in range(40)], None),
+    (4, 2, 64, 8, [5 + i % 11 for i in range(600)], [2 + i % 3 for i in range(600)], 6),
     # rows with many keys before them (the caller tells the launch rule): with between 256 and 512
     # workgroups of two tiles a wave the rule then keeps one set of waves and two tiles, below that
     # it takes two sets

@@ -993,6 +993,96 @@ __global__ void attention_merge_splits_kernel(const float* __restrict__ partial,
 }
 
 // -------------------------------------------------------------------- prefill --
+// Which sequence a row block of a step belongs to.  The row blocks of a step are numbered sequence by
+// sequence (a sequence of n rows has ceil(n / rows_per_block) of them).  Up to SEQS_WALKED sequences a
+// workgroup walks the list by itself (a few scalar loads); beyond, a walk of hundreds of dependent loads
+// would take longer than the attention (256 sequences of 8 rows: 499 us a layer), and the workgroup looks
+// together: every thread takes a sequence, sums within waves by shuffles and across waves through LDS.
+// Both must be called by every thread of the workgroup, before any of them leaves.
+#define SEQS_WALKED 16
+
+// All row blocks of the step.
+__device__ __forceinline__ int count_row_blocks(const int* __restrict__ row_start, int num_seqs, int rows_per_block) {
+    int total = 0;
+    if (num_seqs <= SEQS_WALKED) {
+        for (int seq = 0; seq < num_seqs; ++seq)
+            total += (row_start[seq + 1] - row_start[seq] + rows_per_block - 1) / rows_per_block;
+        return total;
+    }
+    __shared__ int wave_sums[16];
+    const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE, waves = (blockDim.x + TLI_WAVE - 1) / TLI_WAVE;
+    for (int s = threadIdx.x; s < num_seqs; s += blockDim.x)
+        total += (row_start[s + 1] - row_start[s] + rows_per_block - 1) / rows_per_block;
+#pragma unroll
+    for (int off = TLI_WAVE / 2; off > 0; off >>= 1) total += __shfl_xor(total, off, TLI_WAVE);
+    __syncthreads();                                    // (what an earlier call left there has been read)
+    if (lane == 0) wave_sums[wave] = total;
+    __syncthreads();
+    total = 0;
+    for (int w = 0; w < waves; ++w) total += wave_sums[w];
+    return total;
+}
+
+// Row block `block` of the step: its sequence, that sequence's first row and number of rows, and
+// the block's number within the sequence (left in `block`).  False if the step has fewer row blocks.
+__device__ __forceinline__ bool find_row_block(int& block, const int* __restrict__ row_start, int num_seqs,
+                                               int rows_per_block, int& seq, int& first_row, int& n_rows) {
+    if (num_seqs <= SEQS_WALKED) {
+        for (seq = 0; seq < num_seqs; ++seq) {
+            first_row = row_start[seq];
+            n_rows = row_start[seq + 1] - first_row;
+            const int blocks = (n_rows + rows_per_block - 1) / rows_per_block;
+            if (block < blocks) return true;
+            block -= blocks;
+        }
+        return false;
+    }
+    __shared__ int wave_totals[16], found[4];
+    const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE, waves = (blockDim.x + TLI_WAVE - 1) / TLI_WAVE;
+    __syncthreads();                                    // (what an earlier call left there has been read)
+    if (threadIdx.x == 0) found[0] = -1;
+    int base = 0;
+    for (int s0 = 0; s0 < num_seqs; s0 += blockDim.x) {
+        const int s = s0 + threadIdx.x;
+        int fr = 0, nr = 0, blocks = 0;
+        if (s < num_seqs) {
+            fr = row_start[s];
+            nr = row_start[s + 1] - fr;
+            blocks = (nr + rows_per_block - 1) / rows_per_block;
+        }
+        int incl = blocks;                              // sum over the lanes up to this one
+#pragma unroll
+        for (int off = 1; off < TLI_WAVE; off <<= 1) {
+            const int up = __shfl_up(incl, off, TLI_WAVE);
+            if (lane >= off) incl += up;
+        }
+        __syncthreads();                                // (the totals of the round before have been read)
+        if (lane == TLI_WAVE - 1) wave_totals[wave] = incl;
+        __syncthreads();
+        int before = base, total = 0;
+        for (int w = 0; w < waves; ++w) {
+            if (w < wave) before += wave_totals[w];
+            total += wave_totals[w];
+        }
+        before += incl - blocks;                        // row blocks of the sequences before this thread's
+        if (blocks > 0 && block >= before && block < before + blocks) {
+            found[0] = s;
+            found[1] = fr;
+            found[2] = nr;
+            found[3] = block - before;
+        }
+        base += total;
+        if (block < base) break;                        // (the same for every thread)
+    }
+    __syncthreads();
+    seq = found[0];
+    if (seq < 0) return false;
+    first_row = found[1];
+    n_rows = found[2];
+    block = found[3];
+    return true;
+}
+
 // grid (row blocks upper bound, kv_heads * head_tiles); 256 threads.
 // A wave owns CT column tiles; a tile is `rq` consecutive rows of one sequence x
 // min(group, 16) heads; the wave's tiles are consecutive in the sequence and share
@@ -1013,14 +1103,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     const int rows_per_wave = CT * rq, rows_per_block = 4 * rows_per_wave;
     // which sequence and which of its row blocks is this workgroup's?
     int block = blockIdx.x, seq = 0, first_row = 0, n_rows = 0;
-    for (; seq < num_seqs; ++seq) {
-        first_row = row_start[seq];
-        n_rows = row_start[seq + 1] - first_row;
-        const int blocks = (n_rows + rows_per_block - 1) / rows_per_block;
-        if (block < blocks) break;
-        block -= blocks;
-    }
-    if (seq >= num_seqs) return;
+    if (!find_row_block(block, row_start, num_seqs, rows_per_block, seq, first_row, n_rows)) return;
     const int local0 = block * rows_per_block + wave * rows_per_wave;   // this wave's first row in the portion
     if (local0 >= n_rows) return;
     const int wave_rows = min(rows_per_wave, n_rows - local0);
@@ -1101,14 +1184,8 @@ __device__ __forceinline__ void prefill_lds_block(
     const int heads_here = min(16, group - head_tile * 16);
     const int rows_per_wave = CT * rq, rows_per_block = 4 * rows_per_wave;
     int seq = 0, first_row = 0, n_rows = 0;
-    for (; seq < num_seqs; ++seq) {
-        first_row = row_start[seq];
-        n_rows = row_start[seq + 1] - first_row;
-        const int blocks = (n_rows + rows_per_block - 1) / rows_per_block;
-        if (block < blocks) break;
-        block -= blocks;
-    }
-    if (seq >= num_seqs) return;                      // the whole workgroup leaves together
+    if (!find_row_block(block, row_start, num_seqs, rows_per_block, seq, first_row, n_rows))
+        return;                                       // the whole workgroup leaves together
     const int start = seq_start[seq];
     const int block0 = block * rows_per_block;        // first row of the workgroup in the portion
     const int block_rows = min(rows_per_block, n_rows - block0);
@@ -1325,14 +1402,8 @@ __device__ __forceinline__ void prefill_pipe_block(
     const int heads_here = min(16, group - head_tile * 16);
     const int rows_per_wave = CT * rq, rows_per_block = 4 * rows_per_wave;
     int seq = 0, first_row = 0, n_rows = 0;
-    for (; seq < num_seqs; ++seq) {
-        first_row = row_start[seq];
-        n_rows = row_start[seq + 1] - first_row;
-        const int blocks = (n_rows + rows_per_block - 1) / rows_per_block;
-        if (block < blocks) break;
-        block -= blocks;
-    }
-    if (seq >= num_seqs) return;                      // the whole workgroup leaves together
+    if (!find_row_block(block, row_start, num_seqs, rows_per_block, seq, first_row, n_rows))
+        return;                                       // the whole workgroup leaves together
     const int start = seq_start[seq];
     const int block0 = block * rows_per_block;        // first row of the workgroup in the portion
     const int block_rows = min(rows_per_block, n_rows - block0);
@@ -1615,9 +1686,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ 
                              int page_shift, int num_pages, int heads, int kv_heads,
                              float scale_log2, int window, int rq, int pair, RawQkv raw) {
     const int rows_per_block = 4 * CT * rq;
-    int total = 0;
-    for (int seq = 0; seq < num_seqs; ++seq)
-        total += (row_start[seq + 1] - row_start[seq] + rows_per_block - 1) / rows_per_block;
+    const int total = count_row_blocks(row_start, num_seqs, rows_per_block);
     const int head_count = gridDim.y;
     // the row block and head (and for pair = 1 a second row block) of this workgroup
     int rb, hd_i = blockIdx.y, rb2 = -1;
