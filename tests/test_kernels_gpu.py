@@ -613,14 +613,39 @@ RAW_CASES = [
     (6, 3, 256, True, True, 16, [90, 17], [7, 17], 64, True),
     (4, 2, 128, False, False, 32, [45], [45], None, True),
     (16, 1, 64, True, True, 16, [48, 9], [5, 9], None, False),
-    # sequences that decode in front of portions of prompts, as the scheduler puts them: where one of
-    # them has many more keys than the portions, or they are many, they go to the decode kernel and the
-    # rest of the step to the prefill kernel
-    (32, 8, 128, True, True, 16, [1500, 40, 300, 64], [1, 1, 130, 64], None, True),
-    (8, 8, 64, True, True, 8, [130, 257, 16, 17, 9, 700] * 6 + [200, 31], [1] * 36 + [150, 31], 19, True),
-    (8, 2, 128, True, True, 16, [90, 1900, 513], [1, 1, 257], 300, True),
+    # sequences that decode in front of portions of prompts, as the scheduler puts them: where a few of
+    # them have many more keys than the portions, or they are many beside short portions, they go to the
+    # decode kernel and the rest of the step to the prefill kernel
+    (32, 8, 128, True, True, 16, [3100, 40, 300, 64], [1, 1, 130, 64], None, True),
+    (8, 8, 64, True, True, 8, [130, 257, 16, 17, 9, 700] * 11 + [200, 31], [1] * 66 + [150, 31], 19, True),
+    (8, 2, 128, True, True, 16, [90, 3100, 513], [1, 1, 257], 300, True),
     (8, 2, 128, True, True, 16, [90, 300, 513], [1, 1, 257], None, True),          # (these stay in the one kernel)
+    (8, 8, 64, True, True, 8, [130, 257, 16, 17, 9, 700] * 6 + [200, 31], [1] * 36 + [150, 31], 19, True),   # (and these)
 ]
+MIXED_TO_DECODE = {-5: 2, -4: 66, -3: 2, -2: 0, -1: 0}     # how many leading sequences of those cases the decode kernel takes
+
+
+def test_which_rows_of_a_mixed_step_go_to_the_decode_kernel(ops):
+    """The rule itself, on the mixed cases above (so that both ways stay covered by them) and at its edges."""
+    for at, want in MIXED_TO_DECODE.items():
+        heads, kv_heads, hd, _, _, page, seq_lens, new_counts, window, _ = RAW_CASES[at]
+        step, *_ = make_step(seq_lens, new_counts, page, sum((n + page - 1) // page for n in seq_lens) + 3, 7, kv_heads, hd,
+                             torch.bfloat16, window)
+        assert ops._rows_for_the_decode_kernel(step, heads, kv_heads) == want, RAW_CASES[at][6:8]
+    few, many = ops.DECODE_BESIDE_FEW, ops.DECODE_BESIDE_MANY
+
+    def takes(seq_lens, new_counts):
+        step, *_ = make_step(seq_lens, new_counts, 16, sum((n + 15) // 16 for n in seq_lens) + 3, 7, 2, 64, torch.bfloat16, None)
+        return ops._rows_for_the_decode_kernel(step, 8, 2)
+    assert takes([few[1]] * few[0] + [200], [1] * few[0] + [200]) == few[0]
+    assert takes([few[1]] * (few[0] + 1) + [200], [1] * (few[0] + 1) + [200]) == 0          # one row too many
+    assert takes([few[1] - 1] * 2 + [200], [1, 1, 200]) == 0                                # a key too few
+    assert takes([few[1]] * 2 + [few[1] // 2 + 1], [1, 1, 40]) == 0                         # not twice the portion's sequence
+    assert takes([20] * many[0] + [many[1]], [1] * many[0] + [many[1]]) == many[0]
+    assert takes([20] * many[0] + [many[1] + 1], [1] * many[0] + [many[1] + 1]) == 0        # a new token too many
+    assert takes([20] * (many[0] - 1) + [100], [1] * (many[0] - 1) + [100]) == 0
+    assert takes([500] * 70, [1] * 70) == 0                                                 # no portion: a decode step
+    assert takes([500, 300], [2, 300]) == 0                                                 # no row that decodes in front
 
 
 def _solo_cases():
@@ -747,7 +772,7 @@ def test_decode_attention_adds_partial_sums_of_the_projections(ops, case, parts)
     rotary = None
     if rotation:
         half = hd // 2
-        ang = torch.arange(2048, dtype=torch.float64)[:, None] * (10000.0 ** (-2.0 * torch.arange(half, dtype=torch.float64) / hd))[None, :]
+        ang = torch.arange(4096, dtype=torch.float64)[:, None] * (10000.0 ** (-2.0 * torch.arange(half, dtype=torch.float64) / hd))[None, :]
         rotary = (torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV), hd)
     scale = 1.0 / math.sqrt(hd)
     k0, v0 = step.cache.k.clone(), step.cache.v.clone()
@@ -780,7 +805,7 @@ def _raw_projections_case(ops, case):
     rotary = None
     half = hd // 2
     if rotation:
-        ang = torch.arange(2048, dtype=torch.float64)[:, None] * (10000.0 ** (-2.0 * torch.arange(half, dtype=torch.float64) / hd))[None, :]
+        ang = torch.arange(4096, dtype=torch.float64)[:, None] * (10000.0 ** (-2.0 * torch.arange(half, dtype=torch.float64) / hd))[None, :]
         cos, sin = torch.cos(ang).float(), torch.sin(ang).float()
         rotary = (cos.to(DEV), sin.to(DEV), hd)
     scale = 1.0 / math.sqrt(hd)

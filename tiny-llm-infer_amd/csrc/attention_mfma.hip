@@ -1930,10 +1930,13 @@ static int launch_prefill(
         // 2,048 tokens behind up to 30,720: up to a third faster while all workgroups run at once
         // (256), a tenth faster up to 512 workgroups whose rows have no keys before them (the short
         // ones fill the second round), 3 to 15% slower there with keys before them (direct = 13 says
-        // so: the lengths are on the device) and slower beyond.
+        // so: the lengths are on the device) and slower beyond.  Several sequences in a step have no such
+        // long and short row blocks to share out: beyond two sequences the second round does not pay
+        // either (8 sequences of 256 rows: 54 us in two sets, 42 us in one; 4 of 512: 58 and 50; one of
+        // 2,000 beside 16 single rows: 93 and 77).
         const bool dma = head_dim == 64 || head_dim == 128;
         const long groups2 = (blocks2 - num_seqs) * kv_heads * head_tiles;
-        bool sets = dma && groups2 <= (direct == 13 ? units : 2 * units);
+        bool sets = dma && groups2 <= (direct == 13 || num_seqs > 2 ? units : 2 * units);
         if (sets) two = (blocks1 - num_seqs) * kv_heads * head_tiles > units;
         // rows with keys before them are all about as long: two tiles a wave, which read the keys
         // once for both, already pay when one round of them fills the chip (1,536 rows behind

@@ -140,12 +140,18 @@ class HipOps:
     DECODE_WORKGROUPS = 256      # the device's compute units (set to what the device reports when the library is loaded):
                                  # the decode attention splits a row's keys to come near one workgroup for each
     DECODE_SPLIT_KEYS = 1024     # a split walks at least this many keys
-    # A step of prompt portions whose first sequences decode: those go to the decode kernel when the
-    # longest of them has this many times the keys of the longest portion, or as many keys when they
-    # are this many rows (measured at 2 to 63 rows of 200 to 6,000 keys beside portions of 300 to
-    # 2,048 tokens: a second kernel costs 15 to 30 us, which a few short rows do not bring back)
-    DECODE_BESIDE_PROMPTS_KEYS = 2.0
-    DECODE_BESIDE_PROMPTS = 32
+    # A step of prompt portions whose first sequences decode: the prefill kernel takes a row that decodes
+    # as a sequence of one row, beside its other workgroups; the decode kernel is a second launch (8 to 10
+    # us) that runs before it, but splits a long row's keys and puts four waves on a row.  Those rows go
+    # to the decode kernel when they are few and much longer than the portions (up to 8 rows of 3,000
+    # keys and more, twice the longest portion's sequence: 4 rows of 4,000 keys beside 256 / 1,024 /
+    # 2,000 new tokens 62 / 110 / 126 us in the prefill kernel, 47 / 69 / 98 us with the decode kernel),
+    # or many beside short portions (64 rows and more beside at most 512 new tokens: 64 rows of 200 keys
+    # beside 256 tokens 50 against 42 us, 128 rows 75 against 53).  Measured at 4 to 128 rows of 200 to
+    # 4,000 keys beside 256 to 2,000 new tokens behind up to 3,584 keys; elsewhere the prefill kernel
+    # alone is as fast or up to a fifth faster.
+    DECODE_BESIDE_FEW = (8, 3000, 2.0)       # at most so many rows, of at least so many keys and so many times the portions' longest
+    DECODE_BESIDE_MANY = (64, 512)           # at least so many rows, beside at most so many new tokens
 
     def __init__(self, device):
         self.device = torch.device(device)
@@ -692,20 +698,9 @@ class HipOps:
         qw, qe = q_norm if q_norm is not None else (None, 0.0)
         cos, sin = (rotary[0], rotary[1]) if rotary is not None else (None, None)
         out = torch.empty((T, heads * head_dim), dtype=qkv.dtype, device=self.device)
-        # The sequences that decode (one row each) stand first in a step that the scheduler
-        # made.  The prefill kernel would give each of them workgroups that walk all their keys
-        # with one row; where those would be the last to finish they go to the decode kernel instead,
-        # which splits a row's keys over workgroups (their keys and values are in the cache by now).
-        first = 0
-        starts = step.h_row_start
-        while first < step.num_seqs and starts[first + 1] - starts[first] == 1:
-            first += 1
-        if first == step.num_seqs or heads // kv_heads > 16 or self.prefill_direct:
-            first = 0
-        longest = max(step.h_seq_len[:first]) if first else 0
-        beside = max(step.h_seq_len[first:step.num_seqs]) if first else 0
-        if first and (longest >= self.DECODE_BESIDE_PROMPTS_KEYS * beside
-                      or (first >= self.DECODE_BESIDE_PROMPTS and longest >= beside)):
+        first = self._rows_for_the_decode_kernel(step, heads, kv_heads)
+        if first:
+            longest = max(step.h_seq_len[:first])
             kw, ke = k_norm if k_norm is not None else (None, 0.0)
             splits, per_split, partial = self._decode_splits(first, max(128, 1 << (longest - 1).bit_length()), g, heads,
                                                              kv_heads, head_dim, window)
@@ -714,8 +709,6 @@ class HipOps:
                        g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], first, heads, kv_heads,
                        head_dim, _ptr(qw), float(qe), _ptr(kw), float(ke), _ptr(cos), _ptr(sin),
                        0, float(scale), int(window or 0), splits, per_split, None, 0, self._stream())
-        else:
-            first = 0
         direct = self._prefill_mode(step, T - first, first)
         self._call(self.lib.tli_qkv_attention_prefill_bf16, qkv.data_ptr(), out.data_ptr(), kc.data_ptr(),
                    vc.data_ptr(), step.row_start.data_ptr() + 4 * first, step.seq_start.data_ptr() + 4 * first,
@@ -724,6 +717,26 @@ class HipOps:
                    head_dim, _ptr(qw), float(qe), _ptr(cos), _ptr(sin), float(scale), int(window or 0),
                    direct, self._stream())
         return out
+
+    def _rows_for_the_decode_kernel(self, step, heads, kv_heads) -> int:
+        """How many of a mixed step's leading sequences go to the decode kernel.  The sequences that
+        decode (one row each) stand first in a step that the scheduler made.  The prefill kernel gives
+        each of them workgroups that walk all their keys with one row; where that is slower than a
+        second launch (see DECODE_BESIDE_FEW, DECODE_BESIDE_MANY) they go to the decode kernel, which
+        splits a row's keys over workgroups (their keys and values are in the cache by then)."""
+        first = 0
+        starts = step.h_row_start
+        while first < step.num_seqs and starts[first + 1] - starts[first] == 1:
+            first += 1
+        if first == 0 or first == step.num_seqs or heads // kv_heads > 16 or self.prefill_direct:
+            return 0
+        longest = max(step.h_seq_len[:first])
+        beside = max(step.h_seq_len[first:step.num_seqs])
+        few, many = self.DECODE_BESIDE_FEW, self.DECODE_BESIDE_MANY
+        if (first <= few[0] and longest >= few[1] and longest >= few[2] * beside) or \
+                (first >= many[0] and step.num_rows - first <= many[1]):
+            return first
+        return 0
 
     def _prefill_mode(self, step, rows, first=0):
         """The mode argument of the prefill attention kernels for the sequences from ``first`` on
