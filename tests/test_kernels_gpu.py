@@ -327,6 +327,27 @@ def test_library_linear_for_many_rows(ops):
     close(y32, x.double() @ w.double().t(), torch.float32, "float32 logits for many rows", scale=5.0)
 
 
+def test_float32_logits_for_hundreds_of_rows(ops):
+    """A decode step of hundreds of requests (or a replay that wants every position) asks a matrix in
+    the decode layout for float32 logits of more than 128 rows: 128 rows at a time through the
+    x-sharing kernel, the rest through the one for few rows; a row's logits are those it gets alone."""
+    from tiny_llm_infer_amd.parts.base import BuildEnv
+    from tiny_llm_infer_amd.parts.linear import Matrix
+    env = BuildEnv(dtype=torch.bfloat16, device=torch.device(DEV), ops=ops, max_model_len=64)
+    K, N = 264, 1003                                    # a vocabulary that is no multiple of anything
+    w = rnd((N, K), torch.bfloat16, 2, 0.05)
+    m = Matrix(w.to(DEV), env)
+    for M in (129, 256, 300, 391):                      # a last portion of 1, 128, 44 and 7 rows
+        x = rnd((M, K), torch.bfloat16, M)
+        y = ops.linear(x.to(DEV), m, out_dtype=torch.float32)
+        assert y.dtype == torch.float32 and tuple(y.shape) == (M, N)
+        want = x.double() @ w.double().t()
+        close(y, want, torch.float32, f"float32 logits for {M} rows", scale=float(want.abs().max()) * (K ** 0.5) / 8)
+        for r in (0, 127, 128, M - 1):
+            alone = ops.linear(x[r:r + 1].contiguous().to(DEV), m, out_dtype=torch.float32)
+            close(y[r:r + 1], alone.double().cpu(), torch.float32, f"row {r} of {M} and alone", scale=float(want.abs().max()))
+
+
 def test_linear_rows_do_not_depend_on_the_batch(ops):
     """float32: a row's product is bit-identical whatever else is in the batch."""
     x, w = rnd((70, 100), torch.float32, 9), rnd((130, 100), torch.float32, 10)
