@@ -831,7 +831,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
 // a row sees at most 64 pages: the caller checks it.  head_dim == 32 NJ, at most 16 heads a kv
 // head.  grid (kv_heads * head_tiles, ceil(rows / 4)).
 template <int NJ, int ND>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, ND <= 8 ? 2 : 1)      // (two waves a SIMD where the registers allow: a wave on its own waits for every block of its keys)
 attention_decode_solo_kernel(bf16_t* __restrict__ out, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
                              const int* __restrict__ positions, const int* __restrict__ seq_of_row,
                              const int* __restrict__ tables, int table_width, int page_size, int page_shift,
