@@ -330,7 +330,7 @@ def test_library_linear_for_many_rows(ops):
 def test_float32_logits_for_hundreds_of_rows(ops):
     """A decode step of hundreds of requests (or a replay that wants every position) asks a matrix in
     the decode layout for float32 logits of more than 128 rows: 128 rows at a time through the
-    x-sharing kernel, the rest through the one for few rows; a row's logits are those it gets alone."""
+    x-sharing kernel; a row's logits are those it gets alone, and the same bits among more rows."""
     from tiny_llm_infer_amd.parts.base import BuildEnv
     from tiny_llm_infer_amd.parts.linear import Matrix
     env = BuildEnv(dtype=torch.bfloat16, device=torch.device(DEV), ops=ops, max_model_len=64)
@@ -346,6 +346,9 @@ def test_float32_logits_for_hundreds_of_rows(ops):
         for r in (0, 127, 128, M - 1):
             alone = ops.linear(x[r:r + 1].contiguous().to(DEV), m, out_dtype=torch.float32)
             close(y[r:r + 1], alone.double().cpu(), torch.float32, f"row {r} of {M} and alone", scale=float(want.abs().max()))
+        # among more rows (a recorded step is filled up with rows of no request): the same bits
+        more = torch.cat([x, rnd((23, K), torch.bfloat16, 77)])
+        assert torch.equal(ops.linear(more.to(DEV), m, out_dtype=torch.float32)[:M], y)
 
 
 def test_linear_rows_do_not_depend_on_the_batch(ops):

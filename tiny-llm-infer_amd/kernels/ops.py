@@ -362,15 +362,12 @@ class HipOps:
             if tiled is not None and out_dtype == torch.float32 and M > self.MID_ROWS_TO:
                 # float32 logits for many rows (a decode step of hundreds of requests, a replay that wants
                 # every position): the x-sharing kernel, 128 rows at a time (512 rows of the Qwen3-8B
-                # head: 8 x 363 us in the kernel below, 4 x 240 us here)
+                # head: 8 x 363 us in the kernel below, 4 x 240 us here).  The last rows too, however few: a
+                # row's sums are then the same bits whatever the number of rows beside it, which a step
+                # replayed with rows that only fill it up relies on.
                 for m0 in range(0, M, self.MID_ROWS_TO):
                     m1 = min(M, m0 + self.MID_ROWS_TO)
-                    if m1 - m0 >= self.MID_ROWS_FROM:
-                        self._linear_mid(x[m0:m1], tiled, y[m0:m1], m1 - m0, N, K, 0)
-                    else:
-                        self._call(self.lib.tli_gemm_skinny_bf16, x[m0:m1].data_ptr(), tiled.data_ptr(),
-                                   y[m0:m1].data_ptr(), m1 - m0, N, K, _dtype_code(out_dtype), 1, self.skinny_cfg,
-                                   self._stream())
+                    self._linear_mid(x[m0:m1], tiled, y[m0:m1], m1 - m0, N, K, 0)
                 return y
             if M <= self.SKINNY_ROWS or out_dtype == torch.float32:
                 # few rows (decode), or float32 logits: the weight-streaming MFMA kernel,
