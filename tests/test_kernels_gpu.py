@@ -193,6 +193,48 @@ def test_gated_product_writes_the_activation(ops, mki):
     close(two_pass, torch.nn.functional.silu(g) * u, torch.bfloat16, "stacked product, then activation")
 
 
+@pytest.mark.parametrize("mnk", [(129, 264, 1008), (200, 4096, 4096), (256, 6144, 520), (177, 1000, 136), (255, 48, 8), (144, 5120, 384)])
+def test_two_row_blocks_side_by_side_in_the_x_sharing_kernel(ops, mnk):
+    """129..256 rows of a product without a gate: two blocks of 128 rows of gemm_mid in one launch (the
+    second block's workgroups run beside the first's and find the W fragments in their die's L2), at
+    sizes that are no multiples of its tiles, with the planned and with forced launch shapes and ranges
+    of k, the partial sums left for the consumer, and rows that do not depend on the rows beside them."""
+    from tiny_llm_infer_amd.kernels.ops import DeferredSum
+    M, N, K = mnk
+    x, w = rnd((M, K), torch.bfloat16, 1), rnd((N, K), torch.bfloat16, 2, 0.05)
+    behind = torch.full((M * K + 8192,), float("nan"), dtype=torch.bfloat16, device=DEV)     # x lies in front of NaNs
+    xd = behind[:M * K].view(M, K)
+    xd.copy_(x)
+    tiled = ops.tile_matrix(w.to(DEV))
+    want = x.double() @ w.double().t()
+
+    def product(rows=M, deferred=False):
+        y = torch.full((rows, N), 7.0, dtype=torch.bfloat16, device=DEV)
+        return ops._linear_mid(xd[:rows], tiled, y, rows, N, K, 0, deferred)
+    first = product()
+    close(first, want, torch.bfloat16, "two row blocks")
+    assert ops.lib.tli_gemm_mid_splits_rows(M, N, K, 0) >= 1
+    for splits, cfg in ((1, 0), (2, 0), (5, 0), (1, 224), (3, 223), (2, 214), (4, 228)):
+        ops.mid_splits, ops.mid_cfg = splits, cfg
+        try:
+            close(product(), want, torch.bfloat16, f"{splits} ranges of k, shape {cfg}")
+            left = product(deferred=True)
+            if splits > 1:
+                assert isinstance(left, DeferredSum) and tuple(left.parts.shape) == (splits, M, N)
+                close(left.parts.sum(0), want, torch.float32, "partial sums")
+            close(ops.resolve(left), want, torch.bfloat16, "partial sums resolved")
+        finally:
+            ops.mid_splits = ops.mid_cfg = 0
+    # fewer rows, still two blocks: the same bits for the rows that are there
+    if M > 140:
+        assert torch.equal(product(rows=M - 9), first[:M - 9])
+    # through linear(), which takes this kernel for a matrix held in the decode layout
+    class Both:
+        tiled_ = tiled
+    Both.w, Both.tiled = w.to(DEV), tiled
+    assert torch.equal(ops.linear(xd, Both), first)
+
+
 @pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 6])
 @pytest.mark.parametrize("mnk", [(129, 264, 1008), (300, 4096, 4096), (2048, 6144, 512), (513, 1000, 136), (700, 48, 8), (4500, 520, 256),
                                  (1024, 5120, 384)])

@@ -1,5 +1,5 @@
-// Matrix product for 17..128 rows (a large decode batch): y[M,N] = x[M,K] . W^T with W in
-// the decode layout (see gemm_skinny.hip).  Still bound by streaming W once, but with
+// Matrix product for 17..128 rows (a large decode batch), and for plain products of up to 256: y[M,N] =
+// x[M,K] . W^T with W in the decode layout (see gemm_skinny.hip).  Still bound by streaming W once, but with
 // four or eight 16-row tiles of x every W fragment meets as many x fragments, and taking
 // those from L2 for every wave (as the kernel for <= 16 rows does) would cost that many
 // times the traffic of W itself.  Here the waves of a workgroup own different output
@@ -41,12 +41,12 @@ union Pack16m {
     bf16x8 v;
 };
 
-#define MID_MAX_ROWS 128
+#define MID_MAX_ROWS 256
 
 template <int RT, int WAVES, int DEPTH, int MT, typename TO, bool GATED>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* __restrict__ y,
-                float* __restrict__ part, int M, int N, int K, int splits, int steps_per_split) {
+                float* __restrict__ part, int M_all, int N, int K, int splits, int steps_per_split) {
     constexpr int ROWS = MT * 16;
     constexpr int STAGES = DEPTH + 1;                        // W: DEPTH slices on their way, one in use
     constexpr int XSLOTS = DEPTH + 2;                        // x: one slice further ahead
@@ -59,15 +59,26 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
     bf16_t* xs = reinterpret_cast<bf16_t*>(xs_raw);          // [XSLOTS][ROWS][128], rows swizzled
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, r = lane % 16, c = lane / 16;
     const int k_steps = (K + 127) / 128;
-    const int tile0 = (blockIdx.x * WAVES + wave) * RT;       // this wave's first 16-column tile
     const int n_tiles = (N + 15) / 16;
+    // More than ROWS rows: the row blocks of one column group are workgroups 8 apart, which run on the
+    // same die at the same time, so that the second one finds the W fragments in that die's L2.
+    const int row_blocks = (M_all + ROWS - 1) / ROWS;
+    int group = blockIdx.x, row0 = 0;
+    if (row_blocks > 1) {
+        row0 = (group / TLI_DIES) % row_blocks * ROWS;
+        group = group / (TLI_DIES * row_blocks) * TLI_DIES + group % TLI_DIES;
+        if (group * WAVES * RT >= n_tiles) return;            // (the column groups are rounded up to a multiple of 8)
+    }
+    const int M = min(ROWS, M_all - row0);
+    x += (size_t)row0 * K;
+    const int tile0 = (group * WAVES + wave) * RT;            // this wave's first 16-column tile
     const int step_begin = blockIdx.y * steps_per_split;
     const int step_end = min(k_steps, step_begin + steps_per_split);
     // Workgroups walk their k range from different starting slices, wrapping round: a
     // slice of x is rows a power of two apart, which all lie in one channel of the L2
     // cache, and workgroups in step would all wait for that one channel.  (Workgroups go
     // round the eight dies in turn, so neighbours on a die are blockIdx.x / 8 apart.)
-    const int rot = step_begin < step_end ? (blockIdx.x / TLI_DIES) % (step_end - step_begin) : 0;
+    const int rot = step_begin < step_end ? (group / TLI_DIES) % (step_end - step_begin) : 0;
     auto at = [&](int step) { return step + rot < step_end ? step + rot : step + rot - (step_end - step_begin); };
 
     f32x4 acc[RT][MT];
@@ -201,7 +212,7 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
 
     // lane holds y[m*16 + r][tile*16 + 4c + i]
     if (splits > 1) {
-        float* dst = part + (size_t)blockIdx.y * M * N;
+        float* dst = part + ((size_t)blockIdx.y * M_all + row0) * N;
 #pragma unroll
         for (int t = 0; t < RT; ++t) {
             const int n0 = (tile0 + t) * 16 + 4 * c;
@@ -222,6 +233,7 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
     }
     if (GATED) {
         const int n_out = N / 2;
+        y += (size_t)row0 * n_out;
 #pragma unroll
         for (int t = 0; t + 1 < RT; t += 2) {
             const int n0 = ((tile0 + t) / 2) * 16 + 4 * c;
@@ -240,6 +252,7 @@ gemm_mid_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TO* 
         }
         return;
     }
+    y += (size_t)row0 * N;
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
         const int n0 = (tile0 + t) * 16 + 4 * c;
@@ -258,7 +271,8 @@ static int launch_mid_rows(const bf16_t* x, const bf16_t* w, void* y, float* par
                            int y_dtype, int gated, int splits, hipStream_t s) {
     const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
     const int steps_per_split = (k_steps + splits - 1) / splits;
-    dim3 grid((n_tiles + RT * WAVES - 1) / (RT * WAVES), splits);
+    const int groups = (n_tiles + RT * WAVES - 1) / (RT * WAVES), row_blocks = (M + MT * 16 - 1) / (MT * 16);
+    dim3 grid(row_blocks > 1 ? (groups + TLI_DIES - 1) / TLI_DIES * TLI_DIES * row_blocks : groups, splits);
     const size_t lds = (size_t)(DEPTH + 2) * MT * 16 * 128 * sizeof(bf16_t);
     // (more than 64 KiB of LDS has to be allowed for a kernel once)
 #define MID_LAUNCH(TO, G)                                                                                  \
@@ -310,9 +324,33 @@ static int mid_tiles_per_wave(int N, int gated) { return gated || (N + 15) / 16 
 // columns, 160 workgroups, were 9% slower); where the columns alone are more than 128 groups
 // but fewer than 192, two tiles a wave and the ranges that go with them (10,240 columns: 80
 // groups in 3 ranges).  A range keeps at least two slices of 128.  Gated products: see below.
-static void mid_plan(int N, int K, int gated, int* tiles_a_wave, int* waves_a_group, int* ranges) {
+static void mid_plan(int N, int K, int gated, int row_blocks, int* tiles_a_wave, int* waves_a_group, int* ranges) {
     const int n_tiles = (N + 15) / 16, k_steps = (K + 127) / 128;
     const int units = tli_compute_units(), most = 3 * units / 4;      // 256 and 192 on MI355X
+    if (row_blocks > 1) {
+        // Row blocks of 128 rows side by side (the second finds the W fragments in its die's L2): two
+        // column tiles a wave, three or four waves and the ranges of k that come closest to one workgroup
+        // a compute unit from below, all row blocks counted (measured at the Qwen3-8B sizes and 160 to 256
+        // rows: 6,144 columns in 64 groups of three waves and 2 ranges, 4,096 in 32 groups of four waves
+        // and 4 ranges; 7 to 18% faster than the kernel for any number of rows, which stays the faster one
+        // for gated products and beyond 256 rows).
+        int best = -1;
+        for (int w = 4; w >= 3; --w) {
+            const int groups = (n_tiles + 2 * w - 1) / (2 * w);
+            const int r = max(1, min(min(units / max(groups * row_blocks, 1), k_steps / 2), 16));
+            if (groups * r * row_blocks > best && groups * r * row_blocks <= units) {
+                best = groups * r * row_blocks;
+                *waves_a_group = w;
+                *ranges = r;
+            }
+        }
+        if (best < 0) {                       // more column groups than compute units: four waves, k whole
+            *waves_a_group = 4;
+            *ranges = 1;
+        }
+        *tiles_a_wave = 2;
+        return;
+    }
     auto ranges_for = [&](int groups) { return max(1, min(min(units / max(groups, 1), k_steps / 2), 16)); };
     int rt = mid_tiles_per_wave(N, gated), waves = 4;
     if (gated) {
@@ -348,11 +386,18 @@ static void mid_plan(int N, int K, int gated, int* tiles_a_wave, int* waves_a_gr
 // How many ranges of k a product of this shape is cut into (the caller sizes `part` by it).
 extern "C" int tli_gemm_mid_splits(int N, int K, int gated) {
     int rt, waves, splits;
-    mid_plan(N, K, gated, &rt, &waves, &splits);
+    mid_plan(N, K, gated, 1, &rt, &waves, &splits);
     return splits;
 }
 
-// y[M,N] = x[M,K] . W^T for 1 <= M <= 128, W in the decode layout (`gated` as tiled = 2 of
+// The same for M rows (more than 128: row blocks side by side).
+extern "C" int tli_gemm_mid_splits_rows(int M, int N, int K, int gated) {
+    int rt, waves, splits;
+    mid_plan(N, K, gated, (M + 127) / 128, &rt, &waves, &splits);
+    return splits;
+}
+
+// y[M,N] = x[M,K] . W^T for 1 <= M <= 256 (a gated product: 128), W in the decode layout (`gated` as tiled = 2 of
 // tli_gemm_skinny_bf16: y is [M, N/2] bfloat16).  `part`: splits*M*N floats when
 // splits > 1 (splits as returned by tli_gemm_mid_splits, or forced by the caller); with
 // y null the partial sums [splits][M][N] are left for the consumer to add (tli_gemm_mid_reduce,
@@ -361,7 +406,8 @@ extern "C" int tli_gemm_mid_splits(int N, int K, int gated) {
 extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* part, int M, int N, int K,
                                  int y_dtype, int gated, int splits, int cfg, void* stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > MID_MAX_ROWS) return tli_fail("gemm_mid: %d rows, at most %d", M, MID_MAX_ROWS);
+    if (M > MID_MAX_ROWS || (gated && M > 128))
+        return tli_fail("gemm_mid: %d rows, at most %d (%d for a gated product)", M, MID_MAX_ROWS, 128);
     if (K <= 0 || K % 8) return tli_fail("gemm_mid: K = %d must be a positive multiple of 8", K);
     if (y_dtype != TLI_BF16 && y_dtype != TLI_F32) return tli_fail("gemm_mid: bad output dtype %d", y_dtype);
     if (gated && (N % 32 || y_dtype != TLI_BF16))
@@ -378,8 +424,8 @@ extern "C" int tli_gemm_mid_bf16(const void* x, const void* w, void* y, float* p
         // sizes of Qwen3-14B and 32B): a gated product then takes eight waves a workgroup, a
         // plain one whose k ranges push it over takes two column tiles a wave
         int rt, planned, waves;
-        mid_plan(N, K, gated, &rt, &waves, &planned);
-        if (splits != planned) {                                      // (ranges forced by the caller)
+        mid_plan(N, K, gated, (M + 127) / 128, &rt, &waves, &planned);
+        if (splits != planned && M <= 128) {                          // (ranges forced by the caller)
             rt = mid_tiles_per_wave(N, gated);
             const int groups = ((N + 15) / 16 + waves * rt - 1) / (waves * rt);
             if (!gated && rt == 1 && (long)groups * splits > tli_compute_units()) rt = 2;

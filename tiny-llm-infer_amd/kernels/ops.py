@@ -85,6 +85,7 @@ def load_library():
         "tli_gemm_skinny_fused_bf16": [P, P, P, I, I, I, I, P, I, F, P, P, P, P, I, P],
         "tli_gemm_mid_bf16": [P, P, P, P, I, I, I, I, I, I, I, P],
         "tli_gemm_mid_splits": [I, I, I],
+        "tli_gemm_mid_splits_rows": [I, I, I, I],
         "tli_gemm_mid_reduce": [P, P, I, I, I, I, P],
         "tli_gemm_rows_bf16": [P, P, P, P, I, I, I, I, I, I, P],
         "tli_gemm_rows_splits": [I, I, I],
@@ -137,6 +138,7 @@ class HipOps:
     SKINNY_ROWS = 64
     MID_ROWS_FROM = 17           # from this many rows the x-sharing kernel multiplies,
     MID_ROWS_TO = 128            # up to this many
+    MID_ROWS_TO_PLAIN = 256      # a product without a gate: up to this many (two blocks of 128 rows side by side)
     DECODE_WORKGROUPS = 256      # the device's compute units (set to what the device reports when the library is loaded):
                                  # the decode attention splits a row's keys to come near one workgroup for each
     DECODE_SPLIT_KEYS = 1024     # a split walks at least this many keys
@@ -357,7 +359,9 @@ class HipOps:
         if M == 0:
             return y
         if x.dtype == torch.bfloat16 and K % 8 == 0:
-            if tiled is not None and self.MID_ROWS_FROM <= M <= self.MID_ROWS_TO:
+            # (beyond 128 rows only with bfloat16 results, and not where the library or a measurement was asked for)
+            if tiled is not None and self.MID_ROWS_FROM <= M <= (
+                    self.MID_ROWS_TO_PLAIN if out_dtype == torch.bfloat16 and self.many_rows == "own" else self.MID_ROWS_TO):
                 return self._linear_mid(x, tiled, y, M, N, K, 0, deferred or sums_only)
             if tiled is not None and out_dtype == torch.float32 and M > self.MID_ROWS_TO:
                 # float32 logits for many rows (a decode step of hundreds of requests, a replay that wants
@@ -428,10 +432,10 @@ class HipOps:
         return y
 
     def _linear_mid(self, x, tiled, y, M, N, K, gated, deferred=False):
-        """17..128 rows: the kernel that shares x through LDS, k cut into ranges when the
-        output alone gives too few workgroups.  ``deferred``: the partial sums of the
+        """17..128 rows (without a gate: up to 256): the kernel that shares x through LDS, k cut into
+        ranges when the output alone gives too few workgroups.  ``deferred``: the partial sums of the
         ranges are left for the consumer to add, which saves the pass that adds them."""
-        splits = self.mid_splits or self.lib.tli_gemm_mid_splits(N, K, gated)
+        splits = self.mid_splits or self.lib.tli_gemm_mid_splits_rows(M, N, K, gated)
         part = None
         if splits > 1:
             part = torch.empty((splits, M, N), dtype=torch.float32, device=self.device)
