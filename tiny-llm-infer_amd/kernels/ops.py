@@ -365,12 +365,13 @@ class HipOps:
                 return self._linear_mid(x, tiled, y, M, N, K, 0, deferred or sums_only)
             if tiled is not None and out_dtype == torch.float32 and M > self.MID_ROWS_TO:
                 # float32 logits for many rows (a decode step of hundreds of requests, a replay that wants
-                # every position): the x-sharing kernel, 128 rows at a time (512 rows of the Qwen3-8B
-                # head: 8 x 363 us in the kernel below, 4 x 240 us here).  The last rows too, however few: a
-                # row's sums are then the same bits whatever the number of rows beside it, which a step
-                # replayed with rows that only fill it up relies on.
-                for m0 in range(0, M, self.MID_ROWS_TO):
-                    m1 = min(M, m0 + self.MID_ROWS_TO)
+                # every position): the x-sharing kernel, 256 rows (two row blocks side by side) at a time
+                # (512 rows of the Qwen3-8B head: 8 x 363 us in the kernel below, 4 x 240 us in portions of
+                # 128 rows).  The last rows too, however few: a row's sums are then the same bits whatever
+                # the number of rows beside it in its block of 128, which a step replayed with rows that
+                # only fill it up relies on.
+                for m0 in range(0, M, self.MID_ROWS_TO_PLAIN):
+                    m1 = min(M, m0 + self.MID_ROWS_TO_PLAIN)
                     self._linear_mid(x[m0:m1], tiled, y[m0:m1], m1 - m0, N, K, 0)
                 return y
             if M <= self.SKINNY_ROWS or out_dtype == torch.float32:
