@@ -8,7 +8,7 @@ A step is one decode step of the engine (schedule, run the batch, sample,
 post-process).  One JSON line is printed.  Beside the headline, ``points`` holds (all
 with 128-token prompts unless the name says otherwise, tokens a second and the fraction of
 the HBM peak that the bytes a step has to read make of its time):
-  decode_b1, decode_b64                      a few steps at batch 1 and 64
+  decode_b1, decode_b64, decode_b256         a few steps at batch 1, 64 and 256
   decode_b{1,8,64}_128out                    all 128 output tokens of 128-token prompts
   decode_b{8,64}_ctx4096                     contexts that end at 4,096 tokens
   qwen3_14b_*, qwen3_32b_*                   decode at batch 8 and the prefill of 2,048 tokens at
@@ -70,6 +70,7 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip every point beside the headline")
     ap.add_argument("--no-other-shapes", action="store_true", help="skip the points at the layer sizes of the larger models")
+    ap.add_argument("--no-big-batch", action="store_true", help="skip the point at batch 256")
     ap.add_argument("--no-workloads", action="store_true", help="skip the two serving workloads at those sizes")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiles)")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement (for profiles)")
@@ -217,6 +218,16 @@ def main():
             d, _, f = decode_run(engine, cfg_json, b, n, 4, args.prompt_len)
             points[f"decode_b{b}"] = round(b * n / d, 2)
             points[f"decode_b{b}_hbm_frac"] = round(f, 4)
+        # a decode step of hundreds of requests, on an engine of its own over the same model (the cache
+        # of the first one is sized for 64 requests of the full context)
+        if not args.no_big_batch:
+            big = LLMEngine.from_model(model, max_model_len=args.context, page_size=page, max_num_seqs=256,
+                                       num_kv_blocks=256 * ((args.prompt_len + n + 64 + page - 1) // page) + 136,
+                                       max_num_batched_tokens=budget)
+            d, _, f = decode_run(big, cfg_json, 256, n, 4, args.prompt_len)
+            points["decode_b256"] = round(256 * n / d, 2)
+            points["decode_b256_hbm_frac"] = round(f, 4)
+            del big
         # every one of the 128 output tokens of 128-token prompts (the first token comes with the
         # prompt's last step); once untimed before, because the steps past 256 tokens are recorded anew
         for b in (1, 8, 64):
