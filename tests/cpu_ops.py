@@ -133,7 +133,7 @@ class CpuOps:
         h = cls._mix32(token ^ 0x9E3779B9)
         h = cls._mix32(h ^ lo)
         h = cls._mix32((h + hi * 0x85EBCA6B + 0x27D4EB2F) & 0xFFFFFFFF)
-        return ((h >> 8) + 0.5) / 16777216.0
+        return ((h >> 9) + 0.5) / 8388608.0
 
     def sample(self, logits, temperatures=None, seeds=None, top_p=None):
         import math

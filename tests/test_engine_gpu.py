@@ -155,6 +155,61 @@ def test_top_p_kernel_against_plain():
     assert got[5] == int(logits[5].argmax())        # a vanishing top_p keeps the best token only
 
 
+def test_top_p_over_a_large_vocabulary_against_the_rule():
+    """The top-p selection (a histogram of the weights over the logits' range, refined twice) over
+    vocabularies of 40,007 and 151,936 tokens, peaked and flat rows, temperatures from 0.3 to 2 and top_p
+    from 1e-4 to 0.999: for 24 seeds a row the drawn token is the best of the kept ones under the rule
+    written out in float64 (sort, running sum, threshold), with the same Gumbel noise."""
+    import numpy as np
+    from tiny_llm_infer_amd.kernels.ops import HipOps
+    ops = HipOps("cuda:0")
+
+    def uniforms(seed, n):
+        def mix(h):
+            h = h.copy()
+            h ^= h >> np.uint32(16); h *= np.uint32(0x85EBCA6B); h ^= h >> np.uint32(13)
+            h *= np.uint32(0xC2B2AE35); h ^= h >> np.uint32(16)
+            return h
+        lo, hi = np.uint32(seed & 0xFFFFFFFF), np.uint32(seed >> 32)
+        with np.errstate(over="ignore"):
+            h = mix(np.arange(n, dtype=np.uint32) ^ np.uint32(0x9E3779B9))
+            h = mix(h ^ lo)
+            h = mix(h + hi * np.uint32(0x85EBCA6B) + np.uint32(0x27D4EB2F))
+        return ((h >> np.uint32(9)).astype(np.float64) + 0.5) / 8388608.0
+
+    g = torch.Generator().manual_seed(5)
+    for vocab in (40007, 151936):
+        cases = []              # (logits, temperature, top_p)
+        for std, temp, tp in ((3.0, 0.7, 0.9), (3.0, 1.0, 0.5), (1.0, 2.0, 0.999), (8.0, 0.3, 0.95), (0.01, 1.0, 0.3),
+                              (3.0, 0.6, 1e-4), (5.0, 1.0, 0.05), (2.0, 1.5, 0.7)):
+            cases.append((torch.randn(vocab, generator=g) * std, temp, tp))
+        ties = torch.randn(vocab, generator=g).mul(4).round().div(4)               # many equal logits
+        cases.append((ties, 1.0, 0.6))
+        logits = torch.stack([c[0] for c in cases])
+        rows = len(cases)
+        temps = torch.tensor([c[1] for c in cases], dtype=torch.float32)
+        top_p = torch.tensor([c[2] for c in cases], dtype=torch.float32)
+        kept = []
+        for row, temp, tp in cases:
+            x = row.double().numpy()
+            w = np.exp((x - x.max()) / temp)
+            order = np.argsort(-x, kind="stable")
+            before = np.concatenate([[0.0], np.cumsum(w[order])[:-1]])             # weights of the tokens before each one
+            n = int((before < np.float64(np.float32(tp)) * w.sum()).sum())
+            edge = x[order[n - 1]]
+            kept.append((x >= edge, n))                                             # tokens equal to the last one kept share its fate
+        dev = logits.cuda()
+        for s in range(24):
+            seeds = torch.arange(rows, dtype=torch.int64) * 7919 + 1000003 * s + 17
+            got = ops.sample(dev, temps.cuda(), seeds.cuda(), top_p=top_p.cuda()).cpu().tolist()
+            for r, (row, temp, tp) in enumerate(cases):
+                x = row.double().numpy()
+                score = np.where(kept[r][0], x + temp * -np.log(-np.log(uniforms(int(seeds[r]), vocab))), -np.inf)
+                best = int(np.argmax(score))
+                assert kept[r][0][got[r]], f"vocabulary {vocab}, row {r}, seed {s}: token {got[r]} is not among the {kept[r][1]} kept"
+                assert got[r] == best or score[best] - score[got[r]] < 1e-5, (vocab, r, s, got[r], best)
+
+
 def test_command_line_infer(model_folders):
     folder = model_folders["A"]
     cfg, w = plain_qwen3.read_model(folder)

@@ -1172,9 +1172,17 @@ def test_sampling_a_large_vocabulary_in_pieces(ops):
             h = mix(np.arange(n, dtype=np.uint32) ^ np.uint32(0x9E3779B9))
             h = mix(h ^ lo)
             h = mix(h + hi * np.uint32(0x85EBCA6B) + np.uint32(0x27D4EB2F))
-        return ((h >> np.uint32(8)).astype(np.float64) + 0.5) / 16777216.0
+        return ((h >> np.uint32(9)).astype(np.float64) + 0.5) / 8388608.0
 
     assert abs(uniforms(12345, 10)[7] - sample_uniform(12345, 7)) < 1e-9
+    # every uniform lies strictly inside (0, 1), the hash's largest and smallest values included, so no
+    # token's Gumbel value is infinite: (k + 0.5) / 2^23 is a float32 as it stands for every k < 2^23
+    u = uniforms(99, 1 << 20)
+    assert all(sample_uniform(99, int(t)) == u[t] for t in (int(u.argmax()), int(u.argmin()), 0, 1, 12345))
+    assert 0.0 < u.min() and u.max() < 1.0 and np.all(u.astype(np.float32).astype(np.float64) == u)
+    ends = (np.array([0, 1, (1 << 23) - 2, (1 << 23) - 1], dtype=np.float32) + np.float32(0.5)) * np.float32(1.0 / 8388608.0)
+    assert ends.dtype == np.float32 and ends[0] > 0 and ends[-1] < 1 and np.all(np.diff(ends.astype(np.float64)) > 0)
+    assert np.isfinite(-np.log(-np.log(ends.astype(np.float64)))).all()
     for r in (0, 2):
         u = uniforms(int(seeds[r]), vocab)
         score = logits[r].double().numpy() + float(temps[r]) * -np.log(-np.log(u))

@@ -73,8 +73,7 @@ def test_sampling_without_allocation_matches_sampling_with_a_callers_scratch():
             h = mix(np.arange(n, dtype=np.uint32) ^ np.uint32(0x9E3779B9))
             h = mix(h ^ lo)
             h = mix(h + hi * np.uint32(0x85EBCA6B) + np.uint32(0x27D4EB2F))
-        # (in float32, as the kernel computes it: above 2^23 the half is rounded away)
-        return (((h >> np.uint32(8)).astype(np.float32) + np.float32(0.5)) * np.float32(1.0 / 16777216.0)).astype(np.float64)
+        return ((h >> np.uint32(9)).astype(np.float64) + 0.5) / 8388608.0
 
     lib.tli_sample_uniform.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32]
     lib.tli_sample_uniform.restype = ctypes.c_float

@@ -17,61 +17,136 @@ __host__ __device__ inline uint32_t tli_mix32(uint32_t h) {
     return h;
 }
 
-// uniform in (0, 1): 24 bits of a hash of (seed, token)
+// uniform in (0, 1): 23 bits of a hash of (seed, token) and a half, (k + 0.5) / 2^23.  Every such value is
+// a float32 as it stands, the largest 1 - 2^-24.  (With 24 bits the largest, 16777215.5, rounds to 2^24:
+// u = 1, a Gumbel value of +infinity, and that token drawn whatever its logit: one draw in a hundred over a
+// vocabulary of 150 thousand.)
 __host__ __device__ inline float tli_uniform(uint32_t seed_lo, uint32_t seed_hi, uint32_t token) {
     uint32_t h = tli_mix32(token ^ 0x9e3779b9u);
     h = tli_mix32(h ^ seed_lo);
     h = tli_mix32(h + seed_hi * 0x85ebca6bu + 0x27d4eb2fu);
-    return ((float)(h >> 8) + 0.5f) * (1.0f / 16777216.0f);
+    return ((float)(h >> 9) + 0.5f) * (1.0f / 8388608.0f);
 }
 
-__global__ void sample_kernel(const float* __restrict__ logits, int vocab,
+#define TOPP_BINS 4096
+#define TOPP_LEVELS 3
+
+// The bin of logit v in a range that begins at `hi` and goes down: TOPP_BINS bins of 1 / scale each (what
+// lies beyond the range falls into the first or the last bin).  Never smaller for a smaller v.
+__device__ __forceinline__ int topp_bin(float hi, float scale, float v) {
+    const float d = (hi - v) * scale;
+    return d <= 0.f ? 0 : (d >= (float)(TOPP_BINS - 1) ? TOPP_BINS - 1 : (int)d);
+}
+
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_kernel(const float* __restrict__ logits, int vocab,
                               const float* __restrict__ temperatures,
                               const uint32_t* __restrict__ seeds, const float* __restrict__ top_p,
                               int* __restrict__ out) {
     __shared__ float best_v[SAMPLE_THREADS / TLI_WAVE];
     __shared__ int best_i[SAMPLE_THREADS / TLI_WAVE];
     __shared__ float red[16];
+    __shared__ unsigned long long hist[TOPP_BINS], wave_sums[SAMPLE_THREADS / TLI_WAVE], crossing_above[1];
+    __shared__ int crossing[1];
     const int row = blockIdx.x;
     const float* l = logits + (size_t)row * vocab;
     const float temp = temperatures ? temperatures[row] : 0.f;
     const bool draw = temp > 1.0e-6f;
-    const uint32_t lo = seeds ? seeds[2 * row] : 0u, hi = seeds ? seeds[2 * row + 1] : 0u;
+    const uint32_t seed_lo = seeds ? seeds[2 * row] : 0u, seed_hi = seeds ? seeds[2 * row + 1] : 0u;
 
-    // top-p: the smallest logit that is kept.  A token is kept if the weights
-    // exp((l - max)/T) of all tokens strictly above it sum to less than
-    // top_p * total (engine/src/llm_engine.cpp:118-141: tokens are taken in
-    // descending order until the running sum reaches top_p * total).
-    float cutoff = -INFINITY;
+    // top-p (engine/src/llm_engine.cpp:118-141: tokens are taken in descending order until the running
+    // sum of their weights exp((l - max)/T) reaches top_p * total): a token is kept if the weights of all
+    // tokens strictly above it sum to less than top_p * total.  Found without sorting and in three passes
+    // over the row: the weights go into a histogram over the logits' range, 4,096 bins from the top; the
+    // bin in which the running sum reaches the threshold is cut into 4,096 bins again, and that one once
+    // more.  Tokens above the last such bin are kept, tokens below it are not, and the tokens in it (logits
+    // within 2^-36 of the row's range of each other) count as tied with its first, which is kept.  The
+    // weights are summed as 64-bit integers (units of 2^-40), so the sums do not depend on the order in
+    // which the threads add.
+    float hi[TOPP_LEVELS], scale[TOPP_LEVELS];
+    int star[TOPP_LEVELS];
+    int levels = 0;
     if (draw && top_p && top_p[row] < 1.0f) {
         float mx = -INFINITY, mn = INFINITY;
         for (int t = threadIdx.x; t < vocab; t += blockDim.x) { mx = fmaxf(mx, l[t]); mn = fminf(mn, l[t]); }
         mx = block_max(mx, red);
         mn = -block_max(-mn, red);
-        const float inv_t = 1.0f / temp;
-        float total = 0.f;
-        for (int t = threadIdx.x; t < vocab; t += blockDim.x) total += expf((l[t] - mx) * inv_t);
-        total = block_sum(total, red);
-        const float theta = top_p[row] * total;
-        float below = mn - 1.0f, above = mx;       // f(below) >= theta, f(above) = 0 < theta
-        for (int it = 0; it < 64; ++it) {
-            const float mid = below + (above - below) * 0.5f;
-            if (!(mid > below && mid < above)) break;
-            float f = 0.f;
-            for (int t = threadIdx.x; t < vocab; t += blockDim.x)
-                if (l[t] > mid) f += expf((l[t] - mx) * inv_t);
-            f = block_sum(f, red);
-            if (f < theta) above = mid; else below = mid;
+        if (mx > mn) {
+            const float inv_t = 1.0f / temp;
+            unsigned long long above = 0, theta = 0;          // weights above the range in hand; the threshold
+            hi[0] = mx;
+            scale[0] = (float)TOPP_BINS / (mx - mn);
+            for (int lev = 0; lev < TOPP_LEVELS; ++lev) {
+                for (int b = threadIdx.x; b < TOPP_BINS; b += blockDim.x) hist[b] = 0;
+                __syncthreads();
+                for (int t = threadIdx.x; t < vocab; t += blockDim.x) {
+                    const float v = l[t];
+                    bool in = true;
+                    for (int k = 0; k < lev; ++k) in = in && topp_bin(hi[k], scale[k], v) == star[k];
+                    if (in)
+                        atomicAdd(&hist[topp_bin(hi[lev], scale[lev], v)],
+                                  (unsigned long long)(expf((v - mx) * inv_t) * 1099511627776.0f));
+                }
+                __syncthreads();
+                // running sums over the bins: a thread has TOPP_BINS / SAMPLE_THREADS bins in a row
+                constexpr int MINE = TOPP_BINS / SAMPLE_THREADS;
+                unsigned long long mine = 0;
+                for (int j = 0; j < MINE; ++j) mine += hist[threadIdx.x * MINE + j];
+                unsigned long long incl = mine;
+                const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE;
+                for (int off = 1; off < TLI_WAVE; off <<= 1) {
+                    const unsigned long long up = __shfl_up(incl, off, TLI_WAVE);
+                    if (lane >= off) incl += up;
+                }
+                if (lane == TLI_WAVE - 1) wave_sums[wave] = incl;
+                if (threadIdx.x == 0) crossing[0] = -1;
+                __syncthreads();
+                unsigned long long before = above, all = 0;
+                for (int w = 0; w < SAMPLE_THREADS / TLI_WAVE; ++w) {
+                    if (w < wave) before += wave_sums[w];
+                    all += wave_sums[w];
+                }
+                if (lev == 0) {
+                    theta = (unsigned long long)((double)top_p[row] * (double)all);
+                    if (theta < 1) theta = 1;
+                }
+                unsigned long long run = before + incl - mine;        // weights above this thread's first bin
+                for (int j = 0; j < MINE; ++j) {
+                    const unsigned long long h = hist[threadIdx.x * MINE + j];
+                    if (run < theta && run + h >= theta) {             // (one bin of the row: the sums only grow)
+                        crossing[0] = threadIdx.x * MINE + j;
+                        crossing_above[0] = run;
+                    }
+                    run += h;
+                }
+                __syncthreads();
+                if (crossing[0] < 0) break;                            // (cannot be: the last running sum is the total)
+                star[lev] = crossing[0];
+                above = crossing_above[0];
+                levels = lev + 1;
+                if (lev + 1 < TOPP_LEVELS) {
+                    hi[lev + 1] = hi[lev] - (float)star[lev] / scale[lev];
+                    scale[lev + 1] = scale[lev] * (float)TOPP_BINS;
+                }
+                __syncthreads();                                       // (everyone has read the crossing)
+            }
         }
-        cutoff = above;
     }
 
     float bv = -INFINITY;
     int bi = 0x7fffffff;
     for (int t = threadIdx.x; t < vocab; t += blockDim.x) {
         float s = l[t];
-        if (s < cutoff) continue;
-        if (draw) s += temp * -logf(-logf(tli_uniform(lo, hi, (uint32_t)t)));
+        bool kept = true;
+        for (int k = 0; k < levels; ++k) {
+            const int b = topp_bin(hi[k], scale[k], s);
+            if (b != star[k]) {
+                kept = b < star[k];
+                break;
+            }
+        }
+        if (!kept) continue;
+        if (draw) s += temp * -logf(-logf(tli_uniform(seed_lo, seed_hi, (uint32_t)t)));
         if (s > bv || (s == bv && t < bi)) { bv = s; bi = t; }
     }
     for (int off = TLI_WAVE / 2; off > 0; off >>= 1) {
