@@ -28,6 +28,24 @@ __host__ __device__ inline float tli_uniform(uint32_t seed_lo, uint32_t seed_hi,
     return ((float)(h >> 9) + 0.5f) * (1.0f / 8388608.0f);
 }
 
+// f(token, logit) for the tokens t = threadIdx.x, threadIdx.x + blockDim.x, ..: eight loads are asked for
+// before the first is used (one workgroup walks a whole row of 150 thousand logits: what bounds it is the
+// wait for its loads).
+template <typename F>
+__device__ __forceinline__ void for_each_logit(const float* __restrict__ l, int begin, int end, F&& f) {
+    constexpr int U = 8;
+    const int stride = blockDim.x;
+    int t = begin + threadIdx.x;
+    for (; t + (U - 1) * stride < end; t += U * stride) {
+        float v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = l[t + u * stride];
+#pragma unroll
+        for (int u = 0; u < U; ++u) f(t + u * stride, v[u]);
+    }
+    for (; t < end; t += stride) f(t, l[t]);
+}
+
 #define TOPP_BINS 4096
 #define TOPP_LEVELS 3
 
@@ -68,7 +86,7 @@ sample_kernel(const float* __restrict__ logits, int vocab,
     int levels = 0;
     if (draw && top_p && top_p[row] < 1.0f) {
         float mx = -INFINITY, mn = INFINITY;
-        for (int t = threadIdx.x; t < vocab; t += blockDim.x) { mx = fmaxf(mx, l[t]); mn = fminf(mn, l[t]); }
+        for_each_logit(l, 0, vocab, [&](int, float v) { mx = fmaxf(mx, v); mn = fminf(mn, v); });
         mx = block_max(mx, red);
         mn = -block_max(-mn, red);
         if (mx > mn) {
@@ -79,14 +97,13 @@ sample_kernel(const float* __restrict__ logits, int vocab,
             for (int lev = 0; lev < TOPP_LEVELS; ++lev) {
                 for (int b = threadIdx.x; b < TOPP_BINS; b += blockDim.x) hist[b] = 0;
                 __syncthreads();
-                for (int t = threadIdx.x; t < vocab; t += blockDim.x) {
-                    const float v = l[t];
+                for_each_logit(l, 0, vocab, [&](int, float v) {
                     bool in = true;
                     for (int k = 0; k < lev; ++k) in = in && topp_bin(hi[k], scale[k], v) == star[k];
                     if (in)
                         atomicAdd(&hist[topp_bin(hi[lev], scale[lev], v)],
                                   (unsigned long long)(expf((v - mx) * inv_t) * 1099511627776.0f));
-                }
+                });
                 __syncthreads();
                 // running sums over the bins: a thread has TOPP_BINS / SAMPLE_THREADS bins in a row
                 constexpr int MINE = TOPP_BINS / SAMPLE_THREADS;
@@ -135,8 +152,7 @@ sample_kernel(const float* __restrict__ logits, int vocab,
 
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int t = threadIdx.x; t < vocab; t += blockDim.x) {
-        float s = l[t];
+    for_each_logit(l, 0, vocab, [&](int t, float s) {
         bool kept = true;
         for (int k = 0; k < levels; ++k) {
             const int b = topp_bin(hi[k], scale[k], s);
@@ -145,10 +161,10 @@ sample_kernel(const float* __restrict__ logits, int vocab,
                 break;
             }
         }
-        if (!kept) continue;
+        if (!kept) return;
         if (draw) s += temp * -logf(-logf(tli_uniform(seed_lo, seed_hi, (uint32_t)t)));
         if (s > bv || (s == bv && t < bi)) { bv = s; bi = t; }
-    }
+    });
     for (int off = TLI_WAVE / 2; off > 0; off >>= 1) {
         const float ov = __shfl_xor(bv, off, TLI_WAVE);
         const int oi = __shfl_xor(bi, off, TLI_WAVE);
@@ -185,11 +201,10 @@ __global__ void sample_chunks_kernel(const float* __restrict__ logits, int vocab
     const int begin = chunk * per, end = min(vocab, begin + per);
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int t = begin + threadIdx.x; t < end; t += blockDim.x) {
-        float s = l[t];
+    for_each_logit(l, begin, end, [&](int t, float s) {
         if (draw) s += temp * -logf(-logf(tli_uniform(lo, hi, (uint32_t)t)));
         if (s > bv || (s == bv && t < bi)) { bv = s; bi = t; }
-    }
+    });
     for (int off = TLI_WAVE / 2; off > 0; off >>= 1) {
         const float ov = __shfl_xor(bv, off, TLI_WAVE);
         const int oi = __shfl_xor(bi, off, TLI_WAVE);
