@@ -220,6 +220,7 @@ class CacheManager:
                 self.groups.append(g)
             g.cache_layers.append(layer)
             self.group_of_layer[layer] = g.index
+        self._no_window = all(g.need.window is None for g in self.groups)
         self._free_slots = list(range(max_requests - 1, -1, -1))   # pop() gives the lowest
         self._live: Dict[Hashable, RequestCache] = {}
         self.pages_taken_total = 0
@@ -349,8 +350,10 @@ class CacheManager:
         """Per group, pages that must be taken so that the request can run the
         tokens at positions [num_tokens, new_total)."""
         rc = self._live[key]
-        out = []
         nb = _blocks(new_total, self.page_size)
+        if self._no_window:                   # (every step of every request comes through here: the short way)
+            return [max(0, nb - len(table)) for table in rc.tables]
+        out = []
         for gi, g in enumerate(self.groups):
             # every block from the first one a query at num_tokens reads up to the table's end is
             # held (``reserve`` filled them, ``advance`` gives back only what lies before): what is
@@ -412,7 +415,12 @@ class CacheManager:
         rc = self._live[key]
         if new_total < rc.num_tokens:
             raise ValueError("a request cannot shrink")
-        if not self.can_reserve(key, new_total):
+        needs = self.pages_needed(key, new_total)
+        if not any(needs) and self._no_window:            # a token that goes into a page already held
+            if new_total > rc.reserved_tokens:
+                rc.reserved_tokens = new_total
+            return
+        if any(n > g.pool.free_count for n, g in zip(needs, self.groups)):
             raise CacheFull(f"not enough free pages to hold {new_total} tokens of {key!r}")
         nb = _blocks(new_total, self.page_size)
         for gi, g in enumerate(self.groups):
