@@ -236,3 +236,46 @@ def test_a_step_is_told_how_unequal_its_sequences_are(model_folders):
     assert view.num_seqs == 8 and view.skew == 4                      # 101 against (101 + 6 + 6 + 7 + 4) / 8
     view = runner._pack([StepEntry(k, [1], [0]) for k in ("a", "b", "c")])
     assert view.skew == 1
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_serving_scenarios_give_plain_greedy_tokens(model_folders, seed):
+    """A scenario drawn from the seed: one of the tiny configurations, a page size, up to eight requests of
+    1 to 69 prompt tokens and 1 to 13 new ones, a pool between barely enough for the longest request and
+    enough for all, a token budget from 2 to 256, a limit of live requests, steps planned ahead or not,
+    prefix caching (with a shared prefix) where no layer has a window, requests that arrive while others
+    are served.  Every request gets the tokens of plain greedy generation, whatever was preempted and
+    computed again on the way, and the cache is whole at the end."""
+    import random
+    rng = random.Random(1000 + seed)
+    name = rng.choice(sorted(TINY))
+    cfg, w = plain_qwen3.read_model(model_folders[name])
+    vocab = TINY[name]["vocab_size"]
+    page = rng.choice([4, 8, 16, 32]) if rng.random() < 0.5 else TINY[name]["page_size"]
+    nreq = rng.randrange(1, 9)
+    prompts = [random_prompt(vocab, rng.randrange(1, 70), rng.randrange(10 ** 6)) for _ in range(nreq)]
+    outs = [rng.randrange(1, 14) for _ in range(nreq)]
+    prefix = not TINY[name].get("use_sliding_window", False) and rng.random() < 0.5
+    if prefix:
+        head = random_prompt(vocab, rng.randrange(1, 40), 7)
+        prompts = [head + p for p in prompts]
+    need = (max(len(p) + o for p, o in zip(prompts, outs)) + page - 1) // page + 2
+    pool = rng.choice([need, need + 1, need * 2, need * nreq + 4]) + rng.randrange(0, 4)
+    eng = _engine(model_folders[name], name, max_model_len=256, page_size=page, num_kv_blocks=pool,
+                  max_num_seqs=rng.randrange(1, nreq + 2), max_num_batched_tokens=rng.choice([2, 3, 8, 17, 64, 256]),
+                  enable_prefix_caching=prefix)
+    eng.lookahead = rng.random() < 0.6
+    arrive = rng.choice([0, 0, 1, 3])
+    results, index_of, admitted, steps = {}, {}, 0, 0
+    while admitted < nreq or not eng.is_finished():
+        while admitted < nreq and (steps >= arrive * admitted or eng.is_finished()):
+            index_of[eng.add_request(prompts[admitted], SamplingParams(max_tokens=outs[admitted], ignore_eos=True))] = admitted
+            admitted += 1
+        for r in eng.step():
+            results[index_of[r.request_id]] = list(r.token_ids)
+        steps += 1
+        assert steps < 5000, "no progress"
+    for i in range(nreq):
+        assert results[i] == list(plain_qwen3.greedy(cfg, w, prompts[i], outs[i])), (name, i)
+    eng.runner.cache.check()
+    assert eng.runner.cache.free_pages() == eng.runner.cache.pages_per_group()
