@@ -235,7 +235,7 @@ def test_two_row_blocks_side_by_side_in_the_x_sharing_kernel(ops, mnk):
     assert torch.equal(ops.linear(xd, Both), first)
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 6])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("mnk", [(129, 264, 1008), (300, 4096, 4096), (2048, 6144, 512), (513, 1000, 136), (700, 48, 8), (4500, 520, 256),
                                  (1024, 5120, 384)])
 def test_product_of_many_rows_from_the_decode_layout(ops, mnk, cfg):

@@ -423,6 +423,9 @@ static int rows_pick(int M, int N, int K, int splits, int gated) {
     const long k_steps = (K + 127) / 128, per = (k_steps + splits - 1) / splits;
     const double cost2 = shared(a_die(16)) * 256.0, cost4 = shared(a_die(12)) * 192.0 * 1.06;
     const double cost3 = alone(a_die(32)) * 512.0 * 0.84, cost6 = alone(a_die(16)) * 256.0 * 0.88;
+    // 128 x 384 outputs in eight waves of three column tiles (one workgroup a compute unit, not for gated
+    // products): 0.82 a column; 5,120 columns are 14 such groups, 6,144 are 16
+    const double cost5 = alone(a_die(24)) * 384.0 * 0.82;
     // (from three rounds of the 512-column shape on, it was the fastest at every layer size measured:
     // the costs above are those of the first rounds)
     if (alone(a_die(32)) >= 3.0) return 3;
@@ -430,6 +433,7 @@ static int rows_pick(int M, int N, int K, int splits, int gated) {
     double cost = cost2;
     if (cost3 < cost) { best = 3; cost = cost3; }
     if (!gated && cost4 < cost) { best = 4; cost = cost4; }
+    if (!gated && cost5 < cost) { best = 5; cost = cost5; }
     if (!gated && per % 2 == 0 && k_steps % per == 0 && cost6 < cost) best = 6;
     return best;
 }
@@ -441,9 +445,9 @@ static int rows_pick(int M, int N, int K, int splits, int gated) {
 // (tli_gemm_mid_reduce, or tli_add_rmsnorm).
 // cfg 0 picks the launch shape; 1: 256 x 256 outputs a workgroup of eight waves, 2: 128 x 256
 // and four waves, two workgroups a compute unit, 3: 128 x 512 and eight waves, 4: 128 x 192 and
-// four waves (not for a gated product), 6: 128 x 256 by two sets of four waves that take the
-// slices of k in turn; cfg >= 10: the tens for a gated product, the ones for the others
-// (measurements).
+// four waves (not for a gated product), 5: 128 x 384 and eight waves (not for a gated product), 6: 128 x 256
+// by two sets of four waves that take the slices of k in turn; cfg >= 10: the tens for a gated product, the
+// ones for the others (measurements).
 extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, float* part, int M, int N, int K,
                                   int gated, int splits, int cfg, void* stream) {
     if (M <= 0 || N <= 0) return 0;
@@ -471,6 +475,10 @@ extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, float* 
     if (cfg == 4) {
         if (gated) return tli_fail("gemm_rows: three column tiles a wave do not pair up for a gated product");
         return launch_rows<3, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
+    }
+    if (cfg == 5) {
+        if (gated) return tli_fail("gemm_rows: three column tiles a wave do not pair up for a gated product");
+        return launch_rows<3, 8, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     }
     return tli_fail("gemm_rows: unknown configuration %d", cfg);
 }
