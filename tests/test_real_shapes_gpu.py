@@ -3,7 +3,8 @@ larger models of the family (Qwen3-14B: hidden 5120, 40 query heads, intermediat
 Qwen3-32B: hidden 5120, 64 query heads of 128 so that q is wider than the hidden size,
 intermediate 25600), for 1 to 300 rows: every tuned kernel (the weight-streaming ones for
 up to 16 rows with and without the norms taken in, the one for 17..128 rows with its split
-of k, the one for more rows, and the library) beside the plain float32 kernel on the same
+of k and, for products without a gate, up to 256 rows as two row blocks, the one for more rows,
+and the library) beside the plain float32 kernel on the same
 bfloat16 values.  How the tuned kernels deal tiles and cut k depends on N and K, so shapes
 that the smaller model never shows are compared here."""
 import pytest
@@ -14,7 +15,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 BF = torch.bfloat16
 SHAPES = {"14B": dict(H=5120, Q=5120, KV=1024, I=17408), "32B": dict(H=5120, Q=8192, KV=1024, I=25600)}
-ROWS = [1, 8, 16, 64, 128, 300]
+ROWS = [1, 8, 16, 64, 128, 200, 256, 300]
 
 
 @pytest.fixture(scope="module")
