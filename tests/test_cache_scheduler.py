@@ -333,6 +333,114 @@ def test_a_prompt_larger_than_the_pool_is_an_error_and_a_stuck_queue_too():
         s.schedule()
 
 
+def _launch(sched, plan):
+    """What putting a step on the device does to the cache (the host's side of it)."""
+    for item in plan.items:
+        sched.cache.reserve(item.seq.request_id, item.first + item.count)
+        sched.cache.advance(item.seq.request_id, item.first + item.count)
+
+
+def _shape(plan):
+    return [(i.seq.request_id, i.first, i.count, i.prompt_portion) for i in plan.items]
+
+
+def test_a_step_planned_ahead_goes_on_with_prompts_beside_decoding():
+    """While a step runs, the next one is planned from what that step will leave: the request
+    whose prompt ends in it decodes (its token is still on the device), the other's prompt goes
+    on after the portion that runs.  A request that is not admitted yet ends the look ahead."""
+    cache = CacheManager([FULL], page_size=8, num_pages=100, max_requests=4)
+    s = Scheduler(SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=24), cache)
+    a, b = _seq(1, 50), _seq(2, 10)
+    s.add(a)
+    s.add(b)
+    p0 = s.schedule()
+    assert _shape(p0) == [(1, 0, 24, True)]
+    _launch(s, p0)
+    assert s.plan_ahead(p0) is None           # b is next and holds nothing yet
+    s.postprocess(p0, [None], lambda t: False)
+    p1 = s.schedule()                         # b first (a went to the back), then a from token 24 on
+    assert _shape(p1) == [(2, 0, 10, True), (1, 24, 14, True)]
+    _launch(s, p1)
+    p2 = s.plan_ahead(p1)                     # b decodes at position 10 with the token p1 samples
+    assert _shape(p2) == [(2, 10, 1, False), (1, 38, 12, True)]
+    assert [i.samples for i in p2.items] == [True, True] and p2.num_tokens == 13
+    assert a.status == Status.RUNNING and list(s.running) == [b, a] and not s.waiting
+    assert a.tokens_in_cache == 24            # what p1 and p2 run is counted when their results come in
+    _launch(s, p2)
+    s.postprocess(p1, [7, None], lambda t: False)
+    assert b.token_ids[-1] == 7 and b.size == 11 and a.tokens_in_cache == 38
+    p3 = s.plan_ahead(p2)                     # both decode, fed on the device
+    assert _shape(p3) == [(2, 11, 1, False), (1, 50, 1, False)]
+    _launch(s, p3)
+    s.postprocess(p2, [8, 9], lambda t: False)
+    c = _seq(3, 5)
+    s.add(c)                                  # arrives now: not admitted, so the next plan waits for p3's end
+    assert s.plan_ahead(p3) is None
+    s.postprocess(p3, [8, 9], lambda t: False)
+    assert _shape(s.schedule()) == [(2, 12, 1, False), (1, 51, 1, False), (3, 0, 5, True)]
+    cache.check()
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_steps_planned_ahead_are_the_steps_planned_afterwards(seed):
+    """Two schedulers serve the same random requests (several groups of layers, small pools,
+    budgets from 2 tokens, arrivals on the way): one plans every step after the one before has
+    been post-processed, the other plans ahead wherever ``plan_ahead`` gives a plan.  Without
+    end-of-sequence tokens both run the same steps, and no page is lost."""
+    rng = random.Random(300 + seed)
+    needs = [FULL, WIN] if rng.random() < 0.5 else [FULL]
+    page = rng.choice([4, 8, 16])
+    budget = rng.choice([2, 5, 16, 40])
+    nreq = rng.randrange(1, 9)
+    lens = [rng.randrange(1, 90) for _ in range(nreq)]
+    outs = [rng.randrange(1, 9) for _ in range(nreq)]
+    most = max((n + o + page - 1) // page for n, o in zip(lens, outs)) + 1
+    pages = rng.choice([most, most + 2, 3 * most, most * nreq + 2])
+    seqs = rng.randrange(1, 6)
+    arrive = [rng.randrange(0, 12) for _ in range(nreq)]
+
+    def serve(ahead):
+        cache = CacheManager(needs, page_size=page, num_pages=pages, max_requests=seqs, max_step_tokens=budget)
+        s = Scheduler(SchedulerConfig(max_num_seqs=seqs, max_num_batched_tokens=budget), cache)
+
+        def arrivals(n):                      # the requests that are there when plan number n is made
+            for i in range(nreq):
+                if arrive[i] == n:
+                    s.add(_seq(i, lens[i], max_tokens=outs[i]))
+
+        plans, planned_ahead, inflight = [], 0, None
+        for n in range(2000):
+            if inflight is None:
+                arrivals(n)
+                if s.is_finished():
+                    if n > max(arrive):
+                        break
+                    plans.append([])
+                    continue
+                inflight = s.schedule()
+                _launch(s, inflight)
+            cur, inflight = inflight, None
+            plans.append(_shape(cur))
+            if ahead:
+                before = len(s.waiting)
+                arrivals(n + 1)
+                inflight = s.plan_ahead(cur)
+                if inflight is not None:
+                    planned_ahead += 1
+                    _launch(s, inflight)
+                else:                         # they arrive again when the plan is made the ordinary way
+                    while len(s.waiting) > before:
+                        s.waiting.pop()
+            s.postprocess(cur, [1 if i.samples else None for i in cur.items], lambda t: False)
+            cache.check()
+        assert s.is_finished() and cache.free_pages() == cache.pages_per_group()
+        return plans, planned_ahead
+
+    plain, _ = serve(False)
+    looked, planned_ahead = serve(True)
+    assert looked == plain
+
+
 # ------------------------------------------------------------ prefix caching --
 def test_page_hash_is_chained_fnv1a():
     from tiny_llm_infer_amd.cache.manager import page_hash

@@ -481,3 +481,44 @@ def test_a_request_that_ends_while_its_next_step_is_on_the_device(model_folders,
         assert len(outs[1][1]) <= 7
         if dtype == "float32":
             assert runs == [plain_qwen3.greedy(cfg, w, p, 14) for p in prompts]
+
+
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_steps_with_prompt_portions_are_launched_ahead_too(model_folders, name):
+    """A budget of 7 tokens and three live requests among five: while prompts go through in
+    portions beside decoding requests, and while requests wait for a place, the next step is on
+    the device before this one's tokens are read, its decoding rows fed on the device.  Greedy
+    float32 tokens are the plain ones; drawn tokens (seeded) and an end-of-sequence stop are
+    those of the engine that launches nothing ahead."""
+    from tiny_llm_infer_amd.sampling.params import SamplingParams
+    folder = model_folders[name]
+    cfg, w = plain_qwen3.read_model(folder)
+    vocab = TINY[name]["vocab_size"]
+    prompts = [random_prompt(vocab, n, 80 + n) for n in (23, 4, 31, 12, 18)]
+    want = [plain_qwen3.greedy(cfg, w, p, 10) for p in prompts]
+    params = [SamplingParams(max_tokens=10, temperature=t, seed=3 + i, ignore_eos=(i != 2))
+              for i, t in enumerate([0.0, 0.7, 0.0, 0.0, 0.9])]
+    outs = []
+    for ahead in (False, True):
+        eng = _engine(folder, name, "float32", max_num_batched_tokens=7, max_num_seqs=3)
+        eng.lookahead = ahead
+        eng.eos_token_ids = {want[2][5]}                  # request 2 stops in the middle of its run
+        for p, sp in zip(prompts, params):
+            eng.add_request(p, sp)
+        mixed_ahead, results = 0, []
+        while not eng.is_finished():
+            results.extend(eng.step())
+            nxt = eng._inflight
+            if nxt is not None and any(i.prompt_portion for i in nxt.plan.items) \
+                    and any(not i.prompt_portion for i in nxt.plan.items):
+                mixed_ahead += 1
+        assert (mixed_ahead > 3) == ahead
+        results.sort(key=lambda r: r.request_id)
+        outs.append([r.token_ids for r in results])
+        eng.runner.cache.check()
+        assert eng.runner.cache.free_pages() == eng.runner.cache.pages_per_group()
+    assert outs[0] == outs[1]
+    for i in (0, 3):
+        assert outs[1][i] == want[i]
+    assert outs[1][2] == want[2][:want[2].index(want[2][5]) + 1]
+    assert outs[1][1] != want[1] and outs[1][4] != want[4]          # the draws are draws

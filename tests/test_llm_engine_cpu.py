@@ -139,24 +139,38 @@ def test_prefix_caching_gives_the_same_tokens_and_skips_work(model_folders):
     assert small.runner.cache.free_pages() == [14]
 
 
-def test_steps_put_on_the_device_ahead_change_nothing(model_folders):
-    """The next decode step is launched before this step's tokens are read; requests
-    that stop on an end-of-sequence token or at max_tokens meanwhile, and sampling
-    with a temperature, give exactly what the step-by-step engine gives."""
+@pytest.mark.parametrize("budget", [64, 7])
+def test_steps_put_on_the_device_ahead_change_nothing(model_folders, budget):
+    """The next step is launched before this step's tokens are read; requests that
+    stop on an end-of-sequence token or at max_tokens meanwhile, and sampling with a
+    temperature, give exactly what the step-by-step engine gives.  With the small
+    budget the steps ahead carry portions of prompts beside the decoding requests."""
     folder = model_folders["B"]
     prompts = [random_prompt(384, n, 50 + n) for n in (4, 30, 17, 9)]
     params = [SamplingParams(max_tokens=m, temperature=t, seed=7 + i)
               for i, (m, t) in enumerate([(9, 0.0), (14, 0.8), (3, 0.0), (11, 0.5)])]
     outs = []
     for ahead in (False, True):
-        eng = _engine(folder, "B", max_num_batched_tokens=64)
+        eng = _engine(folder, "B", max_num_batched_tokens=budget)
         eng.lookahead = ahead
-        free = _engine(folder, "B", max_num_batched_tokens=64).generate([prompts[0]], [SamplingParams(max_tokens=9)])
+        free = _engine(folder, "B", max_num_batched_tokens=budget).generate([prompts[0]], [SamplingParams(max_tokens=9)])
         eng.eos_token_ids = {free[0].token_ids[4]}            # request 0 stops early on this token
-        outs.append(eng.generate(prompts, params))
+        mixed_ahead = 0
+        for p, sp in zip(prompts, params):
+            eng.add_request(p, sp)
+        results = []
+        while not eng.is_finished():
+            results.extend(eng.step())
+            nxt = eng._inflight
+            if nxt is not None and any(i.prompt_portion for i in nxt.plan.items) \
+                    and any(not i.prompt_portion for i in nxt.plan.items):
+                mixed_ahead += 1
+        results.sort(key=lambda r: r.request_id)
+        outs.append(results)
         assert (eng.num_steps_ahead > 5) == ahead
+        assert (mixed_ahead > 2) == (ahead and budget == 7)
         eng.runner.cache.check()
-        assert eng.runner.cache.free_pages() == [64, 24] and eng.is_finished()     # (the window group's pool is the smaller one)
+        assert eng.runner.cache.free_pages() == eng.runner.cache.pages_per_group() and eng.is_finished()
     assert [r.token_ids for r in outs[0]] == [r.token_ids for r in outs[1]]
     assert len(outs[1][0].token_ids) <= 5 and len(outs[1][2].token_ids) <= 3
 

@@ -60,7 +60,7 @@ class LLMEngine:
         self.total_generated_tokens = 0
         self.num_steps = 0
         self.num_steps_ahead = 0
-        self.lookahead = True                # put the next decode step on the device before reading this one
+        self.lookahead = True                # put the next step on the device before reading this one
         self._inflight: Optional[_Inflight] = None
 
     # ---- construction ---------------------------------------------------------
@@ -164,28 +164,31 @@ class LLMEngine:
     # ---- one step -------------------------------------------------------------------
     def _launch(self, plan: StepPlan, ahead_of: Optional["_Inflight"] = None) -> "_Inflight":
         """Put one planned step on the device: the batch, then the sampling.  Nothing
-        is waited for.  With ``ahead_of``, every item's token is the one that step
-        sampled for the same request and is taken on the device."""
+        is waited for.  With ``ahead_of``, the token of every decoding request is the
+        one that step sampled for it and is taken on the device; portions of prompts
+        are known on the host as ever."""
         entries, sampled_items = [], []
+        fed = {} if ahead_of is None else ahead_of.row_of
         for i, item in enumerate(plan.items):
             seq = item.seq
             want = [item.count - 1] if item.samples else []
-            if ahead_of is None:
-                toks = seq.token_ids[item.first:item.first + item.count]
-                entries.append(StepEntry(seq.request_id, toks, want))
+            if not item.prompt_portion and seq.request_id in fed:
+                entries.append(StepEntry(seq.request_id, [0], want, token_from=fed[seq.request_id]))
             else:
-                entries.append(StepEntry(seq.request_id, [0], want, token_from=ahead_of.row_of[seq.request_id]))
+                toks = seq.token_ids[item.first:item.first + item.count]
+                if len(toks) != item.count:
+                    raise RuntimeError(f"request {seq.request_id}: tokens {item.first} to {item.first + item.count} are planned, it has {seq.size}")
+                entries.append(StepEntry(seq.request_id, toks, want))
             if item.samples:
                 sampled_items.append(i)
-        logits = self.runner.step(entries, feed=None if ahead_of is None else ahead_of.tokens)
+        logits = self.runner.step(entries, feed=ahead_of.tokens if fed else None)
         tokens = None
         row_of = {}
         if sampled_items:
             seqs = [plan.items[i].seq for i in sampled_items]
             # a request whose previous draw is still on the device has one more sample behind it
-            extra = 0 if ahead_of is None else 1
             tokens = self.sampler.launch(logits, [s.sampling for s in seqs], [s.rng_seed for s in seqs],
-                                         [s.num_sampled + extra for s in seqs])
+                                         [s.num_sampled + (1 if s.request_id in fed else 0) for s in seqs])
             row_of = {s.request_id: j for j, s in enumerate(seqs)}
         return _Inflight(plan, sampled_items, tokens, row_of, self._read_back(tokens))
 
@@ -203,9 +206,9 @@ class LLMEngine:
     def step(self) -> List[GenerationResult]:
         """One step of the engine (engine/src/llm_engine.cpp:148-248): schedule, run the
         batch, sample, post-process.  When the step after this one is already known
-        (decode only, see Scheduler.plan_ahead) it is put on the device before this
-        step's tokens are read back, fed on the device with the tokens sampled here,
-        so the device does not wait for the host between steps."""
+        (see Scheduler.plan_ahead) it is put on the device before this step's tokens
+        are read back, its decoding requests fed on the device with the tokens sampled
+        here, so the device does not wait for the host between steps."""
         cur = self._inflight
         if cur is None:
             with self._lock:
@@ -214,7 +217,7 @@ class LLMEngine:
                 return []
             cur = self._launch(plan)
         nxt = None
-        if self.lookahead and cur.tokens is not None:
+        if self.lookahead:
             with self._lock:
                 ahead = self.scheduler.plan_ahead(cur.plan)
             if ahead is not None:

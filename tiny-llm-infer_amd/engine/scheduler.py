@@ -81,35 +81,79 @@ class Scheduler:
 
     def plan_ahead(self, plan: StepPlan) -> Optional[StepPlan]:
         """The plan of the step after ``plan``, made while ``plan`` is still running on
-        the device, or None if it cannot be known yet.  It can when the next step is
-        decode only: nothing waits, ``plan`` covers every running request and every item
-        of it samples (so each request needs exactly its next token), and the pages for
-        those tokens are free.  A request that reaches ``max_tokens`` with the running
-        step is left out; one that will stop on an end-of-sequence token cannot be known
-        and is skipped when its result comes in."""
-        if self.waiting or len(plan.items) != len(self.running) or not plan.items:
+        the device, or None if it cannot be known yet.  It is what ``schedule`` would
+        give once ``plan`` has been post-processed, as far as that can be told now:
+
+        - every running request is in ``plan`` and is sampled there, so its next token
+          (which the host does not know yet) can be fed on the device; it decodes one
+          token, unless the running step's token is its last by ``max_tokens``.  One that
+          will stop on an end-of-sequence token cannot be known and is skipped when its
+          result comes in;
+        - waiting requests that hold their pages already go on with their prompts, in the
+          same order and under the same budget, starting after the portion that ``plan``
+          runs.  A request that is not admitted yet ends the look ahead: admission takes
+          pages and a slot, and which are free is known after ``plan``;
+        - the pages for all of it are free.  The requests compete for the same pools, so
+          the whole step is counted before anything is taken; if it does not fit, nothing
+          is taken and the ordinary path decides who waits and who is preempted."""
+        if not plan.items:
             return None
-        if any(not item.samples or item.seq.status == Status.FINISHED for item in plan.items):
-            return None
+        in_plan = {}
+        for item in plan.items:
+            if item.seq.status == Status.FINISHED:
+                return None
+            in_plan[id(item.seq)] = item
+        cfg = self.config
+        budget = cfg.max_num_batched_tokens
         ahead = StepPlan()
         need = [0] * len(self.cache.groups)
-        for item in plan.items:
-            seq = item.seq
+        tokens = 0
+        for seq in self.running:
+            item = in_plan.get(id(seq))
+            if item is None or not item.samples:
+                return None
             if seq.completion_size + 1 >= seq.sampling.max_tokens:
                 continue                      # the running step's token is its last
+            if len(ahead.items) >= cfg.max_num_seqs or tokens >= budget:
+                return None                   # someone has to wait a turn: the ordinary path rotates them
             # seq.size does not count the running step's token yet: that token goes to position seq.size
             for g, n in enumerate(self.cache.pages_needed(seq.request_id, seq.size + 1)):
                 need[g] += n
             ahead.items.append(PlanItem(seq, seq.size, 1, False))
-        if not ahead.items or len(ahead.items) > self.config.max_num_seqs:
+            tokens += 1
+        visited = 0
+        for seq in self.waiting:
+            if len(ahead.items) >= cfg.max_num_seqs or tokens >= budget:
+                break
+            if not seq.admitted:
+                return None
+            item = in_plan.get(id(seq))
+            first = seq.tokens_in_cache + (item.count if item is not None else 0)
+            count = min(seq.size - first, budget - tokens)
+            if count <= 0:
+                return None
+            for g, n in enumerate(self.cache.pages_needed(seq.request_id, first + count)):
+                need[g] += n
+            ahead.items.append(PlanItem(seq, first, count, True))
+            tokens += count
+            visited += 1
+        if not ahead.items:
             return None
-        # the requests compete for the same pools: the whole step's pages must be free, or
-        # nothing is taken and the ordinary path decides whom to preempt
         if any(n > g.pool.free_count for n, g in zip(need, self.cache.groups)):
             return None
         for item in ahead.items:
-            self.cache.reserve(item.seq.request_id, item.first + 1)
-        ahead.num_tokens = len(ahead.items)
+            self.cache.reserve(item.seq.request_id, item.first + item.count)
+        # the queues move as ``schedule`` moves them: each request that got a portion goes to the
+        # back of the waiting ones, or to the running ones when the portion reaches its last token
+        for item in ahead.items[len(ahead.items) - visited:]:
+            seq = self.waiting.popleft()
+            assert seq is item.seq
+            if item.first + item.count == seq.size:
+                seq.status = Status.RUNNING
+                self.running.append(seq)
+            else:
+                self.waiting.append(seq)
+        ahead.num_tokens = tokens
         return ahead
 
     # ---- pages ------------------------------------------------------------
