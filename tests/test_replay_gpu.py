@@ -83,6 +83,52 @@ def test_cuts_match_plain(model_folders, oracle, name, dtype, cut):
         assert runner.cache.pages_taken_total > runner.cache.num_pages
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random_match_plain(tmp_path, seed):
+    """Sizes beyond the four tiny configurations: a configuration drawn from the seed (head sizes from 16
+    to 256 in steps of 16, one to four kv heads with groups of one to eight, a width that is a multiple
+    of 8, a vocabulary of any size, one to four layers, windows on some of them) with random weights,
+    replayed whole, in portions and mixed on few pages, in float32 and bfloat16, against the plain
+    implementation; the float32 cuts agree bit for bit."""
+    import random
+    from helpers import ARCH
+    from tiny_llm_infer_amd.config import Qwen3Config
+    from tiny_llm_infer_amd.engine.loading import load_model, write_random_model
+    from tiny_llm_infer_amd.engine.runner import ModelRunner
+    rng = random.Random(4000 + seed)
+    kv, group, layers = rng.randrange(1, 5), rng.choice([1, 2, 3, 4, 5, 7, 8]), rng.randrange(1, 5)
+    cfg = dict(hidden_size=8 * rng.randrange(4, 40), intermediate_size=16 * rng.randrange(2, 30),
+               num_hidden_layers=layers, num_attention_heads=kv * group, num_key_value_heads=kv,
+               head_dim=16 * rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16]), vocab_size=rng.randrange(40, 3000),
+               max_position_embeddings=512, rope_theta=rng.choice([1e4, 5e4, 1e6]),
+               rms_norm_eps=rng.choice([1e-6, 1e-5, 3e-6]), tie_word_embeddings=rng.random() < 0.5,
+               use_sliding_window=rng.random() < 0.4, architectures=[ARCH], model_type="qwen3")
+    if cfg["use_sliding_window"]:
+        cfg["sliding_window"] = rng.randrange(5, 70)
+        cfg["layer_types"] = [rng.choice(["sliding_attention", "full_attention"]) for _ in range(layers)]
+    folder = write_random_model(str(tmp_path / "m"), ARCH, Qwen3Config.from_dict(cfg), 100 + seed)
+    lengths = [rng.randrange(2, 150) for _ in range(rng.randrange(2, 6))]
+    reqs = {f"r{i}": random_prompt(cfg["vocab_size"], n, rng.randrange(10 ** 6)) for i, n in enumerate(lengths)}
+    want = plain_logits(folder, reqs)
+    page = rng.choice([8, 16, 32, 64])
+    max_tokens = 64 * ((max(lengths) + 63) // 64) * rng.choice([1, 2, 3])
+    cuts = {"mixed": trace_mixed(reqs, max_tokens=max(max_tokens, 192), seed=seed, max_live=rng.randrange(1, 5)),
+            "whole": trace_whole(reqs), "portions": trace_portions(reqs, seed=seed)}
+    for dtype in ("float32", "bfloat16"):
+        model, _ = load_model(folder, dtype, "cuda:0")
+        first = None
+        for cut, steps in cuts.items():
+            runner = ModelRunner(model, model.env, page_size=page, num_pages=max(max_tokens, 192) // page + (0 if cut == "mixed" else 8),
+                                 max_requests=4, max_batch_tokens=1024)
+            got = collect(steps, _replay(runner, steps))
+            _check(got, want, dtype, f"{cfg}/{dtype}/{cut}", TOL_TINY)
+            if dtype == "float32":
+                first = first or got
+                assert all(np.array_equal(first[rid], got[rid]) for rid in reqs), cut
+            runner.cache.check()
+            assert runner.cache.free_pages() == runner.cache.pages_per_group()
+
+
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_float32_cuts_agree_bit_for_bit(model_folders, oracle, name):
     """In float32 every kernel adds in an order that depends on the row alone,
