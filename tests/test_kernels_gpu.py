@@ -269,10 +269,12 @@ def test_product_of_many_rows_from_the_decode_layout(ops, mnk, cfg):
         ops.rows_cfg = ops.rows_splits = 0
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3])
-@pytest.mark.parametrize("mki", [(130, 264, 1008), (2048, 512, 1536), (300, 4096, 96)])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("mki", [(130, 264, 1008), (2048, 512, 1536), (300, 4096, 96), (260, 256, 400)])
 def test_gated_product_of_many_rows(ops, mki, cfg):
-    """gemm_rows over the interleaved gate/up layout writes silu(x gate^T) * (x up^T)."""
+    """gemm_rows over the interleaved gate/up layout writes silu(x gate^T) * (x up^T), with every launch
+    shape: with three column tiles a wave, a gate tile and its up tile lie in two waves, which exchange
+    their sums; every shape but the last adds a row's products in the same order and gives the same bits."""
     from tiny_llm_infer_amd.parts.base import BuildEnv
     from tiny_llm_infer_amd.parts.linear import GatedMatrix
     M, K, inter = mki
@@ -285,7 +287,11 @@ def test_gated_product_of_many_rows(ops, mki, cfg):
         for splits in (1, 0, 4):
             ops.rows_splits = splits
             close(ops.linear_swiglu(x, m), g / (1 + torch.exp(-g)) * u, torch.bfloat16, f"gated product, {splits} ranges of k")
+        ops.rows_splits = 1
         y = ops.linear_swiglu(x, m)
+        ops.rows_cfg = 2
+        if cfg != 6:                          # (two sets of waves that take the slices of k in turn add in another order)
+            assert torch.equal(y, ops.linear_swiglu(x, m))
     finally:
         ops.many_rows, ops.rows_cfg, ops.rows_splits = "own", 0, 0
     g, u = x.double().cpu() @ gate.double().cpu().t(), x.double().cpu() @ up.double().cpu().t()

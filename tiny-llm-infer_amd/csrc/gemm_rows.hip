@@ -4,7 +4,7 @@
 // library's product, whichever it measured faster for the shape: at the layer sizes of
 // Qwen3-8B to 32B and 512 to 4,096 rows either is ahead by up to 15% somewhere.
 //
-// A workgroup owns ROWS rows and 192, 256 or 512 columns and walks all of k in slices of 128:
+// A workgroup owns ROWS rows and 192, 256, 384 or 512 columns and walks all of k in slices of 128:
 //   x   each slice [ROWS][128] is copied from memory straight into one of two LDS slots
 //       (global_load_lds_dwordx4: lane l of a wave writes the 16 bytes it asked for at LDS
 //       base + 16 l), rows swizzled as in gemm_mid.hip (chunk q of row r at q ^ (r & 15));
@@ -298,9 +298,11 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
     }
     // lane holds y[m*16 + r][tile*16 + 4c + i]
     if (GATED) {
-#pragma unroll
-        for (int t = 0; t + 1 < RT; t += 2) {
-            const int n0 = ((tile0 + t) / 2) * 16 + 4 * c;
+        // one output tile from a gate tile's sums and its up tile's: silu(g) * u with the hardware's exp2 and
+        // reciprocal (1 ulp each; the result is rounded to bfloat16): the library routines would cost more
+        // vector instructions here than the workgroup's MFMAs
+        auto store_pair = [&](const f32x4 (&gate)[MT], const f32x4 (&up)[MT], int gate_tile) {
+            const int n0 = (gate_tile / 2) * 16 + 4 * c;
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 const int row = m * 16 + r;
@@ -308,10 +310,7 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
                 float o[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    // silu(g) * u with the hardware's exp2 and reciprocal (1 ulp each; the result is rounded to
-                    // bfloat16): the library routines would cost more vector instructions here than the
-                    // workgroup's MFMAs
-                    const float g = acc[t][m][i], u = acc[t + 1][m][i];
+                    const float g = gate[m][i], u = up[m][i];
                     o[i] = g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g)) * u;
                 }
                 bf16_t* dst = y + (size_t)row * n_out + n0;
@@ -322,6 +321,33 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, bf1
                     for (int i = 0; i < 4; ++i)
                         if (n0 + i < n_out) dst[i] = f32_to_bf16(o[i]);
                 }
+            }
+        };
+        if constexpr (RT % 2 == 0) {
+#pragma unroll
+            for (int t = 0; t + 1 < RT; t += 2) store_pair(acc[t], acc[t + 1], tile0 + t);
+        } else {
+            // Three tiles a wave: a workgroup's tiles start at an even one (gate), so an even wave holds
+            // gate, up, gate and the odd wave after it up, gate, up.  The odd wave hands the sums of its
+            // first tile over through LDS, [pair of waves][row tile][lane] of 16 bytes, to the even wave,
+            // which holds their gate tile.
+            static_assert(RT == 3 && WAVES % 2 == 0 && KG == 1, "pairs of waves share a gate and an up tile");
+            static_assert((WAVES / 2) * MT * 64 * 16 <= 2 * SLICE * 2, "the sums fit the slots of x");
+            __syncthreads();                   // nobody reads x any more
+            f32x4* sums = reinterpret_cast<f32x4*>(xs_raw) + (size_t)(wave / 2) * MT * 64 + lane;
+            if (wave % 2 == 1) {
+#pragma unroll
+                for (int m = 0; m < MT; ++m) sums[m * 64] = acc[0][m];
+            }
+            __syncthreads();
+            if (wave % 2 == 0) {
+                f32x4 up[MT];
+#pragma unroll
+                for (int m = 0; m < MT; ++m) up[m] = sums[m * 64];
+                store_pair(acc[0], acc[1], tile0);
+                store_pair(acc[2], up, tile0 + 2);
+            } else {
+                store_pair(acc[1], acc[2], tile0 + 1);
             }
         }
         return;
@@ -423,17 +449,18 @@ static int rows_pick(int M, int N, int K, int splits, int gated) {
     const long k_steps = (K + 127) / 128, per = (k_steps + splits - 1) / splits;
     const double cost2 = shared(a_die(16)) * 256.0, cost4 = shared(a_die(12)) * 192.0 * 1.06;
     const double cost3 = alone(a_die(32)) * 512.0 * 0.84, cost6 = alone(a_die(16)) * 256.0 * 0.88;
-    // 128 x 384 outputs in eight waves of three column tiles (one workgroup a compute unit, not for gated
-    // products): 0.82 a column; 5,120 columns are 14 such groups, 6,144 are 16
+    // 128 x 384 outputs in eight waves of three column tiles (one workgroup a compute unit): 0.82 a
+    // column; 5,120 columns are 14 such groups, 6,144 are 16, the 24,576 of a gate/up pair of 12,288 are 64
     const double cost5 = alone(a_die(24)) * 384.0 * 0.82;
     // (from three rounds of the 512-column shape on, it was the fastest at every layer size measured:
-    // the costs above are those of the first rounds)
-    if (alone(a_die(32)) >= 3.0) return 3;
+    // the costs above are those of the first rounds.  A gated product counts whole rounds only: with
+    // two and a bit, the shapes that divide its many columns evenly were 12 to 14% faster)
+    if (gated ? a_die(32) >= 3 * units : alone(a_die(32)) >= 3.0) return 3;
     int best = 2;
     double cost = cost2;
     if (cost3 < cost) { best = 3; cost = cost3; }
-    if (!gated && cost4 < cost) { best = 4; cost = cost4; }
-    if (!gated && cost5 < cost) { best = 5; cost = cost5; }
+    if (cost4 < cost) { best = 4; cost = cost4; }
+    if (cost5 < cost) { best = 5; cost = cost5; }
     if (!gated && per % 2 == 0 && k_steps % per == 0 && cost6 < cost) best = 6;
     return best;
 }
@@ -445,7 +472,8 @@ static int rows_pick(int M, int N, int K, int splits, int gated) {
 // (tli_gemm_mid_reduce, or tli_add_rmsnorm).
 // cfg 0 picks the launch shape; 1: 256 x 256 outputs a workgroup of eight waves, 2: 128 x 256
 // and four waves, two workgroups a compute unit, 3: 128 x 512 and eight waves, 4: 128 x 192 and
-// four waves (not for a gated product), 5: 128 x 384 and eight waves (not for a gated product), 6: 128 x 256
+// four waves, 5: 128 x 384 and eight waves (in a gated product the waves of 4 and 5, which hold three
+// column tiles each, exchange the sums of one tile in pairs), 6: 128 x 256
 // by two sets of four waves that take the slices of k in turn; cfg >= 10: the tens for a gated product, the
 // ones for the others (measurements).
 extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, float* part, int M, int N, int K,
@@ -473,11 +501,9 @@ extern "C" int tli_gemm_rows_bf16(const void* x, const void* w, void* y, float* 
     }
     if (cfg == 2) return launch_rows<4, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     if (cfg == 4) {
-        if (gated) return tli_fail("gemm_rows: three column tiles a wave do not pair up for a gated product");
         return launch_rows<3, 4, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     }
     if (cfg == 5) {
-        if (gated) return tli_fail("gemm_rows: three column tiles a wave do not pair up for a gated product");
         return launch_rows<3, 8, 8, 1>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, part, M, N, K, gated, splits, s);
     }
     return tli_fail("gemm_rows: unknown configuration %d", cfg);
