@@ -497,8 +497,7 @@ __device__ __forceinline__ void head_from_raw(Frag (&out)[NJ], const bf16_t* src
             for (int e = 0; e < 8; ++e) {
                 const float partner = __shfl_xor(x[j][e], 32, 64);
                 const float cs = cos_row[i0 + j * 8 + e], sn = sin_row[i0 + j * 8 + e];
-                // first half: x cos - partner sin; second half: partner sin + x cos
-                x[j][e] = c < 2 ? x[j][e] * cs - partner * sn : partner * sn + x[j][e] * cs;
+                x[j][e] = c < 2 ? rotate_first_half(x[j][e], partner, cs, sn) : rotate_second_half(x[j][e], partner, cs, sn);
             }
     }
 #pragma unroll
@@ -572,8 +571,7 @@ __device__ __forceinline__ uint4 slice_finish(float (&x)[8], bool normed, const 
         for (int e = 0; e < 8; ++e) {
             const float partner = __shfl_xor(x[e], 32, 64);
             const float cs = cos8[e], sn = sin8[e];
-            // first half: x cos - partner sin; second half: partner sin + x cos
-            x[e] = c < 2 ? x[e] * cs - partner * sn : partner * sn + x[e] * cs;
+            x[e] = c < 2 ? rotate_first_half(x[e], partner, cs, sn) : rotate_second_half(x[e], partner, cs, sn);
         }
     }
     return make_uint4(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]), pack_bf16x2(x[4], x[5]), pack_bf16x2(x[6], x[7]));

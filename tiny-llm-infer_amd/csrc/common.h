@@ -106,6 +106,17 @@ __device__ __forceinline__ float quad_rows_sum(float x) {
     return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
+// One element of a rotated pair.  The roundings are written out (a product rounded, then one fused
+// multiply-add) so that every kernel that rotates gives the same bits: left to the compiler, which of the
+// two products of `a b + c d` is fused depends on the code around it.
+// first half of a head: x cos - partner sin;  second half: partner sin + x cos
+__device__ __forceinline__ float rotate_first_half(float x, float partner, float cs, float sn) {
+    return fmaf(x, cs, -(partner * sn));
+}
+__device__ __forceinline__ float rotate_second_half(float x, float partner, float cs, float sn) {
+    return fmaf(partner, sn, x * cs);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = TLI_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, TLI_WAVE);

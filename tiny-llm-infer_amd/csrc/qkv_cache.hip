@@ -92,8 +92,8 @@ __global__ void qkv_to_cache_kernel(
         for (int i = lane; i < head_dim; i += TLI_WAVE) {
             float v = x[i];
             if (cos_row && i < rotary_dim) {
-                if (i < half) v = x[i] * cos_row[i] - x[i + half] * sin_row[i];
-                else v = x[i - half] * sin_row[i - half] + x[i] * cos_row[i - half];
+                if (i < half) v = rotate_first_half(x[i], x[i + half], cos_row[i], sin_row[i]);
+                else v = rotate_second_half(x[i], x[i - half], cos_row[i - half], sin_row[i - half]);
             }
             from_f32(dst + i, v);
         }
@@ -170,8 +170,7 @@ qkv_to_cache_wide_kernel(
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
             const float partner = __shfl_xor(x[e], 32, TLI_WAVE);
-            // first half: x cos - partner sin; second half: partner sin + x cos
-            x[e] = lane < 32 ? x[e] * cr[e] - partner * sr[e] : partner * sr[e] + x[e] * cr[e];
+            x[e] = lane < 32 ? rotate_first_half(x[e], partner, cr[e], sr[e]) : rotate_second_half(x[e], partner, cr[e], sr[e]);
         }
     }
     bf16_t* dst = is_q ? q_out + (size_t)row * q_dim + (size_t)h * HD
@@ -318,25 +317,53 @@ keys_values_to_cache_kernel(
     const size_t stride = (size_t)(heads + 2 * kv_heads) * HD;
     const bf16_t* rows = qkv + (size_t)(first_row + p_lo - start) * stride;
 
-    // keys: position p_lo + j by wave j % 4
+    // keys: position p_lo + j by wave j % 4.  Everything a wave reads for its positions (their key rows, their
+    // rows of the rotation tables) and for its share of the values is asked for before anything is
+    // computed: the kernel is a chain of round trips to memory, and this makes one of what a loop over the
+    // positions made two of for every position.
+    constexpr int TURNS = G / QKV_WAVES;
+    static_assert(G % QKV_WAVES == 0, "every wave takes the same number of positions");
     const bf16_t* ksrc = rows + (size_t)(heads + kvh) * HD + lane * EPL;
     bf16_t* kdst = k_cache + (((size_t)page * kv_heads + kvh) * page_size + slot0) * HD + lane * EPL;
-    for (int j = wave; j < n; j += QKV_WAVES) {
-        const int pos = p_lo + j;
+    const bool rotate = cos_table != nullptr;
+    uint2 kraw[TURNS];
+    float cr[TURNS][EPL], sr[TURNS][EPL];
+#pragma unroll
+    for (int i = 0; i < TURNS; ++i) {
+        const int j = min(wave + i * QKV_WAVES, n - 1);          // (a turn past the last position reads it again, and stores nothing)
         const bf16_t* src = ksrc + (size_t)j * stride;
+        if (EPL == 1) kraw[i] = make_uint2((uint32_t)src[0], 0u);
+        else if (EPL == 2) kraw[i] = make_uint2(*reinterpret_cast<const uint32_t*>(src), 0u);
+        else kraw[i] = *reinterpret_cast<const uint2*>(src);
+        const int pos = p_lo + j;
+        const bool in_table = rotate && pos >= 0 && pos < table_positions;
+        const size_t at = (size_t)(in_table ? pos : 0) * (HD / 2) + (lane % 32) * EPL;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            cr[i][e] = rotate ? cos_table[at + e] : 1.f;
+            sr[i][e] = rotate ? sin_table[at + e] : 0.f;
+        }
+    }
+    float knw[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) knw[e] = k_norm_w ? k_norm_w[lane * EPL + e] : 1.f;
+    // values: one dim a thread, the positions as one run of slots
+    const bf16_t* vsrc = rows + (size_t)(heads + kv_heads + kvh) * HD;
+    const bool has_dim = (int)threadIdx.x < HD;                  // (HD <= 256 = the workgroup: a thread has one dim or none)
+    bf16_t vals[G];
+#pragma unroll
+    for (int j = 0; j < G; ++j) vals[j] = has_dim && j < n ? cache_value(vsrc[(size_t)j * stride + threadIdx.x]) : (bf16_t)0;
+
+#pragma unroll
+    for (int i = 0; i < TURNS; ++i) {
+        const int j = wave + i * QKV_WAVES;
+        const int pos = p_lo + j;
         float x[EPL];
-        if (EPL == 1) {
-            x[0] = bf16_to_f32(src[0]);
-        } else if (EPL == 2) {
-            const uint32_t u = *reinterpret_cast<const uint32_t*>(src);
-            x[0] = bf16_to_f32((bf16_t)(u & 0xffffu));
-            x[1 % EPL] = bf16_to_f32((bf16_t)(u >> 16));
-        } else {
-            const uint2 u = *reinterpret_cast<const uint2*>(src);
-            x[0] = bf16_to_f32((bf16_t)(u.x & 0xffffu));
-            x[1 % EPL] = bf16_to_f32((bf16_t)(u.x >> 16));
-            x[2 % EPL] = bf16_to_f32((bf16_t)(u.y & 0xffffu));
-            x[3 % EPL] = bf16_to_f32((bf16_t)(u.y >> 16));
+        x[0] = bf16_to_f32((bf16_t)(kraw[i].x & 0xffffu));
+        if (EPL >= 2) x[1 % EPL] = bf16_to_f32((bf16_t)(kraw[i].x >> 16));
+        if (EPL == 4) {
+            x[2 % EPL] = bf16_to_f32((bf16_t)(kraw[i].y & 0xffffu));
+            x[3 % EPL] = bf16_to_f32((bf16_t)(kraw[i].y >> 16));
         }
         if (k_norm_w) {
             float ss = 0.f;
@@ -345,17 +372,16 @@ keys_values_to_cache_kernel(
             ss = wave_sum(ss);
             const float scale = 1.0f / sqrtf(ss / (float)HD + k_eps);
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) x[e] = k_norm_w[lane * EPL + e] * x[e] * scale;
+            for (int e = 0; e < EPL; ++e) x[e] = knw[e] * x[e] * scale;
         }
-        if (cos_table && pos >= 0 && pos < table_positions) {
-            const float* cr = cos_table + (size_t)pos * (HD / 2) + (lane % 32) * EPL;
-            const float* sr = sin_table + (size_t)pos * (HD / 2) + (lane % 32) * EPL;
+        if (rotate && pos >= 0 && pos < table_positions) {
 #pragma unroll
             for (int e = 0; e < EPL; ++e) {
                 const float partner = __shfl_xor(x[e], 32, TLI_WAVE);
-                x[e] = lane < 32 ? x[e] * cr[e] - partner * sr[e] : partner * sr[e] + x[e] * cr[e];
+                x[e] = lane < 32 ? rotate_first_half(x[e], partner, cr[i][e], sr[i][e]) : rotate_second_half(x[e], partner, cr[i][e], sr[i][e]);
             }
         }
+        if (j >= n) continue;
         bf16_t* dst = kdst + (size_t)j * HD;
         if (EPL == 1) {
             dst[0] = f32_to_bf16(x[0]);
@@ -366,12 +392,8 @@ keys_values_to_cache_kernel(
         }
     }
 
-    // values: one dim a thread, the positions as one run of slots
-    const bf16_t* vsrc = rows + (size_t)(heads + kv_heads + kvh) * HD;
-    for (int d = threadIdx.x; d < HD; d += QKV_WAVES * TLI_WAVE) {
-        bf16_t vals[G];
-#pragma unroll
-        for (int j = 0; j < G; ++j) vals[j] = j < n ? cache_value(vsrc[(size_t)j * stride + d]) : (bf16_t)0;
+    if (has_dim) {
+        const int d = threadIdx.x;
         bf16_t* dst = v_cache + (((size_t)page * kv_heads + kvh) * HD + d) * page_size + slot0;
         if (n == G) {               // a whole group: its slots start at a multiple of G
             uint32_t w[G / 2];
