@@ -258,8 +258,9 @@ def test_random_serving_scenarios_give_plain_greedy_tokens(model_folders, seed):
     1 to 69 prompt tokens and 1 to 13 new ones, a pool between barely enough for the longest request and
     enough for all, a token budget from 2 to 256, a limit of live requests, steps planned ahead or not,
     prefix caching (with a shared prefix) where no layer has a window, requests that arrive while others
-    are served.  Every request gets the tokens of plain greedy generation, whatever was preempted and
-    computed again on the way, and the cache is whole at the end."""
+    are served, an end-of-sequence token that stops some of them early.  Every request gets the tokens of
+    plain greedy generation, whatever was preempted and computed again on the way, and the cache is whole
+    at the end."""
     import random
     rng = random.Random(1000 + seed)
     name = rng.choice(sorted(TINY))
@@ -280,16 +281,24 @@ def test_random_serving_scenarios_give_plain_greedy_tokens(model_folders, seed):
                   enable_prefix_caching=prefix)
     eng.lookahead = rng.random() < 0.6
     arrive = rng.choice([0, 0, 1, 3])
+    want = [list(plain_qwen3.greedy(cfg, w, prompts[i], outs[i])) for i in range(nreq)]
+    # in half of the scenarios a token that some request meets in the middle of its run ends a request:
+    # requests then stop at times that no plan made ahead can know
+    stops = rng.random() < 0.5 and max(outs) >= 3
+    if stops:
+        eos = rng.choice([run for run in want if len(run) >= 3])[rng.randrange(1, 3)]
+        eng.eos_token_ids = {eos}
+        want = [run[:run.index(eos) + 1] if eos in run else run for run in want]
     results, index_of, admitted, steps = {}, {}, 0, 0
     while admitted < nreq or not eng.is_finished():
         while admitted < nreq and (steps >= arrive * admitted or eng.is_finished()):
-            index_of[eng.add_request(prompts[admitted], SamplingParams(max_tokens=outs[admitted], ignore_eos=True))] = admitted
+            index_of[eng.add_request(prompts[admitted], SamplingParams(max_tokens=outs[admitted], ignore_eos=not stops))] = admitted
             admitted += 1
         for r in eng.step():
             results[index_of[r.request_id]] = list(r.token_ids)
         steps += 1
         assert steps < 5000, "no progress"
     for i in range(nreq):
-        assert results[i] == list(plain_qwen3.greedy(cfg, w, prompts[i], outs[i])), (name, i)
+        assert results[i] == want[i], (name, i)
     eng.runner.cache.check()
     assert eng.runner.cache.free_pages() == eng.runner.cache.pages_per_group()
